@@ -1,0 +1,265 @@
+#!/usr/bin/env python3
+"""Benchmark of the HDLA rank-2 DPLR delta-rule hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload train|fwd|varlen|decode] [--no-cpu-baseline]
+
+Default workload ("train") is the headline configuration: chunked forward + backward at B=4, T=2048, H=16,
+K=V=64, bf16 inputs, fp32 state, random fp32 initial state, upstream gradients do and dht (configuration 2).
+One step = one forward + one backward through the public operator (autograd Function -> C ABI -> HIP kernels)
+with all inputs already resident in HBM.  The script prints ONE JSON line: whole-step throughput, a roofline
+object for the kernel that takes the largest share of the step (every kernel is listed under "kernels"), and the
+CPU oracle timed on this box's host cores on a bounded sample.
+
+Per-kernel durations are measured live with events on the stream the kernels run on, in a second loop of the
+same number of steps that launches the same kernels one at a time through hdla_chunk_stages.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "hdla-impl_amd"))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+METRIC = "chunked fwd+bwd tokens/s (B4,T2048,H16,K=V=64 bf16) + % of MFMA/HBM roofline"
+
+
+def _args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="train", choices=["train", "fwd", "varlen", "decode"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    return ap.parse_args()
+
+
+def interface_bytes(kernel, pass_, K, V, es, gs):
+    """Algorithmic HBM bytes of one kernel per (16-token chunk, head): every distinct input read once, every
+    output written once (es = bytes per element of the inputs, gs = bytes per element of gk)."""
+    W, UT, KGT, BGT, VTT, EGL = 32 * K * es, 32 * V * es, 16 * K * es, 32 * K * es, 16 * V * es, 4 * K
+    QG, AQK, AQB = 16 * K * es, 256 * es, 512 * es
+    AQBT, BG, WT, QGT, TM = 512 * es, 32 * K * es, 32 * K * es, 16 * K * es, 4096
+    HC = DHC = K * V * es
+    VN = DVN = 32 * V * es
+    inputs = 2 * 16 * K * es + 16 * K * gs + 2 * 32 * K * es + 16 * V * es          # q,k,gk,a,b,v
+    if kernel == "prep":
+        out = W + UT + KGT + BGT + VTT + EGL + ((QG + AQK + AQB) if pass_ == 0 else (AQBT + BG + WT + QGT + TM))
+        return inputs + out
+    if kernel == "scan_fwd":
+        rd = W + UT + KGT + BGT + VTT + EGL
+        return rd + (QG + AQK + AQB + 16 * V * es if pass_ == 0 else HC + VN)
+    if kernel == "scan_bwd":
+        return AQBT + BG + WT + QGT + EGL + 16 * V * es + DHC + DVN
+    if kernel == "chunk_grad":
+        outs = 2 * 16 * K * es + 16 * K * gs + 2 * 32 * K * es + 16 * V * es
+        return inputs + 16 * V * es + TM + W + UT + HC + DHC + VN + DVN + outs
+    raise ValueError(kernel)
+
+
+def time_steps(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def stage_times(inp_dev, dims_kw, pass_, steps, outputs):
+    """Average duration (ms) of each kernel of one pass, events on the current stream around single-stage launches."""
+    from hdla_hip import _lib
+    lib = _lib.load()
+    q, k, v, a, b, gk, h0, do, dht = inp_dev
+    dims = _lib.make_dims(**dims_kw)
+    ws = _lib.workspace(dims, pass_, q.device)
+    P = _lib.ptr
+    names = {1: "prep", 2: "scan_fwd", 4: "scan_bwd", 8: "chunk_grad"}
+    masks = [1, 2] if pass_ == 0 else [1, 2, 4, 8]
+    o, ht, dq, dk, dv, da, db, dgk, dh0 = outputs
+    stream = _lib.current_stream(q.device)
+    acc = {m: 0.0 for m in masks}
+
+    def run(mask):
+        rc = lib.hdla_chunk_stages(ctypes.byref(dims), pass_, mask, P(q), P(k), P(v), P(a), P(b), P(gk), P(h0), P(o),
+                                   P(ht), P(do), P(dht), P(dq), P(dk), P(dv), P(da), P(db), P(dgk), P(dh0), P(ws),
+                                   ws.numel(), stream)
+        _lib.check(rc, "hdla_chunk_stages")
+
+    for m in masks:                      # warm
+        run(m)
+    torch.cuda.synchronize()
+    for _ in range(steps):
+        evs = []
+        for m in masks:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            run(m)
+            e1.record()
+            evs.append((m, e0, e1))
+        torch.cuda.synchronize()
+        for m, e0, e1 in evs:
+            acc[m] += e0.elapsed_time(e1)
+    return {names[m]: acc[m] / steps for m in masks}
+
+
+def cpu_baseline_train():
+    """The CPU oracle (chunk form of the reference's naive.py, fp32, chunk 16, torch on all host cores) on one
+    batch row of configuration 2: forward + autograd backward."""
+    from hdla_hip.synthetic import make_config
+    from oracle import hrdplr_oracle as O
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    inp = make_config(2)
+    B_s = 1
+    t = [x[:B_s].bfloat16().float().requires_grad_() for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    h0 = inp.h0[:B_s].clone().requires_grad_()
+    t0 = time.perf_counter()
+    o, ht = O.chunk_naive(*t, 1.0, h0, chunk_size=16)
+    torch.autograd.grad([o, ht], t + [h0], [inp.do[:B_s], inp.dht[:B_s]])
+    dt = time.perf_counter() - t0
+    T = inp.q.shape[1]
+    return {"value": B_s * T / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"one run of batch row 0 of 4 (T=2048, H=16, K=V=64), fp32 chunk-form oracle fwd + autograd bwd, {dt:.1f} s"}
+
+
+def cpu_baseline_decode():
+    from hdla_hip.synthetic import make_config
+    from oracle import hrdplr_oracle as O
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    steps, B_s = 4, 32
+    inp = make_config(4, shape=(B_s, steps, 32, 128, 128))
+    t = [x.bfloat16().float() for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    t0 = time.perf_counter()
+    with torch.no_grad():
+        O.recurrence(*t, 1.0, inp.h0, dtype=torch.float32)
+    dt = time.perf_counter() - t0
+    return {"value": B_s * steps / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"{steps} decode steps of {B_s} of the 256 sequences (H=32, K=V=128), fp32 token recurrence, {dt:.1f} s"}
+
+
+def main():
+    args = _args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU only: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    from hdla_hip import chunk_hrdplr_delta_rule, fused_recurrent_dplr_delta_rule
+    from hdla_hip.synthetic import CONFIG_SHAPES, make_config
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    wl = args.workload
+    cfg = {"train": 2, "fwd": 1, "varlen": 3, "decode": 4}[wl]
+    B, T, H, K, V = CONFIG_SHAPES[cfg]
+    inp = make_config(cfg)
+    dt = torch.bfloat16
+    res = {"metric": METRIC if wl == "train" else f"{wl} tokens/s", "unit": "tokens/s", "n_gpus": 1,
+           "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": "bf16", "data": "synthetic"}
+
+    if wl == "decode":
+        from hdla_hip.recurrent import fused_recurrent_dplr_delta_rule_fwd
+        from hdla_hip.synthetic import make_inputs
+        ncycle = 8                                             # distinct per-step inputs, cycled
+        gen = [inp] + [make_inputs(2000 + i, B, 1, H, K, V, h0_std=0.1) for i in range(1, ncycle)]
+        steps_in = [[x.to(dt).to(dev) for x in (g.q, g.k, g.v, g.a, g.b, g.gk)] for g in gen]
+        state = {"S": inp.h0.to(dev), "i": 0}
+
+        def step():
+            t = steps_in[state["i"] % ncycle]
+            state["i"] += 1
+            _, state["S"] = fused_recurrent_dplr_delta_rule(*t, 2, scale=1.0, initial_state=state["S"],
+                                                            output_final_state=True)
+        sec = time_steps(step, args.steps, args.warmup)
+        # kernel-only duration with events on the launch stream
+        evs = []
+        for _ in range(args.steps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t = steps_in[state["i"] % ncycle]
+            state["i"] += 1
+            q, k, v, a, b, gk = t
+            e0.record()
+            _, state["S"] = fused_recurrent_dplr_delta_rule_fwd(q, k, v, a, b, gk, 2, 1.0, state["S"], True)
+            e1.record()
+            evs.append((e0, e1))
+        torch.cuda.synchronize()
+        kms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+        nbytes = 2 * B * H * K * V * 4 + B * H * (4 * K + 4 * K + V + V) * 2
+        res.update(value=B / sec, ms_per_step=sec * 1e3,
+                   config={"workload": "config 4: fused recurrent decode, B=256 H=32 K=V=128, one token per call, "
+                                       "persistent fp32 state", "batch": B, "heads": H, "K": K, "V": V},
+                   roofline={"bound": "hbm", "kernel": "recurrent_kernel", "achieved": nbytes / (kms * 1e-3) / 1e9,
+                             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                             "traffic": None, "bytes_per_launch": nbytes, "ms_per_launch": kms})
+        if not args.no_cpu_baseline:
+            res["cpu_baseline"] = cpu_baseline_decode()
+        print(json.dumps(res))
+        return
+
+    cu = None if inp.cu_seqlens is None else inp.cu_seqlens.to(dev)
+    N = B if cu is None else cu.numel() - 1
+    leaves = [x.to(dt).to(dev).requires_grad_(wl != "fwd") for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    use_h0 = wl != "fwd"
+    h0 = inp.h0.to(dev).requires_grad_(True) if use_h0 else None
+    do, dht = inp.do.to(dt).to(dev), inp.dht.to(dev)
+
+    def step():
+        o, ht = chunk_hrdplr_delta_rule(*leaves, 2, scale=1.0, initial_state=h0, output_final_state=True,
+                                        chunk_size=16, cu_seqlens=cu)
+        if wl != "fwd":
+            torch.autograd.grad([o, ht], leaves + [h0], [do, dht])
+
+    sec = time_steps(step, args.steps, args.warmup)
+    tokens = B * T
+    # per-kernel durations
+    raw = [x.detach() for x in leaves] + [None if h0 is None else h0.detach(), do, dht]
+    dims_kw = dict(B=B, T=T, H=H, K=K, V=V, R=2, N=N, in_dtype=dt, gk_dtype=dt, scale=1.0, cu_seqlens=cu)
+    q = raw[0]
+    o = torch.empty_like(raw[2])
+    ht = torch.empty(N, H, K, V, dtype=torch.float32, device=dev)
+    grads = [torch.empty_like(x) for x in (raw[0], raw[1], raw[2], raw[3], raw[4], raw[5])]
+    dh0 = torch.empty_like(ht)
+    outs = (o, ht, *grads, dh0)
+    kern = {}
+    for pass_ in ([0] if wl == "fwd" else [0, 1]):
+        for name, ms in stage_times(raw, dims_kw, pass_, args.steps, outs).items():
+            kern[f"{'fwd' if pass_ == 0 else 'bwd'}.{name}"] = ms
+    nchunk_heads = H * sum(-(-int(l) // 16) for l in ([T] * B if cu is None else (cu[1:] - cu[:-1]).tolist()))
+    klist = []
+    for name, ms in kern.items():
+        p_, kn = name.split(".")
+        by = interface_bytes(kn, 0 if p_ == "fwd" else 1, K, V, 2, 2) * nchunk_heads
+        klist.append({"kernel": name, "ms": ms, "bytes": by, "GB/s": by / (ms * 1e-3) / 1e9,
+                      "frac_hbm": by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
+    dom = max(klist, key=lambda x: x["ms"])
+    per_tok_head = (9 * K * 2) if wl == "fwd" else (26 * K * 2)            # compulsory bytes per (token, head), K = V
+    whole = per_tok_head * H * tokens
+    res.update(value=tokens / sec, ms_per_step=sec * 1e3,
+               config={"workload": {"train": "config 2: chunked fwd+bwd, B=4 T=2048 H=16 K=V=64, bf16 in, fp32 state, h0/do/dht",
+                                    "fwd": "config 1: chunked fwd, B=4 T=2048 H=16 K=V=64, bf16 in, fp32 state",
+                                    "varlen": "config 3: chunked fwd+bwd, packed 2048/4096/4096/6144, H=16 K=V=128"}[wl],
+                       "global_batch": B, "seq_len": T, "heads": H, "K": K, "V": V, "chunk": 16},
+               roofline={"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS,
+                         "unit": "GB/s", "frac": dom["frac_hbm"], "traffic": None,
+                         "bytes_per_launch": dom["bytes"], "ms_per_launch": dom["ms"]},
+               kernels=klist,
+               whole_step={"compulsory_bytes": whole, "GB/s": whole / sec / 1e9, "frac_hbm": whole / sec / 1e9 / HBM_PEAK_GBS,
+                           "sum_kernel_ms": sum(x["ms"] for x in klist)})
+    if not args.no_cpu_baseline and wl == "train":
+        res["cpu_baseline"] = cpu_baseline_train()
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,267 @@
+// C ABI of libhdla_hip.so: argument checks, workspace layout and the launch sequences of the three entry points.
+#include "../../include/hdla_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include "hdla_launch.h"
+#include "hdla_ws.h"
+
+using namespace hdla;
+
+namespace {
+
+constexpr int CHUNK = 16;
+
+inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int check_dims(const hdla_dims* d) {
+    if (!d) return HDLA_ERR_NULL;
+    if (d->R != 2) return HDLA_ERR_RANK;
+    if (d->B < 1 || d->T < 0 || d->H < 1 || d->N < 1) return HDLA_ERR_SHAPE;
+    if (!((d->K == 64 || d->K == 128) && (d->V == 64 || d->V == 128))) return HDLA_ERR_SHAPE;
+    if (d->H > 65535) return HDLA_ERR_SHAPE;
+    if (d->in_dtype != HDLA_BF16 && d->in_dtype != HDLA_FP32) return HDLA_ERR_DTYPE;
+    if (d->gk_dtype != HDLA_BF16 && d->gk_dtype != HDLA_FP32) return HDLA_ERR_DTYPE;
+    if (d->in_dtype == HDLA_FP32 && d->gk_dtype != HDLA_FP32) return HDLA_ERR_DTYPE;
+    if (d->cu_seqlens) { if (d->B != 1) return HDLA_ERR_SEQ; }
+    else if (d->N != d->B) return HDLA_ERR_SEQ;
+    return HDLA_OK;
+}
+
+// pass 0 = forward, 1 = backward
+int make_layout(const hdla_dims* d, int pass, WsLayout& L, int& nch) {
+    const int rc = check_dims(d);
+    if (rc) return rc;
+    if (d->N > 65535) return HDLA_ERR_SHAPE;
+    const int NT = (d->T + CHUNK - 1) / CHUNK;
+    nch = d->cu_seqlens ? NT + d->N : d->B * NT;
+    const size_t es = d->in_dtype == HDLA_BF16 ? 2 : 4;
+    const size_t chw = (size_t)d->H * (size_t)nch;
+    const size_t K = d->K, V = d->V;
+    size_t off = 0;
+    auto take = [&](size_t bytes) { const size_t o = off; off += up256(bytes); return o; };
+    L = WsLayout{};
+    L.W = take(chw * 2 * K * 16 * es);
+    L.UT = take(chw * 2 * V * 16 * es);
+    L.KGT = take(chw * K * 16 * es);
+    L.BGT = take(chw * 2 * K * 16 * es);
+    L.VTT = take(chw * V * 16 * es);
+    L.EGL = take(chw * K * 4);
+    if (pass == 0) {
+        L.QG = take(chw * K * 16 * es);
+        L.AQK = take(chw * 256 * es);
+        L.AQB = take(chw * 2 * 256 * es);
+    } else {
+        L.AQBT = take(chw * 2 * 256 * es);
+        L.BG = take(chw * 2 * K * 16 * es);
+        L.WT = take(chw * 2 * K * 16 * es);
+        L.QGT = take(chw * K * 16 * es);
+        L.TM = take(chw * 1024 * 4);
+        L.HC = take(chw * K * V * es);
+        L.DHC = take(chw * K * V * es);
+        L.VN = take(chw * 2 * 16 * V * es);
+        L.DVN = take(chw * 2 * 16 * V * es);
+    }
+    if (d->cu_seqlens) {
+        L.CHUNK_OFF = take((size_t)(d->N + 1) * 4);
+        L.CHUNK_SEQ = take((size_t)(nch > 0 ? nch : 1) * 4);
+    }
+    L.total = off > 0 ? off : 256;
+    return HDLA_OK;
+}
+
+template <typename T>
+void bind_ws(ChunkArgs<T>& a, const hdla_dims* d, const WsLayout& L, int nch, void* workspace) {
+    char* base = static_cast<char*>(workspace);
+    auto at = [&](size_t o) { return reinterpret_cast<T*>(base + o); };
+    a.ws.W = at(L.W); a.ws.UT = at(L.UT); a.ws.KGT = at(L.KGT); a.ws.BGT = at(L.BGT); a.ws.VTT = at(L.VTT);
+    a.ws.QG = at(L.QG); a.ws.AQK = at(L.AQK); a.ws.AQB = at(L.AQB);
+    a.ws.AQBT = at(L.AQBT); a.ws.BG = at(L.BG); a.ws.WT = at(L.WT); a.ws.QGT = at(L.QGT);
+    a.ws.HC = at(L.HC); a.ws.DHC = at(L.DHC); a.ws.VN = at(L.VN); a.ws.DVN = at(L.DVN);
+    a.ws.EGL = reinterpret_cast<float*>(base + L.EGL);
+    a.ws.TM = reinterpret_cast<float*>(base + L.TM);
+    a.st.cu = d->cu_seqlens;
+    a.st.chunk_off = d->cu_seqlens ? reinterpret_cast<const int32_t*>(base + L.CHUNK_OFF) : nullptr;
+    a.st.chunk_seq = d->cu_seqlens ? reinterpret_cast<const int32_t*>(base + L.CHUNK_SEQ) : nullptr;
+    a.st.T = d->T;
+    a.st.NT = (d->T + CHUNK - 1) / CHUNK;
+    a.st.N = d->N;
+    a.st.nch = nch;
+}
+
+template <typename T>
+int run_chunk(const hdla_dims* d, int pass, const void* q, const void* k, const void* v, const void* a_,
+              const void* b, const void* gk, const float* h0, void* o, float* ht, const void* d_o,
+              const float* dht, void* dq, void* dk, void* dv, void* da, void* db, void* dgk, float* dh0,
+              void* workspace, size_t workspace_bytes, hipStream_t stream, int stages = HDLA_STAGE_ALL) {
+    WsLayout L;
+    int nch = 0;
+    int rc = make_layout(d, pass, L, nch);
+    if (rc) return rc;
+    if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255) || workspace_bytes < L.total) return HDLA_ERR_WORKSPACE;
+    ChunkArgs<T> a{};
+    a.q = static_cast<const T*>(q); a.k = static_cast<const T*>(k); a.v = static_cast<const T*>(v);
+    a.a = static_cast<const T*>(a_); a.b = static_cast<const T*>(b);
+    a.gk = gk; a.gk_f32 = d->gk_dtype == HDLA_FP32;
+    a.H = d->H; a.scale = d->scale;
+    a.h0 = h0; a.ht = pass == 0 ? ht : nullptr; a.o = static_cast<T*>(o);
+    a.dout = static_cast<const T*>(d_o); a.dht = dht; a.dh0 = dh0;
+    a.dq = static_cast<T*>(dq); a.dk = static_cast<T*>(dk); a.dv = static_cast<T*>(dv);
+    a.da = static_cast<T*>(da); a.db = static_cast<T*>(db); a.dgk = dgk;
+    bind_ws(a, d, L, nch, workspace);
+    hipError_t e;
+    if (d->cu_seqlens && (stages & HDLA_STAGE_PREP)) {
+        char* base = static_cast<char*>(workspace);
+        e = launch_chunk_table(d->cu_seqlens, d->N, nch, reinterpret_cast<int32_t*>(base + L.CHUNK_OFF),
+                               reinterpret_cast<int32_t*>(base + L.CHUNK_SEQ), stream);
+        if (e != hipSuccess) return (int)e;
+    }
+    if (nch > 0 && (stages & HDLA_STAGE_PREP)) {
+        e = launch_prep<T>(a, d->K, d->V, pass == 1, stream);
+        if (e != hipSuccess) return (int)e;
+    }
+    if (stages & HDLA_STAGE_SCAN_FWD) {
+        e = launch_scan_fwd<T>(a, d->K, d->V, pass == 0, stream);
+        if (e != hipSuccess) return (int)e;
+    }
+    if (pass == 1) {
+        if (stages & HDLA_STAGE_SCAN_BWD) {
+            e = launch_scan_bwd<T>(a, d->K, d->V, stream);
+            if (e != hipSuccess) return (int)e;
+        }
+        if (nch > 0 && (stages & HDLA_STAGE_CHUNK_GRAD)) {
+            e = launch_chunk_grad<T>(a, d->K, d->V, stream);
+            if (e != hipSuccess) return (int)e;
+        }
+    }
+    return HDLA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int hdla_version(void) { return HDLA_VERSION; }
+
+const char* hdla_strerror(int code) {
+    switch (code) {
+        case HDLA_OK: return "success";
+        case HDLA_ERR_NULL: return "a required pointer is NULL";
+        case HDLA_ERR_SHAPE: return "unsupported shape (need K,V in {64,128}, B,H,N >= 1, T >= 0, H,N <= 65535)";
+        case HDLA_ERR_RANK: return "only rank R = 2 is supported";
+        case HDLA_ERR_DTYPE: return "unsupported dtype (in_dtype bf16|fp32; gk fp32, or bf16 with bf16 inputs)";
+        case HDLA_ERR_WORKSPACE: return "workspace is NULL, not 256-byte aligned, or smaller than hdla_workspace_bytes()";
+        case HDLA_ERR_ALIGN: return "tensor pointers must be 16-byte aligned";
+        case HDLA_ERR_SEQ: return "cu_seqlens needs B == 1; without it N must equal B";
+        default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error code";
+    }
+}
+
+size_t hdla_workspace_bytes(const hdla_dims* dims, int pass) {
+    WsLayout L;
+    int nch;
+    if (pass != 0 && pass != 1) return 0;
+    if (make_layout(dims, pass, L, nch)) return 0;
+    return L.total;
+}
+
+int hdla_workspace_layout(const hdla_dims* dims, int pass, hdla_ws_layout* out) {
+    if (!out) return HDLA_ERR_NULL;
+    if (pass != 0 && pass != 1) return HDLA_ERR_SHAPE;
+    WsLayout L;
+    int nch;
+    const int rc = make_layout(dims, pass, L, nch);
+    if (rc) return rc;
+    out->nch = nch;
+    out->W = L.W; out->UT = L.UT; out->KGT = L.KGT; out->BGT = L.BGT; out->VTT = L.VTT; out->EGL = L.EGL;
+    out->QG = L.QG; out->AQK = L.AQK; out->AQB = L.AQB;
+    out->AQBT = L.AQBT; out->BG = L.BG; out->WT = L.WT; out->QGT = L.QGT; out->TM = L.TM;
+    out->HC = L.HC; out->DHC = L.DHC; out->VN = L.VN; out->DVN = L.DVN;
+    out->CHUNK_OFF = L.CHUNK_OFF; out->CHUNK_SEQ = L.CHUNK_SEQ;
+    out->total = L.total;
+    return HDLA_OK;
+}
+
+int hdla_chunk_fwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
+                   const void* b, const void* gk, const float* h0, void* o, float* ht,
+                   void* workspace, size_t workspace_bytes, void* stream) {
+    const int rc = check_dims(dims);
+    if (rc) return rc;
+    if (dims->T > 0 && (!q || !k || !v || !a || !b || !gk || !o)) return HDLA_ERR_NULL;
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(a) || !aligned16(b) || !aligned16(gk) ||
+        !aligned16(o) || !aligned16(h0) || !aligned16(ht)) return HDLA_ERR_ALIGN;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dims->in_dtype == HDLA_BF16)
+        return run_chunk<bf16>(dims, 0, q, k, v, a, b, gk, h0, o, ht, nullptr, nullptr, nullptr, nullptr, nullptr,
+                               nullptr, nullptr, nullptr, nullptr, workspace, workspace_bytes, s);
+    return run_chunk<float>(dims, 0, q, k, v, a, b, gk, h0, o, ht, nullptr, nullptr, nullptr, nullptr, nullptr,
+                            nullptr, nullptr, nullptr, nullptr, workspace, workspace_bytes, s);
+}
+
+int hdla_chunk_bwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
+                   const void* b, const void* gk, const float* h0, const void* d_o, const float* dht,
+                   void* dq, void* dk, void* dv, void* da, void* db, void* dgk, float* dh0,
+                   void* workspace, size_t workspace_bytes, void* stream) {
+    const int rc = check_dims(dims);
+    if (rc) return rc;
+    if (dims->T > 0 && (!q || !k || !v || !a || !b || !gk || !d_o || !dq || !dk || !dv || !da || !db || !dgk))
+        return HDLA_ERR_NULL;
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(a) || !aligned16(b) || !aligned16(gk) ||
+        !aligned16(d_o) || !aligned16(dq) || !aligned16(dk) || !aligned16(dv) || !aligned16(da) || !aligned16(db) ||
+        !aligned16(dgk) || !aligned16(h0) || !aligned16(dht) || !aligned16(dh0)) return HDLA_ERR_ALIGN;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dims->in_dtype == HDLA_BF16)
+        return run_chunk<bf16>(dims, 1, q, k, v, a, b, gk, h0, nullptr, nullptr, d_o, dht, dq, dk, dv, da, db, dgk,
+                               dh0, workspace, workspace_bytes, s);
+    return run_chunk<float>(dims, 1, q, k, v, a, b, gk, h0, nullptr, nullptr, d_o, dht, dq, dk, dv, da, db, dgk,
+                            dh0, workspace, workspace_bytes, s);
+}
+
+int hdla_chunk_stages(const hdla_dims* dims, int pass, int stages, const void* q, const void* k, const void* v,
+                      const void* a, const void* b, const void* gk, const float* h0, void* o, float* ht,
+                      const void* d_o, const float* dht, void* dq, void* dk, void* dv, void* da, void* db, void* dgk,
+                      float* dh0, void* workspace, size_t workspace_bytes, void* stream) {
+    const int rc = check_dims(dims);
+    if (rc) return rc;
+    if (pass != 0 && pass != 1) return HDLA_ERR_SHAPE;
+    if (!q || !k || !v || !a || !b || !gk) return HDLA_ERR_NULL;
+    if (pass == 0 ? !o : (!d_o || !dq || !dk || !dv || !da || !db || !dgk)) return HDLA_ERR_NULL;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dims->in_dtype == HDLA_BF16)
+        return run_chunk<bf16>(dims, pass, q, k, v, a, b, gk, h0, o, ht, d_o, dht, dq, dk, dv, da, db, dgk, dh0,
+                               workspace, workspace_bytes, s, stages);
+    return run_chunk<float>(dims, pass, q, k, v, a, b, gk, h0, o, ht, d_o, dht, dq, dk, dv, da, db, dgk, dh0,
+                            workspace, workspace_bytes, s, stages);
+}
+
+int hdla_recurrent_fwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
+                       const void* b, const void* gk, int reverse, const float* h0, void* o, float* ht,
+                       void* stream) {
+    const int rc = check_dims(dims);
+    if (rc) return rc;
+    if (dims->T > 0 && (!q || !k || !v || !a || !b || !gk || !o)) return HDLA_ERR_NULL;
+    if (!aligned16(h0) || !aligned16(ht)) return HDLA_ERR_ALIGN;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e;
+    if (dims->in_dtype == HDLA_BF16) {
+        RecurrentArgs<bf16> r{};
+        r.q = static_cast<const bf16*>(q); r.k = static_cast<const bf16*>(k); r.v = static_cast<const bf16*>(v);
+        r.a = static_cast<const bf16*>(a); r.b = static_cast<const bf16*>(b);
+        r.gk = gk; r.gk_f32 = dims->gk_dtype == HDLA_FP32;
+        r.H = dims->H; r.T_ = dims->T; r.N = dims->N; r.scale = dims->scale; r.reverse = reverse;
+        r.cu = dims->cu_seqlens; r.h0 = h0; r.ht = ht; r.o = static_cast<bf16*>(o);
+        e = launch_recurrent<bf16>(r, dims->K, dims->V, s);
+    } else {
+        RecurrentArgs<float> r{};
+        r.q = static_cast<const float*>(q); r.k = static_cast<const float*>(k); r.v = static_cast<const float*>(v);
+        r.a = static_cast<const float*>(a); r.b = static_cast<const float*>(b);
+        r.gk = gk; r.gk_f32 = 1;
+        r.H = dims->H; r.T_ = dims->T; r.N = dims->N; r.scale = dims->scale; r.reverse = reverse;
+        r.cu = dims->cu_seqlens; r.h0 = h0; r.ht = ht; r.o = static_cast<float*>(o);
+        e = launch_recurrent<float>(r, dims->K, dims->V, s);
+    }
+    return e == hipSuccess ? HDLA_OK : (int)e;
+}
+
+}  // extern "C"

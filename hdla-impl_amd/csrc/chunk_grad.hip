@@ -1,0 +1,272 @@
+// chunk_grad kernel: everything of the backward pass that is local to one 16-token chunk.
+//
+// One wavefront per (chunk, head) fuses what the reference runs as five launches: the dA part of
+// HRDPLR/bwd_triton.py:30-105, the dv kernel :239-290, the dqg/dkg/dbg/dw/dgk_last kernel :309-487, the WY
+// backward :503-612, the score backward :627-883 and the log-decay gradient :899-948.  Its inputs are the
+// original tensors, do, and per chunk the state entering it (h), the gradient of the state leaving it (dh),
+// v_new and its gradient, all left in the workspace by the two scans.  Nothing but the seven gradients is
+// written back.
+//
+// Two differences from the reference's algebra, both exact:
+//  * the WY backward never forms d(Tm): with X = [w | u] = Tm R, R = [ag | A_ak v] one has dR = Tm^T dX and
+//    dA_ab = mask(dR X^T), which replaces the Tm^T dTm Tm^T chain of bwd_triton.py:577-612;
+//  * the score backward covers the whole 16 x 16 (x2 ranks) tile with MFMA products against the same
+//    factorised operands as the forward pass instead of a serial per-column loop.
+#include "hdla_common.cuh"
+#include "hdla_launch.h"
+
+namespace hdla {
+
+constexpr int LDG = 36;
+
+template <typename T, int K, int V>
+__global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
+    constexpr int KT = K / 16, VT = V / 16;
+    __shared__ __attribute__((aligned(16))) float sT[32 * LDG];   // (I - A_ab)^-1, rank-major
+
+    const int cid = blockIdx.x, h = blockIdx.y;
+    ChunkPos cp;
+    if (!locate_chunk(p.st, cid, cp)) return;
+    const int l = lane_id(), g = l >> 4, c = l & 15;
+    const int H = p.H;
+    const bool rowok = c < cp.len;
+    const int64_t tok = cp.tok0 + c;
+    const int64_t qoff = (tok * H + h) * K + 4 * g;
+    const int64_t aoff0 = ((tok * RANK + 0) * H + h) * K + 4 * g;
+    const int64_t aoff1 = ((tok * RANK + 1) * H + h) * K + 4 * g;
+    const int64_t voff = (tok * H + h) * V + 4 * g;
+    const int64_t chw = (int64_t)h * p.st.nch + cid;
+    const float scale = p.scale;
+    const T* HC = p.ws.HC + chw * (K * V);
+    const T* DHC = p.ws.DHC + chw * (K * V);
+    const T* VN = p.ws.VN + chw * (2 * CH * V);
+    const T* DVN = p.ws.DVN + chw * (2 * CH * V);
+
+    {
+        const float* tmw = p.ws.TM + chw * 1024;
+        const int row = l >> 1, c0 = (l & 1) * 16;
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+            *reinterpret_cast<f32x4*>(&sT[row * LDG + c0 + 4 * x]) = *reinterpret_cast<const f32x4*>(tmw + row * 32 + c0 + 4 * x);
+    }
+    __syncthreads();
+    // tmT[s][r] = F((Tm^{s r})^T): lane (g,c) reg i = Tm^{s r}[4g+i][c]
+    Frag<T> tmT[2][2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            f32x4 t;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) t[i] = sT[(16 * s + 4 * g + i) * LDG + 16 * r + c];
+            tmT[s][r] = to_frag<T>(t);
+        }
+    const Frag<T> ident = ident_frag<T>();
+
+    // ---- cumulative decays; A_qk^T and A_ak^T (rows j, inner i) -----------------------------------------------
+    f32x4 gi[KT], ge[KT];
+    f32x4 aqkT = zero4(), aakT[2] = {zero4(), zero4()};
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+        const f32x4 g4 = ld_gk4(p.gk, qoff + 16 * kt, p.gk_f32, rowok);
+        gi[kt] = scan16_incl(g4);
+        ge[kt] = gi[kt] - g4;
+        const f32x4 m = bcast16(gi[kt], MID);
+        const f32x4 eq = exp4<T>(gi[kt] - m), ek = exp4<T>(m - gi[kt]), ea = exp4<T>(ge[kt] - m);
+        const f32x4 q4 = to_f32(ld_frag_if(p.q + qoff + 16 * kt, rowok));
+        const f32x4 k4 = to_f32(ld_frag_if(p.k + qoff + 16 * kt, rowok));
+        const f32x4 a0 = to_f32(ld_frag_if(p.a + aoff0 + 16 * kt, rowok));
+        const f32x4 a1 = to_f32(ld_frag_if(p.a + aoff1 + 16 * kt, rowok));
+        const Frag<T> qh = to_frag<T>(q4 * eq * scale), kh = to_frag<T>(k4 * ek);
+        aqkT = mm(kh, qh, aqkT);
+        aakT[0] = mm(kh, to_frag<T>(a0 * ea), aakT[0]);
+        aakT[1] = mm(kh, to_frag<T>(a1 * ea), aakT[1]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {          // row j = c, inner i = 4g+i
+        const int ii = 4 * g + i;
+        if (!(c <= ii)) aqkT[i] = 0.f;
+        if (!(c < ii)) { aakT[0][i] = 0.f; aakT[1][i] = 0.f; }
+    }
+    const Frag<T> aqkTf = to_frag<T>(aqkT);
+    const Frag<T> aakTf[2] = {to_frag<T>(aakT[0]), to_frag<T>(aakT[1])};
+
+    // ---- products over the value dimension -------------------------------------------------------------------
+    f32x4 dAqk = zero4(), dAqb[2] = {zero4(), zero4()}, dAak[2] = {zero4(), zero4()};
+    f32x4 dAab[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
+    f32x4 dv[VT];
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt) {
+        const Frag<T> doN = ld_frag_if(p.dout + voff + 16 * vt, rowok);
+        const Frag<T> vN = ld_frag_if(p.v + voff + 16 * vt, rowok);
+        const Frag<T> vnN[2] = {ld_frag(VN + (0 * CH + c) * V + 16 * vt + 4 * g), ld_frag(VN + (1 * CH + c) * V + 16 * vt + 4 * g)};
+        const Frag<T> dvnN[2] = {ld_frag(DVN + (0 * CH + c) * V + 16 * vt + 4 * g), ld_frag(DVN + (1 * CH + c) * V + 16 * vt + 4 * g)};
+        dAqk = mm(doN, vN, dAqk);
+        dAqb[0] = mm(doN, vnN[0], dAqb[0]);
+        dAqb[1] = mm(doN, vnN[1], dAqb[1]);
+        const Frag<T> doT = transpose(doN, ident);
+        const Frag<T> dvnT[2] = {transpose(dvnN[0], ident), transpose(dvnN[1], ident)};
+        Frag<T> dMf[2], dMTf[2];
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            f32x4 x = mm(tmT[0][r], dvnT[0], zero4());
+            x = mm(tmT[1][r], dvnT[1], x);
+            dMf[r] = to_frag<T>(x);                       // dM_r   rows i, inner value
+            f32x4 y = mm(dvnT[0], tmT[0][r], zero4());
+            y = mm(dvnT[1], tmT[1][r], y);
+            dMTf[r] = to_frag<T>(y);                      // dM_r^T rows value, inner i
+        }
+        const Frag<T> uN[2] = {transpose(ld_tile(p.ws.UT + ((chw * 2 + 0) * VT + vt) * TILE), ident),
+                               transpose(ld_tile(p.ws.UT + ((chw * 2 + 1) * VT + vt) * TILE), ident)};
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            dAak[r] = mm(dMf[r], vN, dAak[r]);
+            dAab[r][0] = mm(dMf[r], uN[0], dAab[r][0]);
+            dAab[r][1] = mm(dMf[r], uN[1], dAab[r][1]);
+        }
+        f32x4 x = mm(aqkTf, doT, zero4());
+        x = mm(aakTf[0], dMTf[0], x);
+        x = mm(aakTf[1], dMTf[1], x);
+        dv[vt] = x;                                       // rows token, inner value; kg dS is added below
+    }
+
+    // ---- first pass over channel tiles: dw -> dag, and the w part of dA_ab ------------------------------------
+    f32x4 dag[2][KT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+        f32x4 dwT[2] = {zero4(), zero4()};                // rows channel, inner token
+#pragma unroll
+        for (int vt = 0; vt < VT; ++vt) {
+            const Frag<T> Sf = ld_frag(HC + (16 * kt + c) * V + 16 * vt + 4 * g);
+            dwT[0] = mm(Sf, ld_frag(DVN + (0 * CH + c) * V + 16 * vt + 4 * g), dwT[0]);
+            dwT[1] = mm(Sf, ld_frag(DVN + (1 * CH + c) * V + 16 * vt + 4 * g), dwT[1]);
+        }
+        const Frag<T> dwTf[2] = {to_frag<T>(dwT[0]), to_frag<T>(dwT[1])};
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            f32x4 x = mm(tmT[0][r], dwTf[0], zero4());
+            x = mm(tmT[1][r], dwTf[1], x);
+            dag[r][kt] = x;                               // rows token, inner channel
+            const Frag<T> dagf = to_frag<T>(x);
+            dAab[r][0] = mm(dagf, ld_tile(p.ws.W + ((chw * 2 + 0) * KT + kt) * TILE), dAab[r][0]);
+            dAab[r][1] = mm(dagf, ld_tile(p.ws.W + ((chw * 2 + 1) * KT + kt) * TILE), dAab[r][1]);
+        }
+    }
+
+    // ---- masks; both orientations of the nine score-gradient tiles --------------------------------------------
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {          // row i = c, inner j = 4g+i
+        const int j = 4 * g + i;
+        if (!(j <= c)) { dAqk[i] = 0.f; dAqb[0][i] = 0.f; dAqb[1][i] = 0.f; }
+        if (!(j < c)) { dAak[0][i] = 0.f; dAak[1][i] = 0.f; dAab[0][0][i] = 0.f; dAab[0][1][i] = 0.f; dAab[1][0][i] = 0.f; dAab[1][1][i] = 0.f; }
+    }
+    const Frag<T> fAqk = to_frag<T>(dAqk), fAqkT = transpose(fAqk, ident);
+    Frag<T> fAqb[2], fAqbT[2], fAak[2], fAakT[2], fAab[2][2], fAabT[2][2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+        fAqb[s] = to_frag<T>(dAqb[s]); fAqbT[s] = transpose(fAqb[s], ident);
+        fAak[s] = to_frag<T>(dAak[s]); fAakT[s] = transpose(fAak[s], ident);
+#pragma unroll
+        for (int r = 0; r < 2; ++r) { fAab[r][s] = to_frag<T>(dAab[r][s]); fAabT[r][s] = transpose(fAab[r][s], ident); }
+    }
+
+    // ---- second pass over channel tiles: state products, score backward, final gradients ----------------------
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+        const f32x4 m = bcast16(gi[kt], MID), gl = bcast16(gi[kt], CH - 1);
+        const f32x4 eq = exp4<T>(gi[kt] - m), ek = exp4<T>(m - gi[kt]), ea = exp4<T>(ge[kt] - m);
+        const f32x4 egi = exp4<T>(gi[kt]), ege = exp4<T>(ge[kt]), edn = exp4<T>(gl - gi[kt]);
+        const f32x4 q4 = to_f32(ld_frag_if(p.q + qoff + 16 * kt, rowok));
+        const f32x4 k4 = to_f32(ld_frag_if(p.k + qoff + 16 * kt, rowok));
+        const f32x4 a4[2] = {to_f32(ld_frag_if(p.a + aoff0 + 16 * kt, rowok)), to_f32(ld_frag_if(p.a + aoff1 + 16 * kt, rowok))};
+        const f32x4 b4[2] = {to_f32(ld_frag_if(p.b + aoff0 + 16 * kt, rowok)), to_f32(ld_frag_if(p.b + aoff1 + 16 * kt, rowok))};
+        const Frag<T> qhT = transpose(to_frag<T>(q4 * eq * scale), ident), khT = transpose(to_frag<T>(k4 * ek), ident);
+        const Frag<T> ahT[2] = {transpose(to_frag<T>(a4[0] * ea), ident), transpose(to_frag<T>(a4[1] * ea), ident)};
+        const Frag<T> bhT[2] = {transpose(to_frag<T>(b4[0] * ek), ident), transpose(to_frag<T>(b4[1] * ek), ident)};
+        const f32x4 kg4 = k4 * edn;
+        const f32x4 bg4[2] = {b4[0] * edn, b4[1] * edn};
+        const Frag<T> kgf = to_frag<T>(kg4);
+
+        f32x4 dqg = zero4(), dkg = zero4(), dbg[2] = {zero4(), zero4()};
+        float hh = 0.f;                                    // partial of sum_v S * dS for channel 16kt + c
+#pragma unroll
+        for (int vt = 0; vt < VT; ++vt) {
+            const Frag<T> Sf = ld_frag(HC + (16 * kt + c) * V + 16 * vt + 4 * g);
+            const Frag<T> dSf = ld_frag(DHC + (16 * kt + c) * V + 16 * vt + 4 * g);
+            const Frag<T> doN = ld_frag_if(p.dout + voff + 16 * vt, rowok);
+            const Frag<T> vN = ld_frag_if(p.v + voff + 16 * vt, rowok);
+            dqg = mm(doN, Sf, dqg);
+            dkg = mm(vN, dSf, dkg);
+            dbg[0] = mm(ld_frag(VN + (0 * CH + c) * V + 16 * vt + 4 * g), dSf, dbg[0]);
+            dbg[1] = mm(ld_frag(VN + (1 * CH + c) * V + 16 * vt + 4 * g), dSf, dbg[1]);
+            const f32x4 s4 = to_f32(Sf), d4 = to_f32(dSf);
+            hh += s4[0] * d4[0] + s4[1] * d4[1] + s4[2] * d4[2] + s4[3] * d4[3];
+            dv[vt] = mm(kgf, transpose(dSf, ident), dv[vt]);
+        }
+        hh += __shfl_xor(hh, 16);
+        hh += __shfl_xor(hh, 32);
+        f32x4 hh4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) hh4[i] = __shfl(hh, 4 * g + i);
+
+        f32x4 dqh = mm(fAqk, khT, zero4());
+        dqh = mm(fAqb[0], bhT[0], dqh);
+        dqh = mm(fAqb[1], bhT[1], dqh);
+        f32x4 dkh = mm(fAqkT, qhT, zero4());
+        dkh = mm(fAakT[0], ahT[0], dkh);
+        dkh = mm(fAakT[1], ahT[1], dkh);
+        f32x4 dah[2], dbh[2];
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            f32x4 x = mm(fAak[r], khT, zero4());
+            x = mm(fAab[r][0], bhT[0], x);
+            x = mm(fAab[r][1], bhT[1], x);
+            dah[r] = x;
+            f32x4 y = mm(fAqbT[r], qhT, zero4());          // here r plays the role of the b rank s
+            y = mm(fAabT[0][r], ahT[0], y);
+            y = mm(fAabT[1][r], ahT[1], y);
+            dbh[r] = y;
+        }
+        const f32x4 dq = (dqh * eq + dqg * egi) * scale;
+        const f32x4 dk = dkh * ek + dkg * edn;
+        const f32x4 da[2] = {dah[0] * ea + dag[0][kt] * ege, dah[1] * ea + dag[1][kt] * ege};
+        const f32x4 db[2] = {dbh[0] * ek + dbg[0] * edn, dbh[1] * ek + dbg[1] * edn};
+        const f32x4 Dge = da[0] * a4[0] + da[1] * a4[1];
+        const f32x4 Dgi = dq * q4 - dk * k4 - db[0] * b4[0] - db[1] * b4[1];
+        const f32x4 dgl = exp4<T>(gl) * hh4 + sum16(dkg * kg4 + dbg[0] * bg4[0] + dbg[1] * bg4[1]);
+        const f32x4 dg = rscan16_incl(Dgi + Dge) - Dge + dgl;
+        if (rowok) {
+            st_frag(p.dq + qoff + 16 * kt, to_frag<T>(dq));
+            st_frag(p.dk + qoff + 16 * kt, to_frag<T>(dk));
+            st_frag(p.da + aoff0 + 16 * kt, to_frag<T>(da[0]));
+            st_frag(p.da + aoff1 + 16 * kt, to_frag<T>(da[1]));
+            st_frag(p.db + aoff0 + 16 * kt, to_frag<T>(db[0]));
+            st_frag(p.db + aoff1 + 16 * kt, to_frag<T>(db[1]));
+            st_gk4(p.dgk, qoff + 16 * kt, p.gk_f32, dg);
+        }
+    }
+    if (rowok) {
+#pragma unroll
+        for (int vt = 0; vt < VT; ++vt) st_frag(p.dv + voff + 16 * vt, to_frag<T>(dv[vt]));
+    }
+}
+
+template <typename T, int K, int V>
+static hipError_t launch_chunk_grad_kv(const ChunkArgs<T>& a, hipStream_t stream) {
+    dim3 grid(a.st.nch, a.H), block(64);
+    hipLaunchKernelGGL((chunk_grad_kernel<T, K, V>), grid, block, 0, stream, a);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_chunk_grad(const ChunkArgs<T>& a, int K, int V, hipStream_t stream) {
+    if (K == 64 && V == 64) return launch_chunk_grad_kv<T, 64, 64>(a, stream);
+    if (K == 128 && V == 128) return launch_chunk_grad_kv<T, 128, 128>(a, stream);
+    if (K == 64 && V == 128) return launch_chunk_grad_kv<T, 64, 128>(a, stream);
+    if (K == 128 && V == 64) return launch_chunk_grad_kv<T, 128, 64>(a, stream);
+    return hipErrorInvalidValue;
+}
+template hipError_t launch_chunk_grad<bf16>(const ChunkArgs<bf16>&, int, int, hipStream_t);
+template hipError_t launch_chunk_grad<float>(const ChunkArgs<float>&, int, int, hipStream_t);
+
+}  // namespace hdla

@@ -1,0 +1,199 @@
+// Shared device-side building blocks of the HDLA rank-2 DPLR delta-rule kernels for gfx950 (CDNA4, wave64).
+//
+// Everything in the chunked path is phrased as products of 16x16 tiles held in MFMA register fragments.
+// A "row fragment" F(X) of a 16 x 16 tile X is 4 values per lane: lane (g, c) = (lane / 16, lane % 16)
+// holds X[c][4g .. 4g+3], i.e. row c, four consecutive entries of the inner (contracted) dimension.
+//
+//     mm(F(P), F(Q), acc)   accumulates   Z = P * Q^T   as a row fragment:  lane (g,c) reg i  +=  Z[c][4g+i]
+//
+// so the rows of the first argument become the rows of the result and the rows of the second argument become
+// the inner index of the result.  The result of one product is therefore directly the operand of the next one
+// (after conversion to the operand type), which is what lets the inter-chunk state scan run entirely in
+// registers.  The two instantiations are bf16 operands (v_mfma_f32_16x16x16_bf16) and fp32 operands
+// (four v_mfma_f32_16x16x4_f32 steps with the inner index permuted to match); both accumulate in fp32.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "hdla_ws.h"
+
+namespace hdla {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+
+constexpr int CH = 16;       // tokens per chunk
+constexpr int MID = 7;       // token whose cumulative log-decay centres the factorised scores
+constexpr int RANK = 2;      // rank of the a/b update
+constexpr int TILE = 256;    // elements of one 16x16 tile (64 lanes x 4)
+
+template <typename T> struct Frag;
+template <> struct Frag<bf16> { s16x4 v; };
+template <> struct Frag<float> { f32x4 v; };
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+
+// ---- conversions -------------------------------------------------------------------------------------------
+__device__ __forceinline__ float bf2f(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+__device__ __forceinline__ uint16_t f2bf(float f) {
+    // round to nearest even; inputs here are finite by construction
+    __bf16 h = (__bf16)f;
+    return __builtin_bit_cast(uint16_t, h);
+}
+
+template <typename T> __device__ __forceinline__ Frag<T> to_frag(f32x4 a);
+template <> __device__ __forceinline__ Frag<bf16> to_frag<bf16>(f32x4 a) {
+    Frag<bf16> r;
+    r.v[0] = (short)f2bf(a[0]); r.v[1] = (short)f2bf(a[1]); r.v[2] = (short)f2bf(a[2]); r.v[3] = (short)f2bf(a[3]);
+    return r;
+}
+template <> __device__ __forceinline__ Frag<float> to_frag<float>(f32x4 a) { Frag<float> r; r.v = a; return r; }
+
+__device__ __forceinline__ f32x4 to_f32(Frag<bf16> a) {
+    f32x4 r;
+    r[0] = bf2f((uint16_t)a.v[0]); r[1] = bf2f((uint16_t)a.v[1]); r[2] = bf2f((uint16_t)a.v[2]); r[3] = bf2f((uint16_t)a.v[3]);
+    return r;
+}
+__device__ __forceinline__ f32x4 to_f32(Frag<float> a) { return a.v; }
+
+__device__ __forceinline__ f32x4 zero4() { f32x4 z = {0.f, 0.f, 0.f, 0.f}; return z; }
+
+// ---- the tile product --------------------------------------------------------------------------------------
+// acc[lane(g,c)][i] += sum_k P[c][k] * Q[4g+i][k]     (frows = F(P), finner = F(Q))
+__device__ __forceinline__ f32x4 mm(Frag<bf16> frows, Frag<bf16> finner, f32x4 acc) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(finner.v, frows.v, acc, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mm(Frag<float> frows, Frag<float> finner, f32x4 acc) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(finner.v[s], frows.v[s], acc, 0, 0, 0);
+    return acc;
+}
+
+// F(I16): used to transpose a tile with one product, F(X^T) = mm(F(I), F(X)).
+template <typename T> __device__ __forceinline__ Frag<T> ident_frag() {
+    const int l = lane_id(), g = l >> 4, c = l & 15;
+    f32x4 e;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) e[i] = (c == 4 * g + i) ? 1.f : 0.f;
+    return to_frag<T>(e);
+}
+template <typename T> __device__ __forceinline__ Frag<T> transpose(Frag<T> x, Frag<T> ident) {
+    return to_frag<T>(mm(ident, x, zero4()));
+}
+
+// ---- fragment loads / stores -------------------------------------------------------------------------------
+// four consecutive elements at p (8-byte aligned for bf16, 16-byte aligned for fp32)
+__device__ __forceinline__ Frag<bf16> ld_frag(const bf16* p) { Frag<bf16> r; r.v = *reinterpret_cast<const s16x4*>(p); return r; }
+__device__ __forceinline__ Frag<float> ld_frag(const float* p) { Frag<float> r; r.v = *reinterpret_cast<const f32x4*>(p); return r; }
+__device__ __forceinline__ void st_frag(bf16* p, Frag<bf16> f) { *reinterpret_cast<s16x4*>(p) = f.v; }
+__device__ __forceinline__ void st_frag(float* p, Frag<float> f) { *reinterpret_cast<f32x4*>(p) = f.v; }
+template <typename T> __device__ __forceinline__ Frag<T> zero_frag() { return to_frag<T>(zero4()); }
+
+template <typename T> __device__ __forceinline__ Frag<T> ld_frag_if(const T* p, bool ok) {
+    return ok ? ld_frag(p) : zero_frag<T>();
+}
+
+// one element stores (used for the strided, 4-rows-per-lane writes of row-major checkpoints)
+__device__ __forceinline__ void st_elem(bf16* p, float x) { p->x = f2bf(x); }
+__device__ __forceinline__ void st_elem(float* p, float x) { *p = x; }
+__device__ __forceinline__ float ld_elem(const bf16* p) { return bf2f(p->x); }
+__device__ __forceinline__ float ld_elem(const float* p) { return *p; }
+
+// whole tile in fragment order: lane l owns elements [4l, 4l+4) of a 256-element block
+template <typename T> __device__ __forceinline__ Frag<T> ld_tile(const T* tile) { return ld_frag(tile + 4 * lane_id()); }
+template <typename T> __device__ __forceinline__ void st_tile(T* tile, Frag<T> f) { st_frag(tile + 4 * lane_id(), f); }
+
+// gk may be stored as bf16 or fp32 independently of the other inputs
+__device__ __forceinline__ f32x4 ld_gk4(const void* base, int64_t elem_off, int is_f32, bool ok) {
+    if (!ok) return zero4();
+    if (is_f32) return *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(base) + elem_off);
+    return to_f32(ld_frag(reinterpret_cast<const bf16*>(base) + elem_off));
+}
+__device__ __forceinline__ void st_gk4(void* base, int64_t elem_off, int is_f32, f32x4 x) {
+    if (is_f32) *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(base) + elem_off) = x;
+    else st_frag(reinterpret_cast<bf16*>(base) + elem_off, to_frag<bf16>(x));
+}
+
+// ---- exp: fast hardware exp2 for the bf16 path, full-accuracy expf for the fp32 path -----------------------
+template <typename T> __device__ __forceinline__ float exp_t(float x);
+template <> __device__ __forceinline__ float exp_t<bf16>(float x) { return __expf(x); }
+template <> __device__ __forceinline__ float exp_t<float>(float x) { return expf(x); }
+template <typename T> __device__ __forceinline__ f32x4 exp4(f32x4 x) {
+    f32x4 r; r[0] = exp_t<T>(x[0]); r[1] = exp_t<T>(x[1]); r[2] = exp_t<T>(x[2]); r[3] = exp_t<T>(x[3]); return r;
+}
+
+// ---- sequence / chunk addressing ---------------------------------------------------------------------------
+struct ChunkPos {
+    int64_t tok0;  // first token row of the chunk on the flattened axis
+    int len;       // valid tokens in the chunk (1..16)
+    int n;         // sequence
+};
+
+__device__ __forceinline__ bool locate_chunk(const SeqTab& st, int cid, ChunkPos& cp) {
+    if (st.cu == nullptr) {
+        if (cid >= st.N * st.NT) return false;
+        cp.n = cid / st.NT;
+        const int ic = cid - cp.n * st.NT;
+        cp.tok0 = (int64_t)cp.n * st.T + (int64_t)ic * CH;
+        cp.len = min(CH, st.T - ic * CH);
+        return true;
+    }
+    if (cid >= st.chunk_off[st.N]) return false;
+    cp.n = st.chunk_seq[cid];
+    const int ic = cid - st.chunk_off[cp.n];
+    const int64_t bos = st.cu[cp.n], eos = st.cu[cp.n + 1];
+    cp.tok0 = bos + (int64_t)ic * CH;
+    cp.len = (int)min((int64_t)CH, eos - cp.tok0);
+    return true;
+}
+
+// chunk range [c0, c1) of sequence n
+__device__ __forceinline__ void seq_chunks(const SeqTab& st, int n, int& c0, int& c1) {
+    if (st.cu == nullptr) { c0 = n * st.NT; c1 = c0 + st.NT; }
+    else { c0 = st.chunk_off[n]; c1 = st.chunk_off[n + 1]; }
+}
+
+// ---- per-chunk decay quantities in fragment layout ---------------------------------------------------------
+// lane (g,c) holds token c of the chunk and channels 16*kt + 4g + i.  An inclusive prefix sum over the 16 lanes
+// of a group gives the cumulative log-decay gi; ge = gi - g is the exclusive one.
+__device__ __forceinline__ f32x4 scan16_incl(f32x4 x) {
+    const int c = lane_id() & 15;
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+        f32x4 t;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) t[i] = __shfl_up(x[i], off, 16);
+        if (c >= off) x += t;
+    }
+    return x;
+}
+__device__ __forceinline__ f32x4 rscan16_incl(f32x4 x) {   // suffix sum over the 16 lanes of a group
+    const int c = lane_id() & 15;
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+        f32x4 t;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) t[i] = __shfl_down(x[i], off, 16);
+        if (c + off < 16) x += t;
+    }
+    return x;
+}
+__device__ __forceinline__ f32x4 bcast16(f32x4 x, int src) {  // value of lane `src` of the own 16-lane group
+    f32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = __shfl(x[i], src, 16);
+    return r;
+}
+__device__ __forceinline__ f32x4 sum16(f32x4 x) {             // sum over the 16 lanes of a group, on all of them
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+        f32x4 t;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) t[i] = __shfl_xor(x[i], off, 16);
+        x += t;
+    }
+    return x;
+}
+
+}  // namespace hdla

@@ -1,0 +1,96 @@
+// Workspace layout and kernel argument blocks shared by the kernels and the C-ABI host code.
+//
+// Every per-chunk buffer is laid out [head][chunk slot][per-chunk elements]: the chunks of one (sequence, head)
+// are contiguous, which is the order the two state scans walk them in.  Buffers marked "tiles" hold 16x16 tiles
+// in fragment order (lane-major, 256 elements per tile) so that the consumer reads back exactly the registers
+// the producer held; buffers marked "rows" are plain row-major.
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+
+namespace hdla {
+
+struct bf16 { uint16_t x; };  // storage type tag for bf16 tensors (raw bits)
+
+// Tokens live on one flattened axis of B*T rows.  Without cu_seqlens sequence n covers rows [n*T, (n+1)*T) and
+// has NT = ceil(T/16) chunks; with cu_seqlens (device int64[N+1], batch 1) sequence n covers [cu[n], cu[n+1])
+// and its chunks are numbered from chunk_off[n] (device int32[N+1], built by build_chunk_table_kernel).
+struct SeqTab {
+    const int64_t* cu;        // nullable
+    const int32_t* chunk_off; // valid when cu != nullptr
+    const int32_t* chunk_seq; // valid when cu != nullptr: sequence of each chunk
+    int T, NT, N;
+    int nch;                  // chunk slots the workspace is laid out for (an upper bound with cu_seqlens)
+};
+
+// Byte offsets into the caller's workspace; 0-sized entries are unused in the given pass.
+struct WsLayout {
+    // written by prep, read by the scans
+    size_t W;      // tiles  [2][K/16]   F(w_s)        rows token, inner channel
+    size_t UT;     // tiles  [2][V/16]   F(u_s^T)      rows value, inner token
+    size_t KGT;    // tiles  [K/16]      F(kg^T)       rows channel, inner token
+    size_t BGT;    // tiles  [2][K/16]   F(bg_s^T)     rows channel, inner token
+    size_t VTT;    // tiles  [V/16]      F(v^T)        rows value, inner token
+    size_t EGL;    // fp32   [K]         exp(g_last)
+    // forward pass only
+    size_t QG;     // tiles  [K/16]      F(qg)         rows token, inner channel
+    size_t AQK;    // tiles  [1]         F(A_qk)       rows i, inner j
+    size_t AQB;    // tiles  [2]         F(A_qb^s)     rows i, inner j
+    // backward pass only
+    size_t AQBT;   // tiles  [2]         F(A_qb^s^T)   rows j, inner i
+    size_t BG;     // tiles  [2][K/16]   F(bg_s)       rows token, inner channel
+    size_t WT;     // tiles  [2][K/16]   F(w_s^T)      rows channel, inner token
+    size_t QGT;    // tiles  [K/16]      F(qg^T)       rows channel, inner token
+    size_t TM;     // fp32   [32][32]    (I - A_ab)^-1 in rank-major order (row r*16+i, column s*16+j)
+    size_t HC;     // rows   [K][V]      state entering the chunk
+    size_t DHC;    // rows   [K][V]      gradient of the state leaving the chunk
+    size_t VN;     // rows   [2][16][V]  v_new, rank-major
+    size_t DVN;    // rows   [2][16][V]  gradient of v_new, rank-major
+    // chunk table (only with cu_seqlens)
+    size_t CHUNK_OFF;  // int32 [N+1]
+    size_t CHUNK_SEQ;  // int32 [nch]
+    size_t total;
+};
+
+template <typename T>
+struct Ws {
+    T *W, *UT, *KGT, *BGT, *VTT, *QG, *AQK, *AQB, *AQBT, *BG, *WT, *QGT, *HC, *DHC, *VN, *DVN;
+    float *EGL, *TM;
+};
+
+template <typename T>
+struct ChunkArgs {            // inputs of the chunked operator + workspace
+    const T *q, *k, *v, *a, *b;
+    const void* gk;
+    int gk_f32;
+    int H;
+    float scale;
+    SeqTab st;
+    Ws<T> ws;
+    // forward scan
+    const float* h0;          // nullable [N][H][K][V]
+    float* ht;                // nullable
+    T* o;                     // forward pass output
+    // backward
+    const T* dout;            // do [B,T,H,V]
+    const float* dht;         // nullable
+    float* dh0;               // nullable
+    T *dq, *dk, *dv, *da, *db;
+    void* dgk;
+};
+
+template <typename T>
+struct RecurrentArgs {
+    const T *q, *k, *v, *a, *b;
+    const void* gk;
+    int gk_f32;
+    int H, T_, N;
+    float scale;
+    int reverse;
+    const int64_t* cu;        // nullable, device
+    const float* h0;          // nullable
+    float* ht;                // nullable
+    T* o;
+};
+
+}  // namespace hdla

@@ -1,0 +1,228 @@
+// prep kernel: everything of a 16-token chunk that does not depend on the recurrent state.
+//
+// Replaces, for one (chunk, head) per wavefront, the reference's chunk-local cumsum (fla chunk_rwkv6_fwd_cumsum,
+// called at HRDPLR/hrdplr.py:44), the two score kernels (HRDPLR/fwd_triton.py:22-290 and :305-514), the
+// triangular inverse (HRDPLR/fwd_triton.py:601-667) and the WY kernel (HRDPLR/fwd_triton.py:685-790).
+// The four score matrices never reach HBM: they are MFMA accumulators, (I - A_ab)^-1 is solved in LDS, and
+// w, u and the gated copies are written once, in the fragment order the state scans read them in.
+#include "hdla_common.cuh"
+#include "hdla_launch.h"
+
+namespace hdla {
+
+constexpr int LDP = 36;   // padded row length of the 32x32 LDS matrices (keeps 16-byte row alignment)
+
+template <typename T, int K, int V, bool BWD>
+__global__ __launch_bounds__(64) void prep_kernel(ChunkArgs<T> p) {
+    constexpr int KT = K / 16, VT = V / 16;
+    __shared__ __attribute__((aligned(16))) float sN[32 * LDP];   // A_ab, rank-major
+    __shared__ __attribute__((aligned(16))) float sT[32 * LDP];   // (I - A_ab)^-1
+
+    const int cid = blockIdx.x, h = blockIdx.y;
+    ChunkPos cp;
+    if (!locate_chunk(p.st, cid, cp)) return;
+    const int l = lane_id(), g = l >> 4, c = l & 15;
+    const int H = p.H;
+    const bool rowok = c < cp.len;
+    const int64_t tok = cp.tok0 + c;
+    const int64_t qoff = (tok * H + h) * K + 4 * g;                 // + 16*kt
+    const int64_t aoff0 = ((tok * RANK + 0) * H + h) * K + 4 * g;
+    const int64_t aoff1 = ((tok * RANK + 1) * H + h) * K + 4 * g;
+    const int64_t voff = (tok * H + h) * V + 4 * g;
+    const int64_t chw = (int64_t)h * p.st.nch + cid;                // chunk-head slot in the workspace
+    const float scale = p.scale;
+
+    // ---- phase A: cumulative decays and the score tiles (rows i, inner j) -----------------------------------
+    f32x4 gi[KT], ge[KT];
+    f32x4 aqk = zero4(), aqb[2] = {zero4(), zero4()}, aak[2] = {zero4(), zero4()};
+    f32x4 aab[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
+    f32x4 aqbT[2] = {zero4(), zero4()};
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+        const f32x4 g4 = ld_gk4(p.gk, qoff + 16 * kt, p.gk_f32, rowok);
+        gi[kt] = scan16_incl(g4);
+        ge[kt] = gi[kt] - g4;
+        const f32x4 m = bcast16(gi[kt], MID);
+        const f32x4 eq = exp4<T>(gi[kt] - m), ek = exp4<T>(m - gi[kt]), ea = exp4<T>(ge[kt] - m);
+        const f32x4 q4 = to_f32(ld_frag_if(p.q + qoff + 16 * kt, rowok));
+        const f32x4 k4 = to_f32(ld_frag_if(p.k + qoff + 16 * kt, rowok));
+        const f32x4 a0 = to_f32(ld_frag_if(p.a + aoff0 + 16 * kt, rowok));
+        const f32x4 a1 = to_f32(ld_frag_if(p.a + aoff1 + 16 * kt, rowok));
+        const f32x4 b0 = to_f32(ld_frag_if(p.b + aoff0 + 16 * kt, rowok));
+        const f32x4 b1 = to_f32(ld_frag_if(p.b + aoff1 + 16 * kt, rowok));
+        const Frag<T> qh = to_frag<T>(q4 * eq * scale), kh = to_frag<T>(k4 * ek);
+        const Frag<T> ah[2] = {to_frag<T>(a0 * ea), to_frag<T>(a1 * ea)};
+        const Frag<T> bh[2] = {to_frag<T>(b0 * ek), to_frag<T>(b1 * ek)};
+        aqk = mm(qh, kh, aqk);
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            aqb[s] = mm(qh, bh[s], aqb[s]);
+            aak[s] = mm(ah[s], kh, aak[s]);
+            if (BWD) aqbT[s] = mm(bh[s], qh, aqbT[s]);
+#pragma unroll
+            for (int r = 0; r < 2; ++r) aab[r][s] = mm(ah[r], bh[s], aab[r][s]);
+        }
+    }
+    // causal masks: lane (g,c) reg i is entry (row c, inner 4g+i)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int j = 4 * g + i;
+        const bool le = j <= c, lt = j < c, tle = c <= j;
+        if (!le) { aqk[i] = 0.f; aqb[0][i] = 0.f; aqb[1][i] = 0.f; }
+        if (!lt) { aak[0][i] = 0.f; aak[1][i] = 0.f; aab[0][0][i] = 0.f; aab[0][1][i] = 0.f; aab[1][0][i] = 0.f; aab[1][1][i] = 0.f; }
+        if (!tle) { aqbT[0][i] = 0.f; aqbT[1][i] = 0.f; }
+    }
+    if (!BWD) {
+        st_tile(p.ws.AQK + chw * TILE, to_frag<T>(aqk));
+        st_tile(p.ws.AQB + (chw * 2 + 0) * TILE, to_frag<T>(aqb[0]));
+        st_tile(p.ws.AQB + (chw * 2 + 1) * TILE, to_frag<T>(aqb[1]));
+    } else {
+        st_tile(p.ws.AQBT + (chw * 2 + 0) * TILE, to_frag<T>(aqbT[0]));
+        st_tile(p.ws.AQBT + (chw * 2 + 1) * TILE, to_frag<T>(aqbT[1]));
+    }
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+            *reinterpret_cast<f32x4*>(&sN[(16 * r + c) * LDP + 16 * s + 4 * g]) = aab[r][s];
+    __syncthreads();
+
+    // ---- phase B: (I - A_ab)^-1 by forward substitution over tokens, two rank rows x 32 columns per step ----
+    {
+        const int r = l >> 5, col = l & 31;
+        for (int i = 0; i < 16; ++i) {
+            const int row = 16 * r + i;
+            float acc = (col == row) ? 1.f : 0.f;
+            for (int j = 0; j < i; ++j) {
+                acc = fmaf(sN[row * LDP + j], sT[j * LDP + col], acc);
+                acc = fmaf(sN[row * LDP + 16 + j], sT[(16 + j) * LDP + col], acc);
+            }
+            sT[row * LDP + col] = acc;
+            __syncthreads();
+        }
+    }
+    Frag<T> tm[2][2];   // F(Tm^{s s'}): rows i, inner j
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+            tm[s][s2] = to_frag<T>(*reinterpret_cast<const f32x4*>(&sT[(16 * s + c) * LDP + 16 * s2 + 4 * g]));
+    if (BWD) {
+        float* tmw = p.ws.TM + chw * 1024;
+        const int row = l >> 1, c0 = (l & 1) * 16;
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+            *reinterpret_cast<f32x4*>(tmw + row * 32 + c0 + 4 * x) = *reinterpret_cast<const f32x4*>(&sT[row * LDP + c0 + 4 * x]);
+    }
+
+    const Frag<T> ident = ident_frag<T>();
+
+    // ---- phase C: w = Tm ag and the gated copies, one channel tile at a time ---------------------------------
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+        const f32x4 gl = bcast16(gi[kt], CH - 1);
+        const f32x4 egi = exp4<T>(gi[kt]), ege = exp4<T>(ge[kt]), edn = exp4<T>(gl - gi[kt]);
+        const f32x4 q4 = to_f32(ld_frag_if(p.q + qoff + 16 * kt, rowok));
+        const f32x4 k4 = to_f32(ld_frag_if(p.k + qoff + 16 * kt, rowok));
+        const f32x4 a0 = to_f32(ld_frag_if(p.a + aoff0 + 16 * kt, rowok));
+        const f32x4 a1 = to_f32(ld_frag_if(p.a + aoff1 + 16 * kt, rowok));
+        const f32x4 b0 = to_f32(ld_frag_if(p.b + aoff0 + 16 * kt, rowok));
+        const f32x4 b1 = to_f32(ld_frag_if(p.b + aoff1 + 16 * kt, rowok));
+        const Frag<T> agT[2] = {transpose(to_frag<T>(a0 * ege), ident), transpose(to_frag<T>(a1 * ege), ident)};
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            f32x4 w = zero4();
+            w = mm(tm[s][0], agT[0], w);
+            w = mm(tm[s][1], agT[1], w);
+            st_tile(p.ws.W + ((chw * 2 + s) * KT + kt) * TILE, to_frag<T>(w));
+            if (BWD) {
+                f32x4 wT = zero4();
+                wT = mm(agT[0], tm[s][0], wT);
+                wT = mm(agT[1], tm[s][1], wT);
+                st_tile(p.ws.WT + ((chw * 2 + s) * KT + kt) * TILE, to_frag<T>(wT));
+            }
+        }
+        const Frag<T> qg = to_frag<T>(q4 * egi * scale);
+        const Frag<T> kg = to_frag<T>(k4 * edn);
+        const Frag<T> bg[2] = {to_frag<T>(b0 * edn), to_frag<T>(b1 * edn)};
+        st_tile(p.ws.KGT + (chw * KT + kt) * TILE, transpose(kg, ident));
+        st_tile(p.ws.BGT + ((chw * 2 + 0) * KT + kt) * TILE, transpose(bg[0], ident));
+        st_tile(p.ws.BGT + ((chw * 2 + 1) * KT + kt) * TILE, transpose(bg[1], ident));
+        if (!BWD) {
+            st_tile(p.ws.QG + (chw * KT + kt) * TILE, qg);
+        } else {
+            st_tile(p.ws.QGT + (chw * KT + kt) * TILE, transpose(qg, ident));
+            st_tile(p.ws.BG + ((chw * 2 + 0) * KT + kt) * TILE, bg[0]);
+            st_tile(p.ws.BG + ((chw * 2 + 1) * KT + kt) * TILE, bg[1]);
+        }
+        if (c == 0) *reinterpret_cast<f32x4*>(p.ws.EGL + chw * K + 16 * kt + 4 * g) = exp4<T>(gl);
+    }
+
+    // ---- phase D: u = Tm (A_ak v), kept transposed (rows value, inner token) ---------------------------------
+    const Frag<T> aakf[2] = {to_frag<T>(aak[0]), to_frag<T>(aak[1])};
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt) {
+        const Frag<T> vT = transpose(ld_frag_if(p.v + voff + 16 * vt, rowok), ident);
+        st_tile(p.ws.VTT + (chw * VT + vt) * TILE, vT);
+        const Frag<T> mT[2] = {to_frag<T>(mm(vT, aakf[0], zero4())), to_frag<T>(mm(vT, aakf[1], zero4()))};
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            f32x4 uT = zero4();
+            uT = mm(mT[0], tm[s][0], uT);
+            uT = mm(mT[1], tm[s][1], uT);
+            st_tile(p.ws.UT + ((chw * 2 + s) * VT + vt) * TILE, to_frag<T>(uT));
+        }
+    }
+}
+
+// ---- chunk table for packed variable-length batches ----------------------------------------------------------
+__global__ void build_chunk_table_kernel(const int64_t* cu, int N, int nch, int32_t* chunk_off, int32_t* chunk_seq) {
+    // one workgroup; N is small (number of packed sequences)
+    __shared__ int total;
+    if (threadIdx.x == 0) {
+        int acc = 0;
+        for (int n = 0; n < N; ++n) {
+            chunk_off[n] = acc;
+            const int64_t len = cu[n + 1] - cu[n];
+            acc += (int)((len + CH - 1) / CH);
+        }
+        if (acc > nch) acc = nch;   // cannot happen for a monotone cu_seqlens ending at T; guards the table writes
+        chunk_off[N] = acc;
+        total = acc;
+    }
+    __syncthreads();
+    for (int cid = threadIdx.x; cid < total; cid += blockDim.x) {
+        int lo = 0, hi = N - 1;   // last n with chunk_off[n] <= cid
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (chunk_off[mid] <= cid) lo = mid; else hi = mid - 1;
+        }
+        chunk_seq[cid] = lo;
+    }
+}
+
+template <typename T, int K, int V>
+static hipError_t launch_prep_kv(const ChunkArgs<T>& a, bool bwd, hipStream_t stream) {
+    dim3 grid(a.st.nch, a.H), block(64);
+    if (bwd) hipLaunchKernelGGL((prep_kernel<T, K, V, true>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((prep_kernel<T, K, V, false>), grid, block, 0, stream, a);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_prep(const ChunkArgs<T>& a, int K, int V, bool bwd, hipStream_t stream) {
+    if (K == 64 && V == 64) return launch_prep_kv<T, 64, 64>(a, bwd, stream);
+    if (K == 128 && V == 128) return launch_prep_kv<T, 128, 128>(a, bwd, stream);
+    if (K == 64 && V == 128) return launch_prep_kv<T, 64, 128>(a, bwd, stream);
+    if (K == 128 && V == 64) return launch_prep_kv<T, 128, 64>(a, bwd, stream);
+    return hipErrorInvalidValue;
+}
+template hipError_t launch_prep<bf16>(const ChunkArgs<bf16>&, int, int, bool, hipStream_t);
+template hipError_t launch_prep<float>(const ChunkArgs<float>&, int, int, bool, hipStream_t);
+
+hipError_t launch_chunk_table(const int64_t* cu, int N, int nch, int32_t* chunk_off, int32_t* chunk_seq, hipStream_t stream) {
+    hipLaunchKernelGGL(build_chunk_table_kernel, dim3(1), dim3(256), 0, stream, cu, N, nch, chunk_off, chunk_seq);
+    return hipGetLastError();
+}
+
+}  // namespace hdla

@@ -1,0 +1,110 @@
+"""ctypes binding of libhdla_hip.so (the C ABI declared in include/hdla_hip.h).
+
+The library is the only compute path: if it cannot be loaded every operator raises, there is no fallback.
+"""
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+HDLA_BF16, HDLA_FP32 = 0, 1
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_NAME = "libhdla_hip.so"
+_lib = None
+
+
+class HdlaDims(ctypes.Structure):
+    _fields_ = [
+        ("B", ctypes.c_int32), ("T", ctypes.c_int32), ("H", ctypes.c_int32), ("K", ctypes.c_int32),
+        ("V", ctypes.c_int32), ("R", ctypes.c_int32), ("N", ctypes.c_int32),
+        ("in_dtype", ctypes.c_int32), ("gk_dtype", ctypes.c_int32), ("scale", ctypes.c_float),
+        ("cu_seqlens", ctypes.c_void_p),
+    ]
+
+
+class HdlaWsLayout(ctypes.Structure):
+    _names = ["nch", "W", "UT", "KGT", "BGT", "VTT", "EGL", "QG", "AQK", "AQB", "AQBT", "BG", "WT", "QGT", "TM",
+              "HC", "DHC", "VN", "DVN", "CHUNK_OFF", "CHUNK_SEQ", "total"]
+    _fields_ = [(n, ctypes.c_int64) for n in _names]
+
+
+class HdlaError(RuntimeError):
+    pass
+
+
+def lib_path() -> str:
+    return os.environ.get("HDLA_HIP_LIB", os.path.join(_HERE, _LIB_NAME))
+
+
+def load():
+    """Load the shared library once; raise if it is missing (build it with __graft_entry__.build() or
+    `make -C hdla-impl_amd/csrc`)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = lib_path()
+    if not os.path.exists(path):
+        raise HdlaError(f"{path} not found: build the HIP library first (make -C hdla-impl_amd/csrc); "
+                        "there is no CPU or PyTorch fallback for these operators")
+    lib = ctypes.CDLL(path)
+    P, F = ctypes.c_void_p, ctypes.POINTER(HdlaDims)
+    lib.hdla_version.restype = ctypes.c_int
+    lib.hdla_version.argtypes = []
+    lib.hdla_strerror.restype = ctypes.c_char_p
+    lib.hdla_strerror.argtypes = [ctypes.c_int]
+    lib.hdla_workspace_bytes.restype = ctypes.c_size_t
+    lib.hdla_workspace_bytes.argtypes = [F, ctypes.c_int]
+    lib.hdla_workspace_layout.restype = ctypes.c_int
+    lib.hdla_workspace_layout.argtypes = [F, ctypes.c_int, ctypes.POINTER(HdlaWsLayout)]
+    lib.hdla_chunk_fwd.restype = ctypes.c_int
+    lib.hdla_chunk_fwd.argtypes = [F] + [P] * 9 + [P, ctypes.c_size_t, P]
+    lib.hdla_chunk_bwd.restype = ctypes.c_int
+    lib.hdla_chunk_bwd.argtypes = [F] + [P] * 16 + [P, ctypes.c_size_t, P]
+    lib.hdla_chunk_stages.restype = ctypes.c_int
+    lib.hdla_chunk_stages.argtypes = [F, ctypes.c_int, ctypes.c_int] + [P] * 18 + [P, ctypes.c_size_t, P]
+    lib.hdla_recurrent_fwd.restype = ctypes.c_int
+    lib.hdla_recurrent_fwd.argtypes = [F] + [P] * 6 + [ctypes.c_int] + [P] * 4
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().hdla_strerror(rc).decode()
+        raise HdlaError(f"{what} failed with code {rc}: {msg}")
+
+
+def ptr(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.bfloat16:
+        return HDLA_BF16
+    if dt == torch.float32:
+        return HDLA_FP32
+    raise HdlaError(f"unsupported dtype {dt}")
+
+
+def make_dims(B, T, H, K, V, R, N, in_dtype, gk_dtype, scale, cu_seqlens: Optional[torch.Tensor]) -> HdlaDims:
+    return HdlaDims(B, T, H, K, V, R, N, dtype_code(in_dtype), dtype_code(gk_dtype), float(scale),
+                    None if cu_seqlens is None else cu_seqlens.data_ptr())
+
+
+def current_stream(device) -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def workspace(dims: HdlaDims, pass_: int, device) -> torch.Tensor:
+    n = load().hdla_workspace_bytes(ctypes.byref(dims), pass_)
+    if n == 0:
+        raise HdlaError("hdla_workspace_bytes rejected the dimensions "
+                        f"(B={dims.B},T={dims.T},H={dims.H},K={dims.K},V={dims.V},R={dims.R},N={dims.N})")
+    return torch.empty(n, dtype=torch.uint8, device=device)
+
+
+def workspace_layout(dims: HdlaDims, pass_: int) -> dict:
+    out = HdlaWsLayout()
+    check(load().hdla_workspace_layout(ctypes.byref(dims), pass_, ctypes.byref(out)), "hdla_workspace_layout")
+    return {n: getattr(out, n) for n in HdlaWsLayout._names}

@@ -1,0 +1,119 @@
+/* libhdla_hip.so -- C ABI of the MI355X (gfx950) kernels for HDLA's rank-2 DPLR delta-rule linear attention.
+ *
+ * This is the boundary a host binding talks to (ctypes in this repository; any FFI works): plain pointers
+ * and sizes, no C++ or torch types.  It stands in for the reference's Python launcher layer, which is the
+ * level at which its Triton kernels are driven:
+ *
+ *   hdla_chunk_fwd      <-  chunk_hrdplr_fwd                     HRDPLR/hrdplr.py:25-99
+ *                           (chunk_fwd_intra_dplr_fn HRDPLR/fwd_func.py:16, fwd_prepare_wy_repr :153,
+ *                            chunk_dplr_fwd_h :210, chunk_dplr_fwd_o :274 and fla's chunk_rwkv6_fwd_cumsum)
+ *   hdla_chunk_bwd      <-  ChunkDPLRDeltaRuleFunction.backward   HRDPLR/hrdplr.py:149-284
+ *                           (chunk_dplr_bwd_dAu HRDPLR/bwd_func.py:18, _dhu :63, _dv :125, _bwd_o :155,
+ *                            _bwd_wy :218, _bwd_dqk_intra :274)
+ *   hdla_recurrent_fwd  <-  fused_recurrent_dplr_delta_rule_fwd   HRDPLR/recurrent.py:121-177
+ *
+ * Conventions
+ *   - All tensor pointers are DEVICE pointers to contiguous, 16-byte aligned buffers owned by the caller.
+ *     Layouts are the reference's (head_first = False): q,k,gk [B,T,H,K]; v,o,do [B,T,H,V];
+ *     a,b [B,T*R,H,K] with row t*R + r (HRDPLR/recurrent.py:66-67); states [N,H,K,V] fp32.
+ *   - The library allocates nothing.  The caller passes a workspace of hdla_workspace_bytes() bytes
+ *     (256-byte aligned); its contents are scratch and may be discarded after the call.
+ *   - Calls are asynchronous on `stream` (a hipStream_t passed as void*; NULL = the default stream), never
+ *     synchronise, keep no global mutable state and are reentrant as long as workspaces are distinct.
+ *   - Return value: 0 = success, < 0 = argument error detected on the host before any launch (see
+ *     hdla_strerror), > 0 = a hipError_t from a kernel launch.
+ *   - Supported: R = 2; K, V in {64, 128}; in_dtype bf16 or fp32; gk fp32, or bf16 when in_dtype is bf16.
+ *     Scores are factorised around the middle of each 16-token chunk, which is exact as long as the summed
+ *     log-decay of any 8 consecutive tokens of one channel stays above about -80.
+ */
+#ifndef HDLA_HIP_H
+#define HDLA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HDLA_VERSION 100
+
+enum { HDLA_BF16 = 0, HDLA_FP32 = 1 };
+
+enum {
+    HDLA_OK = 0,
+    HDLA_ERR_NULL = -1,        /* a required pointer is NULL */
+    HDLA_ERR_SHAPE = -2,       /* unsupported K/V, non-positive dimension, or grid limit exceeded */
+    HDLA_ERR_RANK = -3,        /* R != 2 */
+    HDLA_ERR_DTYPE = -4,       /* unknown dtype code or unsupported combination */
+    HDLA_ERR_WORKSPACE = -5,   /* workspace NULL, misaligned or too small */
+    HDLA_ERR_ALIGN = -6,       /* a tensor pointer is not 16-byte aligned */
+    HDLA_ERR_SEQ = -7          /* cu_seqlens given with B != 1, or N inconsistent with B */
+};
+
+typedef struct hdla_dims {
+    int32_t B, T, H, K, V, R;
+    int32_t N;                 /* sequences: B without cu_seqlens, else len(cu_seqlens) - 1 (and B == 1) */
+    int32_t in_dtype;          /* q,k,v,a,b,o,do and dq,dk,dv,da,db */
+    int32_t gk_dtype;          /* gk and dgk */
+    float scale;               /* applied to q (HRDPLR/hrdplr.py:302) */
+    const int64_t* cu_seqlens; /* DEVICE int64[N+1] cumulative sequence starts on the T axis, or NULL */
+} hdla_dims;
+
+/* Byte offsets of the named intermediates inside the workspace (0 = not part of this pass); for tests and
+ * debugging: after hdla_chunk_bwd every stage's output is still there.  "tiles" are 16x16 blocks in MFMA
+ * fragment order (element 4*lane + i of a block is row lane%16, inner index 4*(lane/16) + i), laid out
+ * [H][nch][...]; "rows" are row-major. */
+typedef struct hdla_ws_layout {
+    int64_t nch;               /* chunk slots per head */
+    int64_t W, UT, KGT, BGT, VTT, EGL, QG, AQK, AQB, AQBT, BG, WT, QGT, TM, HC, DHC, VN, DVN;
+    int64_t CHUNK_OFF, CHUNK_SEQ;
+    int64_t total;
+} hdla_ws_layout;
+
+int hdla_version(void);
+const char* hdla_strerror(int code);
+
+/* pass: 0 = forward, 1 = backward.  Returns 0 for invalid dims. */
+size_t hdla_workspace_bytes(const hdla_dims* dims, int pass);
+int hdla_workspace_layout(const hdla_dims* dims, int pass, hdla_ws_layout* out);
+
+/* Chunked forward (HRDPLR/hrdplr.py:25-99).  h0 and ht are optional (NULL): zero initial state / final state
+ * not wanted.  o has q's dtype (HRDPLR/hrdplr.py:144), ht is fp32 (HRDPLR/fwd_func.py:244). */
+int hdla_chunk_fwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
+                   const void* b, const void* gk, const float* h0, void* o, float* ht,
+                   void* workspace, size_t workspace_bytes, void* stream);
+
+/* Chunked backward (HRDPLR/hrdplr.py:149-284): recomputes the forward intermediates from the inputs, then
+ * writes dq,dk,dv,da,db (in_dtype), dgk (gk_dtype) and, if dh0 != NULL, dh0 (fp32).  dht may be NULL. */
+int hdla_chunk_bwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
+                   const void* b, const void* gk, const float* h0, const void* d_o, const float* dht,
+                   void* dq, void* dk, void* dv, void* da, void* db, void* dgk, float* dh0,
+                   void* workspace, size_t workspace_bytes, void* stream);
+
+/* Profiling / debugging aid with no counterpart in the reference: runs only the kernels selected by `stages`
+ * (a bit mask) of the forward (pass 0) or backward (pass 1) launch sequence, in order, on the same workspace, so
+ * that a caller can bracket each kernel with events on `stream`.  A stage reads what the earlier stages left
+ * in the workspace.  Unused tensor arguments of the other pass may be NULL. */
+enum {
+    HDLA_STAGE_PREP = 1,        /* chunk table (with cu_seqlens) + prep kernel */
+    HDLA_STAGE_SCAN_FWD = 2,    /* forward state scan (writes o in pass 0; h and v_new in pass 1) */
+    HDLA_STAGE_SCAN_BWD = 4,    /* reverse state-gradient scan (pass 1 only) */
+    HDLA_STAGE_CHUNK_GRAD = 8,  /* per-chunk gradient assembly (pass 1 only) */
+    HDLA_STAGE_ALL = 15
+};
+int hdla_chunk_stages(const hdla_dims* dims, int pass, int stages, const void* q, const void* k, const void* v,
+                      const void* a, const void* b, const void* gk, const float* h0, void* o, float* ht,
+                      const void* d_o, const float* dht, void* dq, void* dk, void* dv, void* da, void* db, void* dgk,
+                      float* dh0, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Token-serial recurrence over T tokens per sequence (HRDPLR/recurrent.py:121-177), forward only.
+ * reverse != 0 walks each sequence from its last token to its first (recurrent.py:63,108). */
+int hdla_recurrent_fwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
+                       const void* b, const void* gk, int reverse, const float* h0, void* o, float* ht,
+                       void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HDLA_HIP_H */

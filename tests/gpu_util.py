@@ -1,0 +1,38 @@
+"""Helpers shared by the GPU parity tests: decoding of workspace buffers written by the HIP kernels."""
+import torch
+
+
+def _raw(ws: torch.Tensor, off: int, count: int, dtype: torch.dtype) -> torch.Tensor:
+    nbytes = count * torch.empty((), dtype=dtype).element_size()
+    return ws[off:off + nbytes].view(dtype)
+
+
+def tiles(ws, off, dtype, H, nch, *lead):
+    """Buffer of 16x16 tiles in fragment order -> float64 tensor [H, nch, *lead, 16 (row), 16 (inner)].
+
+    Element 4*lane + i of a tile is row lane % 16, inner index 4*(lane // 16) + i."""
+    n = 1
+    for x in lead:
+        n *= x
+    t = _raw(ws, off, H * nch * n * 256, dtype).double().reshape(H, nch, *lead, 4, 16, 4)   # [g][c][i]
+    nd = t.dim()
+    t = t.transpose(nd - 3, nd - 2)                                                          # [c][g][i]
+    return t.reshape(H, nch, *lead, 16, 16).cpu()
+
+
+def rows(ws, off, dtype, H, nch, *shape):
+    n = 1
+    for x in shape:
+        n *= x
+    return _raw(ws, off, H * nch * n, dtype).double().reshape(H, nch, *shape).cpu()
+
+
+def cat_tiles(t, dim_tiles, transpose=False):
+    """[..., nt, 16, 16] -> rows x (nt*16) (or its transpose view when the tiles hold the transposed matrix).
+
+    With transpose=False the tile index runs along the inner dimension: result [..., 16, nt*16].
+    With transpose=True each tile is (rows = tiled dimension, inner = other): result [..., 16 (inner), nt*16]."""
+    assert dim_tiles == t.dim() - 3
+    if not transpose:
+        return torch.cat([t[..., i, :, :] for i in range(t.shape[-3])], dim=-1)
+    return torch.cat([t[..., i, :, :].transpose(-1, -2) for i in range(t.shape[-3])], dim=-1)

@@ -1,0 +1,239 @@
+"""GPU parity of the chunked operator (forward + backward) against the CPU oracle, through the public API and
+hence through the C ABI.  Tolerances are the ones the task states, in relative L2 norm: outputs and final state
+<= 5e-3, gradients <= 1e-2 for bf16 inputs; <= 1e-5 for fp32 inputs."""
+import pytest
+import torch
+
+from hdla_hip import chunk_hrdplr_delta_rule, fused_recurrent_dplr_delta_rule
+from hdla_hip.synthetic import make_config, make_inputs
+from oracle import hrdplr_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+TOL = {torch.bfloat16: (5e-3, 1e-2), torch.float32: (1e-5, 1e-5)}
+GRADS = ["dq", "dk", "dv", "da", "db", "dgk", "dh0"]
+
+
+def _oracle(inp, dtype, scale, heads=None, use_h0=True, use_dht=True, cu=None, R=2):
+    """float64 recurrence + autograd on the dtype-rounded inputs (optionally on a subset of heads)."""
+    sl = (lambda x: x) if heads is None else (lambda x: x[:, :, heads])
+    slh = (lambda x: x) if heads is None else (lambda x: x[:, heads])
+    leaves = [sl(t.to(dtype)).double().requires_grad_() for t in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    h0 = slh(inp.h0).double().requires_grad_() if use_h0 else None
+    o, ht = O.recurrence(*leaves, scale, h0, cu_seqlens=cu, rank_ab=R)
+    do = sl(inp.do.to(dtype)).double()
+    outs, gos = [o], [do]
+    if use_dht:
+        outs.append(ht); gos.append(slh(inp.dht).double())
+    g = torch.autograd.grad(outs, leaves + ([h0] if use_h0 else []), gos)
+    return o.detach(), ht.detach(), dict(zip(GRADS, g))
+
+
+def _gpu(inp, dtype, scale, use_h0=True, use_dht=True, cu=None, R=2, chunk_size=16):
+    leaves = [t.to(dtype).to(DEV).requires_grad_() for t in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    h0 = inp.h0.to(DEV).requires_grad_() if use_h0 else None
+    o, ht = chunk_hrdplr_delta_rule(*leaves, R, scale=scale, initial_state=h0, output_final_state=True,
+                                    chunk_size=chunk_size, cu_seqlens=None if cu is None else cu.to(DEV))
+    assert o.dtype == dtype and ht.dtype == torch.float32
+    outs, gos = [o], [inp.do.to(dtype).to(DEV)]
+    if use_dht:
+        outs.append(ht); gos.append(inp.dht.to(DEV))
+    g = torch.autograd.grad(outs, leaves + ([h0] if use_h0 else []), gos)
+    for x, l in zip(g, leaves):
+        assert x.dtype == l.dtype and x.shape == l.shape
+    return o.detach(), ht.detach(), dict(zip(GRADS, g))
+
+
+def _compare(got, ref, dtype, heads=None, what=""):
+    tol_o, tol_g = TOL[dtype]
+    o, ht, g = got
+    o_r, ht_r, g_r = ref
+    if heads is not None:
+        o, ht = o[:, :, heads], ht[:, heads]
+    errs = {"o": O.rel_l2(o, o_r), "ht": O.rel_l2(ht, ht_r)}
+    for n in g_r:
+        x = g[n]
+        if heads is not None:
+            x = x[:, heads] if n == "dh0" else x[:, :, heads]
+        errs[n] = O.rel_l2(x, g_r[n])
+    print(what, {k: f"{v:.2e}" for k, v in errs.items()}, flush=True)
+    assert errs["o"] <= tol_o and errs["ht"] <= tol_o, errs
+    for n in g_r:
+        assert errs[n] <= tol_g, (n, errs)
+
+
+CASES = [
+    # dtype, B, T, H, K, V, gk_div, scale
+    (torch.float32, 2, 40, 2, 64, 64, 1.0, 0.7),
+    (torch.float32, 1, 64, 2, 128, 128, 1.0, 1.0),
+    (torch.float32, 1, 50, 2, 128, 64, 16.0, 0.5),
+    (torch.float32, 1, 33, 2, 64, 128, 4.0, 1.0),
+    (torch.bfloat16, 2, 40, 2, 64, 64, 1.0, 0.7),
+    (torch.bfloat16, 1, 100, 3, 128, 64, 1.0, 1.0),
+    (torch.bfloat16, 2, 256, 2, 64, 128, 16.0, 1.0),
+    (torch.bfloat16, 1, 256, 2, 128, 128, 16.0, 0.125),
+    (torch.bfloat16, 1, 1, 1, 64, 64, 1.0, 1.0),
+    (torch.bfloat16, 1, 15, 1, 64, 64, 1.0, 1.0),
+    (torch.bfloat16, 1, 17, 1, 64, 64, 1.0, 1.0),
+]
+
+
+@pytest.mark.parametrize("dtype,B,T,H,K,V,gk_div,scale", CASES)
+def test_forward_backward_parity(dtype, B, T, H, K, V, gk_div, scale):
+    inp = make_inputs(100 + T, B, T, H, K, V, gk_div=gk_div)
+    _compare(_gpu(inp, dtype, scale), _oracle(inp, dtype, scale), dtype, what=f"{dtype} B{B} T{T} H{H} K{K} V{V}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_no_initial_state_no_final_gradient(dtype):
+    inp = make_inputs(7, 2, 48, 2, 64, 64)
+    _compare(_gpu(inp, dtype, 1.0, use_h0=False, use_dht=False), _oracle(inp, dtype, 1.0, use_h0=False, use_dht=False),
+             dtype)
+
+
+def test_reference_integrated_test_shape_fp32():
+    """Shape and distributions of the reference's end-to-end test (test_integrated.py:9-42): B2 H4 T256 K128 V64
+    fp32, scale 1, gk = logsigmoid(randn), random initial state, random do / dht."""
+    inp = make_inputs(8, 2, 256, 4, 128, 64, gk_div=1.0)
+    _compare(_gpu(inp, torch.float32, 1.0), _oracle(inp, torch.float32, 1.0), torch.float32)
+
+
+@pytest.mark.parametrize("cfg,dtype", [(1, torch.bfloat16), (2, torch.bfloat16), (2, torch.float32)])
+def test_benchmark_config_full_size_head_subset(cfg, dtype):
+    """Configurations 1 and 2 at full size (B4 T2048 H16 K=V=64) on the GPU; the CPU oracle covers three
+    (batch, head) pairs of them at the full sequence length (heads are independent recurrences)."""
+    inp = make_config(cfg)
+    use_h0 = cfg == 2
+    got = _gpu(inp, dtype, 1.0, use_h0=use_h0, use_dht=use_h0)
+    heads = [0, 7, 15]
+    sub = type(inp)(*[None if x is None else x[:1] for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk, inp.h0, inp.do,
+                                                                 inp.dht)])
+    ref = _oracle(sub, dtype, 1.0, heads=heads, use_h0=use_h0, use_dht=use_h0)
+    got1 = (got[0][:1], got[1][:1], {n: x[:1] for n, x in got[2].items()})
+    _compare(got1, ref, dtype, heads=heads, what=f"cfg{cfg} {dtype}")
+
+
+def test_full_size_chunk_vs_recurrent_kernel_and_fp32_path():
+    """Size-independent cross checks at configuration 2's full size, all on the GPU: the bf16 chunked forward
+    against the fp32-state recurrent kernel, and the bf16 gradients against the fp32-input chunked path."""
+    inp = make_config(2)
+    o, ht, g = _gpu(inp, torch.bfloat16, 1.0)
+    t = [x.bfloat16().to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    o_r, ht_r = fused_recurrent_dplr_delta_rule(*t, 2, scale=1.0, initial_state=inp.h0.to(DEV), output_final_state=True)
+    assert O.rel_l2(o, o_r) <= 5e-3 and O.rel_l2(ht, ht_r) <= 5e-3
+    inp32 = type(inp)(*[x.bfloat16().float() if i < 6 or i == 7 else x
+                        for i, x in enumerate((inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk, inp.h0, inp.do, inp.dht))])
+    o32, ht32, g32 = _gpu(inp32, torch.float32, 1.0)
+    errs = {n: O.rel_l2(g[n], g32[n]) for n in GRADS}
+    print({k: f"{v:.2e}" for k, v in errs.items()}, O.rel_l2(o, o32), O.rel_l2(ht, ht32), flush=True)
+    assert all(e <= 1e-2 for e in errs.values()), errs
+    assert O.rel_l2(o, o32) <= 5e-3 and O.rel_l2(ht, ht32) <= 5e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_varlen_config3_reduced(dtype):
+    """Configuration 3's packed layout (four sequences 1:2:2:3) at T = 1024 (K = V = 128), forward + backward."""
+    inp = make_config(3, shape=(1, 1024, 2, 128, 128))
+    cu = inp.cu_seqlens
+    _compare(_gpu(inp, dtype, 1.0, cu=cu), _oracle(inp, dtype, 1.0, cu=cu), dtype, what=f"varlen {dtype}")
+
+
+def test_varlen_ragged_and_empty_sequences():
+    inp = make_inputs(9, 1, 100, 2, 64, 64, n_states=5)
+    cu = torch.tensor([0, 3, 3, 36, 83, 100])
+    _compare(_gpu(inp, torch.float32, 1.0, cu=cu), _oracle(inp, torch.float32, 1.0, cu=cu), torch.float32)
+
+
+def test_varlen_equals_per_sequence_calls_bitwise():
+    inp = make_inputs(10, 1, 96, 2, 64, 64, n_states=3)
+    cu = torch.tensor([0, 32, 48, 96])
+    t = [x.bfloat16().to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    o, ht = chunk_hrdplr_delta_rule(*t, 2, scale=1.0, initial_state=inp.h0.to(DEV), output_final_state=True,
+                                    cu_seqlens=cu.to(DEV))
+    for n in range(3):
+        s, e = int(cu[n]), int(cu[n + 1])
+        q, k, v, a, b, gk = t
+        on, hn = chunk_hrdplr_delta_rule(q[:, s:e], k[:, s:e], v[:, s:e], a[:, 2 * s:2 * e], b[:, 2 * s:2 * e],
+                                         gk[:, s:e], 2, scale=1.0, initial_state=inp.h0[n:n + 1].to(DEV),
+                                         output_final_state=True)
+        assert torch.equal(o[:, s:e], on) and torch.equal(ht[n:n + 1], hn)
+
+
+def test_state_hand_off_and_chunk_size_hint():
+    inp = make_inputs(11, 2, 128, 2, 64, 64)
+    t = [x.bfloat16().to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    q, k, v, a, b, gk = t
+    h0 = inp.h0.to(DEV)
+    o, ht = chunk_hrdplr_delta_rule(*t, 2, scale=1.0, initial_state=h0, output_final_state=True, chunk_size=16)
+    o64, ht64 = chunk_hrdplr_delta_rule(*t, 2, scale=1.0, initial_state=h0, output_final_state=True, chunk_size=64)
+    assert torch.equal(o, o64) and torch.equal(ht, ht64)
+    s = 48                                  # a multiple of 16: the split run sees the same chunks, so bitwise equal
+    o1, hm = chunk_hrdplr_delta_rule(q[:, :s], k[:, :s], v[:, :s], a[:, :2 * s], b[:, :2 * s], gk[:, :s], 2, scale=1.0,
+                                     initial_state=h0, output_final_state=True)
+    o2, h2 = chunk_hrdplr_delta_rule(q[:, s:], k[:, s:], v[:, s:], a[:, 2 * s:], b[:, 2 * s:], gk[:, s:], 2, scale=1.0,
+                                     initial_state=hm, output_final_state=True)
+    assert torch.equal(torch.cat([o1, o2], 1), o) and torch.equal(h2, ht)
+    on, hn = chunk_hrdplr_delta_rule(*t, 2, scale=1.0, initial_state=h0, output_final_state=False)
+    assert hn is None and torch.equal(on, o)
+
+
+def test_default_scale_and_prescaled_q():
+    inp = make_inputs(12, 1, 64, 2, 64, 64)
+    t = [x.float().to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    o1, _ = chunk_hrdplr_delta_rule(*t, 2)                                   # scale = K ** -0.5
+    o2, _ = chunk_hrdplr_delta_rule(t[0] * 64 ** -0.5, *t[1:], 2, scale=1.0)
+    assert O.rel_l2(o1, o2) < 1e-6
+
+
+def test_determinism_bitwise():
+    inp = make_inputs(13, 2, 200, 4, 64, 64)
+    a = _gpu(inp, torch.bfloat16, 1.0)
+    b = _gpu(inp, torch.bfloat16, 1.0)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    for n in GRADS:
+        assert torch.equal(a[2][n], b[2][n]), n
+
+
+@pytest.mark.parametrize("K,V", [(96, 64), (32, 48), (128, 96)])
+def test_padded_head_dims(K, V):
+    """Head sizes of the reference's stage tests (K = 96, test_fwd_o.py:98-111; V = 96, test_bwd_dhu.py:9-29)."""
+    inp = make_inputs(14, 1, 40, 2, K, V)
+    _compare(_gpu(inp, torch.float32, 1.0), _oracle(inp, torch.float32, 1.0), torch.float32, what=f"K{K} V{V}")
+
+
+def test_rank_one():
+    inp = make_inputs(15, 1, 40, 2, 64, 64, R=1)
+    _compare(_gpu(inp, torch.float32, 1.0, R=1), _oracle(inp, torch.float32, 1.0, R=1), torch.float32)
+
+
+def test_float16_inputs_and_fp32_gk_with_bf16():
+    inp = make_inputs(16, 1, 40, 2, 64, 64)
+    t = [x.half().to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    o, ht = chunk_hrdplr_delta_rule(*t, 2, scale=1.0, output_final_state=True)
+    assert o.dtype == torch.float16
+    o_r, ht_r = O.recurrence(*[x.half() for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)], 1.0, None)
+    assert O.rel_l2(o, o_r) < 2e-3 and O.rel_l2(ht, ht_r) < 1e-5
+    tb = [x.bfloat16().to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b)] + [inp.gk.to(DEV)]   # fp32 gk
+    for x in tb:
+        x.requires_grad_()
+    o, ht = chunk_hrdplr_delta_rule(*tb, 2, scale=1.0, output_final_state=True)
+    (dgk,) = torch.autograd.grad(o.float().sum() + ht.sum(), [tb[5]])
+    assert dgk.dtype == torch.float32
+    ref = [x.bfloat16().double() for x in (inp.q, inp.k, inp.v, inp.a, inp.b)] + [inp.gk.double().requires_grad_()]
+    o_r, ht_r = O.recurrence(*ref, 1.0, None)
+    (dgk_r,) = torch.autograd.grad(o_r.sum() + ht_r.sum(), [ref[5]])
+    assert O.rel_l2(o, o_r) <= 5e-3 and O.rel_l2(dgk, dgk_r) <= 1e-2
+
+
+def test_non_contiguous_inputs_and_non_default_stream():
+    inp = make_inputs(17, 2, 64, 2, 64, 64)
+    t = [x.bfloat16().to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    o, ht = chunk_hrdplr_delta_rule(*t, 2, scale=1.0, output_final_state=True)
+    nc = [x.transpose(1, 2).contiguous().transpose(1, 2) for x in t]         # same values, head-major strides
+    assert not nc[0].is_contiguous()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        o2, ht2 = chunk_hrdplr_delta_rule(*nc, 2, scale=1.0, output_final_state=True)
+    s.synchronize()
+    assert torch.equal(o, o2) and torch.equal(ht, ht2)

@@ -1,0 +1,88 @@
+"""GPU parity of the fused recurrent kernel (decode path) against the CPU oracle and against the chunked path."""
+import pytest
+import torch
+
+from hdla_hip import chunk_hrdplr_delta_rule, fused_recurrent_dplr_delta_rule
+from hdla_hip.synthetic import make_config, make_inputs
+from oracle import hrdplr_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _run(inp, dtype, **kw):
+    t = [x.to(dtype).to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    return fused_recurrent_dplr_delta_rule(*t, 2, **kw)
+
+
+def _ref(inp, dtype, **kw):
+    t = [x.to(dtype) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    return O.recurrence(*t, kw.pop("scale"), kw.pop("initial_state", None), **kw)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 5e-3)])
+@pytest.mark.parametrize("B,T,H,K,V", [(2, 37, 2, 64, 64), (1, 20, 3, 128, 128), (2, 9, 2, 64, 128), (1, 5, 2, 128, 64)])
+def test_parity(dtype, tol, B, T, H, K, V):
+    inp = make_inputs(200 + T, B, T, H, K, V, gk_div=1.0)
+    o, ht = _run(inp, dtype, scale=0.5, initial_state=inp.h0.to(DEV), output_final_state=True)
+    o_r, ht_r = _ref(inp, dtype, scale=0.5, initial_state=inp.h0)
+    assert o.dtype == dtype and ht.dtype == torch.float32
+    assert O.rel_l2(o, o_r) <= tol and O.rel_l2(ht, ht_r) <= min(tol, 1e-5)
+
+
+def test_reverse_varlen_and_no_state():
+    inp = make_inputs(31, 1, 60, 2, 64, 64, n_states=3)
+    cu = torch.tensor([0, 11, 40, 60])
+    o, ht = _run(inp, torch.float32, scale=1.0, initial_state=inp.h0.to(DEV), output_final_state=True, reverse=True,
+                 cu_seqlens=cu.to(DEV))
+    o_r, ht_r = _ref(inp, torch.float32, scale=1.0, initial_state=inp.h0, reverse=True, cu_seqlens=cu)
+    assert O.rel_l2(o, o_r) <= 1e-5 and O.rel_l2(ht, ht_r) <= 1e-5
+    o, ht = _run(inp, torch.float32)                                         # defaults: no state in or out
+    o_r, _ = _ref(inp, torch.float32, scale=64 ** -0.5)
+    assert ht is None and O.rel_l2(o, o_r) <= 1e-5
+
+
+def test_matches_chunked_entry():
+    """The reference's own cross check (test_recurrent.py:66-67): chunk output == recurrent output, final states too."""
+    inp = make_inputs(32, 2, 256, 4, 128, 64, gk_div=1.0)
+    t = [x.float().to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    h0 = inp.h0.to(DEV)
+    o1, h1 = chunk_hrdplr_delta_rule(*t, 2, scale=1.0, initial_state=h0, output_final_state=True, chunk_size=16)
+    o2, h2 = fused_recurrent_dplr_delta_rule(*t, 2, scale=1.0, initial_state=h0, output_final_state=True)
+    assert O.rel_l2(o1, o2) <= 1e-5 and O.rel_l2(h1, h2) <= 1e-5
+
+
+def test_decode_steps_config4_reduced():
+    """Configuration 4's loop at B = 8, H = 4: 16 single-token calls carrying the fp32 state, against one
+    16-token oracle run."""
+    steps = 16
+    inp = make_config(4, shape=(8, steps, 4, 128, 128))
+    t = [x.bfloat16().to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    q, k, v, a, b, gk = t
+    S = inp.h0.to(DEV)
+    outs = []
+    for i in range(steps):
+        o, S = fused_recurrent_dplr_delta_rule(q[:, i:i + 1], k[:, i:i + 1], v[:, i:i + 1], a[:, 2 * i:2 * i + 2],
+                                               b[:, 2 * i:2 * i + 2], gk[:, i:i + 1], 2, scale=1.0, initial_state=S,
+                                               output_final_state=True)
+        outs.append(o)
+    o = torch.cat(outs, 1)
+    o_r, S_r = O.recurrence(*[x.bfloat16() for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)], 1.0, inp.h0)
+    assert O.rel_l2(o, o_r) <= 5e-3 and O.rel_l2(S, S_r) <= 1e-5
+
+
+def test_rank_one_and_padded_dims():
+    inp = make_inputs(33, 2, 12, 2, 96, 48, R=1)
+    t = [x.float().to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    o, ht = fused_recurrent_dplr_delta_rule(*t, 1, scale=1.0, initial_state=inp.h0.to(DEV), output_final_state=True)
+    o_r, ht_r = O.recurrence(inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk, 1.0, inp.h0, rank_ab=1)
+    assert o.shape == (2, 12, 2, 48) and ht.shape == (2, 2, 96, 48)
+    assert O.rel_l2(o, o_r) <= 1e-5 and O.rel_l2(ht, ht_r) <= 1e-5
+
+
+def test_backward_raises():
+    inp = make_inputs(34, 1, 4, 1, 64, 64)
+    t = [x.float().to(DEV).requires_grad_() for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    o, _ = fused_recurrent_dplr_delta_rule(*t, 2, scale=1.0)
+    with pytest.raises(NotImplementedError):
+        o.sum().backward()

@@ -1,0 +1,144 @@
+"""Host side without a GPU: the C-ABI library loads and exports every symbol include/hdla_hip.h declares, its
+argument checks return the documented codes before any launch, and the Python operators raise like the reference's."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import hdla_hip
+from hdla_hip import _lib, chunk_hrdplr_delta_rule, fused_recurrent_dplr_delta_rule
+from hdla_hip.synthetic import make_inputs
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _dims(**kw):
+    d = dict(B=2, T=64, H=2, K=64, V=64, R=2, N=2, in_dtype=torch.bfloat16, gk_dtype=torch.bfloat16, scale=1.0,
+             cu_seqlens=None)
+    d.update(kw)
+    dims = _lib.make_dims(d["B"], d["T"], d["H"], d["K"], d["V"], d["R"], d["N"], d["in_dtype"], d["gk_dtype"],
+                          d["scale"], None)
+    if d["cu_seqlens"] is not None:
+        dims.cu_seqlens = d["cu_seqlens"]
+    return dims
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    header = open(os.path.join(ROOT, "include", "hdla_hip.h")).read()
+    names = set(re.findall(r"\b(hdla_[a-z_]+)\s*\(", header))
+    assert {"hdla_version", "hdla_strerror", "hdla_workspace_bytes", "hdla_workspace_layout", "hdla_chunk_fwd",
+            "hdla_chunk_bwd", "hdla_chunk_stages", "hdla_recurrent_fwd"} <= names
+    for n in names:
+        assert hasattr(lib, n), n
+    assert lib.hdla_version() == 100
+    assert lib.hdla_strerror(0) == b"success"
+
+
+def test_workspace_size_and_layout():
+    lib = _lib.load()
+    d = _dims()
+    fwd, bwd = lib.hdla_workspace_bytes(ctypes.byref(d), 0), lib.hdla_workspace_bytes(ctypes.byref(d), 1)
+    assert 0 < fwd < bwd
+    L = _lib.workspace_layout(d, 1)
+    assert L["nch"] == 2 * 4 and L["total"] == bwd
+    offs = [L[k] for k in ("W", "UT", "KGT", "BGT", "VTT", "EGL", "AQBT", "BG", "WT", "QGT", "TM", "HC", "DHC", "VN", "DVN")]
+    assert offs == sorted(offs) and all(o % 256 == 0 for o in offs)
+    # ragged T and packed sequences reserve one extra chunk per sequence
+    assert _lib.workspace_layout(_dims(T=65), 0)["nch"] == 2 * 5
+    assert _lib.workspace_layout(_dims(B=1, N=3, T=64, cu_seqlens=256), 0)["nch"] == 4 + 3
+    assert lib.hdla_workspace_bytes(ctypes.byref(d), 2) == 0
+
+
+@pytest.mark.parametrize("kw,code", [
+    (dict(K=96), -2), (dict(V=32), -2), (dict(R=1), -3), (dict(R=3), -3), (dict(H=0), -2), (dict(T=-1), -2),
+    (dict(in_dtype=torch.float32, gk_dtype=torch.bfloat16), -4), (dict(N=3), -7), (dict(B=2, cu_seqlens=256), -7),
+])
+def test_bad_dims_are_rejected_before_launch(kw, code):
+    lib = _lib.load()
+    d = _dims(**kw)
+    assert lib.hdla_workspace_bytes(ctypes.byref(d), 0) == 0
+    one = ctypes.c_void_p(256)
+    rc = lib.hdla_chunk_fwd(ctypes.byref(d), one, one, one, one, one, one, None, one, None, one, 1 << 40, None)
+    assert rc == code
+    assert lib.hdla_recurrent_fwd(ctypes.byref(d), one, one, one, one, one, one, 0, None, one, None, None) == code
+    assert len(lib.hdla_strerror(rc)) > 8
+
+
+def test_null_misaligned_and_small_workspace():
+    lib = _lib.load()
+    d = _dims()
+    ok = ctypes.c_void_p(4096)
+    assert lib.hdla_chunk_fwd(ctypes.byref(d), None, ok, ok, ok, ok, ok, None, ok, None, ok, 1 << 40, None) == -1
+    bad = ctypes.c_void_p(4096 + 8)
+    assert lib.hdla_chunk_fwd(ctypes.byref(d), bad, ok, ok, ok, ok, ok, None, ok, None, ok, 1 << 40, None) == -6
+    assert lib.hdla_chunk_fwd(ctypes.byref(d), ok, ok, ok, ok, ok, ok, None, ok, None, ok, 1024, None) == -5
+    assert lib.hdla_chunk_fwd(ctypes.byref(d), ok, ok, ok, ok, ok, ok, None, ok, None, None, 1 << 40, None) == -5
+    assert lib.hdla_chunk_fwd(ctypes.byref(d), ok, ok, ok, ok, ok, ok, None, ok, None, ctypes.c_void_p(4096 + 16), 1 << 40, None) == -5
+    assert lib.hdla_chunk_bwd(ctypes.byref(d), ok, ok, ok, ok, ok, ok, None, None, None, ok, ok, ok, ok, ok, ok, None,
+                              ok, 1 << 40, None) == -1
+    assert lib.hdla_workspace_layout(ctypes.byref(d), 0, None) == -1
+
+
+def _cpu_args(T=32, K=64, V=64, R=2, B=2):
+    x = make_inputs(3, B, T, 2, K, V, R=R)
+    return [t.bfloat16() for t in (x.q, x.k, x.v, x.a, x.b, x.gk)], x
+
+
+def test_python_entry_points_validate_like_the_reference():
+    (q, k, v, a, b, gk), x = _cpu_args()
+    with pytest.raises(AssertionError):
+        chunk_hrdplr_delta_rule(q, k, v, a, b, gk, 2, head_first=True)
+    with pytest.raises(AssertionError):
+        chunk_hrdplr_delta_rule(q, k.float(), v, a, b, gk, 2)
+    with pytest.raises(ValueError):
+        chunk_hrdplr_delta_rule(q, k, v, a[:, :-1], b, gk, 2)
+    with pytest.raises(ValueError, match="batch size is expected to be 1"):
+        chunk_hrdplr_delta_rule(q, k, v, a, b, gk, 2, cu_seqlens=torch.tensor([0, 16, 32]))
+    with pytest.raises(ValueError, match="number of initial states"):
+        chunk_hrdplr_delta_rule(q[:1], k[:1], v[:1], a[:1], b[:1], gk[:1], 2, initial_state=x.h0,
+                                cu_seqlens=torch.tensor([0, 8, 16, 32]))
+    with pytest.raises(AssertionError):
+        fused_recurrent_dplr_delta_rule(q, k, v, a, b, gk, 2, head_first=True)
+    with pytest.raises(ValueError, match="batch size is expected to be 1"):
+        fused_recurrent_dplr_delta_rule(q, k, v, a, b, gk, 2, cu_seqlens=torch.tensor([0, 16, 32]))
+    with pytest.raises(ValueError, match="a must have 4 dimensions"):
+        fused_recurrent_dplr_delta_rule(q, k, v, a[0], b, gk, 2)
+    with pytest.raises(AssertionError, match="must be divisible"):
+        fused_recurrent_dplr_delta_rule(q, k, v, a[:, :-1], b[:, :-1], gk, 2)
+    with pytest.raises(NotImplementedError):
+        chunk_hrdplr_delta_rule(q, k, v, torch.cat([a, a[:, :32]], 1), torch.cat([b, b[:, :32]], 1), gk, 3)
+
+
+def test_no_cpu_fallback():
+    (q, k, v, a, b, gk), _ = _cpu_args()
+    with pytest.raises(_lib.HdlaError, match="GPU only"):
+        chunk_hrdplr_delta_rule(q, k, v, a, b, gk, 2)
+    with pytest.raises(_lib.HdlaError, match="GPU only"):
+        fused_recurrent_dplr_delta_rule(q, k, v, a, b, gk, 2)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setenv("HDLA_HIP_LIB", "/nonexistent/libhdla_hip.so")
+    with pytest.raises(_lib.HdlaError, match="no CPU or PyTorch fallback"):
+        _lib.load()
+
+
+def test_product_code_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "hdla-impl_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cuh")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.replace("no CPU or PyTorch fallback", ""), os.path.join(dirpath, f)
+
+
+def test_recurrent_backward_is_not_implemented():
+    class Ctx:
+        _fwd_used_autocast = False
+        _dtype = torch.float32
+    with pytest.raises(NotImplementedError, match="only for inference"):
+        hdla_hip.FusedRecurrentDPLRDeltaRuleFunction.backward(Ctx(), None, None)
