@@ -8,6 +8,11 @@
 
 using namespace hdla;
 
+#ifdef HDLA_PHASE_TIMING
+static long long* g_phase_clk = nullptr;
+extern "C" void hdla_debug_set_phase_buffer(long long* p) { g_phase_clk = p; }
+#endif
+
 namespace {
 
 constexpr int CHUNK = 16;
@@ -110,6 +115,9 @@ int run_chunk(const hdla_dims* d, int pass, const void* q, const void* k, const 
     a.dq = static_cast<T*>(dq); a.dk = static_cast<T*>(dk); a.dv = static_cast<T*>(dv);
     a.da = static_cast<T*>(da); a.db = static_cast<T*>(db); a.dgk = dgk;
     bind_ws(a, d, L, nch, workspace);
+#ifdef HDLA_PHASE_TIMING
+    a.phase_clk = g_phase_clk;
+#endif
     hipError_t e;
     if (d->cu_seqlens && (stages & HDLA_STAGE_PREP)) {
         char* base = static_cast<char*>(workspace);

@@ -19,7 +19,7 @@ namespace hdla {
 
 constexpr int LDG = 36;
 
-template <typename T, int K, int V>
+template <typename T, bool GKF32, int K, int V>
 __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     constexpr int KT = K / 16, VT = V / 16;
     __shared__ __attribute__((aligned(16))) float sT[32 * LDG];   // (I - A_ab)^-1, rank-major
@@ -30,7 +30,7 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     const int l = lane_id(), g = l >> 4, c = l & 15;
     const int H = p.H;
     const bool rowok = c < cp.len;
-    const int64_t tok = cp.tok0 + c;
+    const int64_t tok = cp.tok0 + min(c, cp.len - 1);   // rows past the end alias the last valid row, masked by rowok
     const int64_t qoff = (tok * H + h) * K + 4 * g;
     const int64_t aoff0 = ((tok * RANK + 0) * H + h) * K + 4 * g;
     const int64_t aoff1 = ((tok * RANK + 1) * H + h) * K + 4 * g;
@@ -41,6 +41,8 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     const T* DHC = p.ws.DHC + chw * (K * V);
     const T* VN = p.ws.VN + chw * (2 * CH * V);
     const T* DVN = p.ws.DVN + chw * (2 * CH * V);
+    const int blk = blockIdx.y * gridDim.x + blockIdx.x;
+    PHASE_CLOCK(p, blk, 0);
 
     {
         const float* tmw = p.ws.TM + chw * 1024;
@@ -68,15 +70,15 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     f32x4 aqkT = zero4(), aakT[2] = {zero4(), zero4()};
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
-        const f32x4 g4 = ld_gk4(p.gk, qoff + 16 * kt, p.gk_f32, rowok);
+        const f32x4 g4 = ld_gk4<GKF32>(p.gk, qoff + 16 * kt, rowok);
         gi[kt] = scan16_incl(g4);
         ge[kt] = gi[kt] - g4;
         const f32x4 m = bcast16(gi[kt], MID);
         const f32x4 eq = exp4<T>(gi[kt] - m), ek = exp4<T>(m - gi[kt]), ea = exp4<T>(ge[kt] - m);
-        const f32x4 q4 = to_f32(ld_frag_if(p.q + qoff + 16 * kt, rowok));
-        const f32x4 k4 = to_f32(ld_frag_if(p.k + qoff + 16 * kt, rowok));
-        const f32x4 a0 = to_f32(ld_frag_if(p.a + aoff0 + 16 * kt, rowok));
-        const f32x4 a1 = to_f32(ld_frag_if(p.a + aoff1 + 16 * kt, rowok));
+        const f32x4 q4 = to_f32(ld_frag_sel(p.q + qoff + 16 * kt, rowok));
+        const f32x4 k4 = to_f32(ld_frag_sel(p.k + qoff + 16 * kt, rowok));
+        const f32x4 a0 = to_f32(ld_frag_sel(p.a + aoff0 + 16 * kt, rowok));
+        const f32x4 a1 = to_f32(ld_frag_sel(p.a + aoff1 + 16 * kt, rowok));
         const Frag<T> qh = to_frag<T>(q4 * eq * scale), kh = to_frag<T>(k4 * ek);
         aqkT = mm(kh, qh, aqkT);
         aakT[0] = mm(kh, to_frag<T>(a0 * ea), aakT[0]);
@@ -91,14 +93,15 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     const Frag<T> aqkTf = to_frag<T>(aqkT);
     const Frag<T> aakTf[2] = {to_frag<T>(aakT[0]), to_frag<T>(aakT[1])};
 
+    PHASE_CLOCK(p, blk, 1);
     // ---- products over the value dimension -------------------------------------------------------------------
     f32x4 dAqk = zero4(), dAqb[2] = {zero4(), zero4()}, dAak[2] = {zero4(), zero4()};
     f32x4 dAab[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
     f32x4 dv[VT];
 #pragma unroll
     for (int vt = 0; vt < VT; ++vt) {
-        const Frag<T> doN = ld_frag_if(p.dout + voff + 16 * vt, rowok);
-        const Frag<T> vN = ld_frag_if(p.v + voff + 16 * vt, rowok);
+        const Frag<T> doN = ld_frag_sel(p.dout + voff + 16 * vt, rowok);
+        const Frag<T> vN = ld_frag_sel(p.v + voff + 16 * vt, rowok);
         const Frag<T> vnN[2] = {ld_frag(VN + (0 * CH + c) * V + 16 * vt + 4 * g), ld_frag(VN + (1 * CH + c) * V + 16 * vt + 4 * g)};
         const Frag<T> dvnN[2] = {ld_frag(DVN + (0 * CH + c) * V + 16 * vt + 4 * g), ld_frag(DVN + (1 * CH + c) * V + 16 * vt + 4 * g)};
         dAqk = mm(doN, vN, dAqk);
@@ -116,8 +119,8 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
             y = mm(dvnT[1], tmT[1][r], y);
             dMTf[r] = to_frag<T>(y);                      // dM_r^T rows value, inner i
         }
-        const Frag<T> uN[2] = {transpose(ld_tile(p.ws.UT + ((chw * 2 + 0) * VT + vt) * TILE), ident),
-                               transpose(ld_tile(p.ws.UT + ((chw * 2 + 1) * VT + vt) * TILE), ident)};
+        const Frag<T> uN[2] = {transpose(ld_pair_one(p.ws.UT + (chw * VT + vt) * PAIR, 0), ident),
+                               transpose(ld_pair_one(p.ws.UT + (chw * VT + vt) * PAIR, 1), ident)};
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
             dAak[r] = mm(dMf[r], vN, dAak[r]);
@@ -130,6 +133,7 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         dv[vt] = x;                                       // rows token, inner value; kg dS is added below
     }
 
+    PHASE_CLOCK(p, blk, 2);
     // ---- first pass over channel tiles: dw -> dag, and the w part of dA_ab ------------------------------------
     f32x4 dag[2][KT];
 #pragma unroll
@@ -148,11 +152,12 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
             x = mm(tmT[1][r], dwTf[1], x);
             dag[r][kt] = x;                               // rows token, inner channel
             const Frag<T> dagf = to_frag<T>(x);
-            dAab[r][0] = mm(dagf, ld_tile(p.ws.W + ((chw * 2 + 0) * KT + kt) * TILE), dAab[r][0]);
-            dAab[r][1] = mm(dagf, ld_tile(p.ws.W + ((chw * 2 + 1) * KT + kt) * TILE), dAab[r][1]);
+            dAab[r][0] = mm(dagf, ld_pair_one(p.ws.W + ((chw * 2 + 0) * (KT / 2) + kt / 2) * PAIR, kt & 1), dAab[r][0]);
+            dAab[r][1] = mm(dagf, ld_pair_one(p.ws.W + ((chw * 2 + 1) * (KT / 2) + kt / 2) * PAIR, kt & 1), dAab[r][1]);
         }
     }
 
+    PHASE_CLOCK(p, blk, 3);
     // ---- masks; both orientations of the nine score-gradient tiles --------------------------------------------
 #pragma unroll
     for (int i = 0; i < 4; ++i) {          // row i = c, inner j = 4g+i
@@ -170,16 +175,17 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         for (int r = 0; r < 2; ++r) { fAab[r][s] = to_frag<T>(dAab[r][s]); fAabT[r][s] = transpose(fAab[r][s], ident); }
     }
 
+    PHASE_CLOCK(p, blk, 4);
     // ---- second pass over channel tiles: state products, score backward, final gradients ----------------------
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
         const f32x4 m = bcast16(gi[kt], MID), gl = bcast16(gi[kt], CH - 1);
         const f32x4 eq = exp4<T>(gi[kt] - m), ek = exp4<T>(m - gi[kt]), ea = exp4<T>(ge[kt] - m);
         const f32x4 egi = exp4<T>(gi[kt]), ege = exp4<T>(ge[kt]), edn = exp4<T>(gl - gi[kt]);
-        const f32x4 q4 = to_f32(ld_frag_if(p.q + qoff + 16 * kt, rowok));
-        const f32x4 k4 = to_f32(ld_frag_if(p.k + qoff + 16 * kt, rowok));
-        const f32x4 a4[2] = {to_f32(ld_frag_if(p.a + aoff0 + 16 * kt, rowok)), to_f32(ld_frag_if(p.a + aoff1 + 16 * kt, rowok))};
-        const f32x4 b4[2] = {to_f32(ld_frag_if(p.b + aoff0 + 16 * kt, rowok)), to_f32(ld_frag_if(p.b + aoff1 + 16 * kt, rowok))};
+        const f32x4 q4 = to_f32(ld_frag_sel(p.q + qoff + 16 * kt, rowok));
+        const f32x4 k4 = to_f32(ld_frag_sel(p.k + qoff + 16 * kt, rowok));
+        const f32x4 a4[2] = {to_f32(ld_frag_sel(p.a + aoff0 + 16 * kt, rowok)), to_f32(ld_frag_sel(p.a + aoff1 + 16 * kt, rowok))};
+        const f32x4 b4[2] = {to_f32(ld_frag_sel(p.b + aoff0 + 16 * kt, rowok)), to_f32(ld_frag_sel(p.b + aoff1 + 16 * kt, rowok))};
         const Frag<T> qhT = transpose(to_frag<T>(q4 * eq * scale), ident), khT = transpose(to_frag<T>(k4 * ek), ident);
         const Frag<T> ahT[2] = {transpose(to_frag<T>(a4[0] * ea), ident), transpose(to_frag<T>(a4[1] * ea), ident)};
         const Frag<T> bhT[2] = {transpose(to_frag<T>(b4[0] * ek), ident), transpose(to_frag<T>(b4[1] * ek), ident)};
@@ -193,8 +199,8 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         for (int vt = 0; vt < VT; ++vt) {
             const Frag<T> Sf = ld_frag(HC + (16 * kt + c) * V + 16 * vt + 4 * g);
             const Frag<T> dSf = ld_frag(DHC + (16 * kt + c) * V + 16 * vt + 4 * g);
-            const Frag<T> doN = ld_frag_if(p.dout + voff + 16 * vt, rowok);
-            const Frag<T> vN = ld_frag_if(p.v + voff + 16 * vt, rowok);
+            const Frag<T> doN = ld_frag_sel(p.dout + voff + 16 * vt, rowok);
+            const Frag<T> vN = ld_frag_sel(p.v + voff + 16 * vt, rowok);
             dqg = mm(doN, Sf, dqg);
             dkg = mm(vN, dSf, dkg);
             dbg[0] = mm(ld_frag(VN + (0 * CH + c) * V + 16 * vt + 4 * g), dSf, dbg[0]);
@@ -242,19 +248,22 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
             st_frag(p.da + aoff1 + 16 * kt, to_frag<T>(da[1]));
             st_frag(p.db + aoff0 + 16 * kt, to_frag<T>(db[0]));
             st_frag(p.db + aoff1 + 16 * kt, to_frag<T>(db[1]));
-            st_gk4(p.dgk, qoff + 16 * kt, p.gk_f32, dg);
+            st_gk4<GKF32>(p.dgk, qoff + 16 * kt, dg);
         }
     }
     if (rowok) {
 #pragma unroll
         for (int vt = 0; vt < VT; ++vt) st_frag(p.dv + voff + 16 * vt, to_frag<T>(dv[vt]));
     }
+    PHASE_CLOCK(p, blk, 5);
 }
 
 template <typename T, int K, int V>
 static hipError_t launch_chunk_grad_kv(const ChunkArgs<T>& a, hipStream_t stream) {
     dim3 grid(a.st.nch, a.H), block(64);
-    hipLaunchKernelGGL((chunk_grad_kernel<T, K, V>), grid, block, 0, stream, a);
+    constexpr bool kAlwaysF32 = sizeof(T) == 4;
+    if (kAlwaysF32 || a.gk_f32) hipLaunchKernelGGL((chunk_grad_kernel<T, true, K, V>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((chunk_grad_kernel<T, kAlwaysF32, K, V>), grid, block, 0, stream, a);
     return hipGetLastError();
 }
 

@@ -23,6 +23,14 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
+// Developer profiling: with -DHDLA_PHASE_TIMING the first 64 workgroups of a kernel record the shader clock at
+// marked points into ChunkArgs::phase_clk[block][16]; in normal builds the macro expands to nothing.
+#ifdef HDLA_PHASE_TIMING
+#define PHASE_CLOCK(p, blk, i) do { if ((p).phase_clk && (blk) < 64 && lane_id() == 0) (p).phase_clk[(blk) * 16 + (i)] = clock64(); } while (0)
+#else
+#define PHASE_CLOCK(p, blk, i) do { } while (0)
+#endif
+
 constexpr int CH = 16;       // tokens per chunk
 constexpr int MID = 7;       // token whose cumulative log-decay centres the factorised scores
 constexpr int RANK = 2;      // rank of the a/b update
@@ -90,8 +98,15 @@ __device__ __forceinline__ void st_frag(bf16* p, Frag<bf16> f) { *reinterpret_ca
 __device__ __forceinline__ void st_frag(float* p, Frag<float> f) { *reinterpret_cast<f32x4*>(p) = f.v; }
 template <typename T> __device__ __forceinline__ Frag<T> zero_frag() { return to_frag<T>(zero4()); }
 
-template <typename T> __device__ __forceinline__ Frag<T> ld_frag_if(const T* p, bool ok) {
-    return ok ? ld_frag(p) : zero_frag<T>();
+// Masked load without a branch: p must be a readable address on every lane (callers clamp the row index);
+// lanes with ok == false get zeros by a select after the load.  A branch around the load would stop the
+// compiler from batching the loads of an unrolled loop, so every load would pay its own memory latency.
+template <typename T> __device__ __forceinline__ Frag<T> ld_frag_sel(const T* p, bool ok) {
+    Frag<T> f = ld_frag(p);
+    Frag<T> z = zero_frag<T>();
+    Frag<T> r;
+    r.v = ok ? f.v : z.v;
+    return r;
 }
 
 // one element stores (used for the strided, 4-rows-per-lane writes of row-major checkpoints)
@@ -104,14 +119,37 @@ __device__ __forceinline__ float ld_elem(const float* p) { return *p; }
 template <typename T> __device__ __forceinline__ Frag<T> ld_tile(const T* tile) { return ld_frag(tile + 4 * lane_id()); }
 template <typename T> __device__ __forceinline__ void st_tile(T* tile, Frag<T> f) { st_frag(tile + 4 * lane_id(), f); }
 
-// gk may be stored as bf16 or fp32 independently of the other inputs
-__device__ __forceinline__ f32x4 ld_gk4(const void* base, int64_t elem_off, int is_f32, bool ok) {
-    if (!ok) return zero4();
-    if (is_f32) return *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(base) + elem_off);
-    return to_f32(ld_frag(reinterpret_cast<const bf16*>(base) + elem_off));
+// Two tiles that one consumer lane always needs together are stored interleaved as a pair (1024 bytes for bf16):
+// element 8*lane + 4*which + i, so that both fragments arrive with one 16-byte load per lane.  The scans are
+// limited by the number of memory instructions a wave may have in flight, not by bytes.
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+constexpr int PAIR = 2 * TILE;
+__device__ __forceinline__ void ld_pair(const bf16* pair, Frag<bf16>& f0, Frag<bf16>& f1) {
+    const s16x8 x = *reinterpret_cast<const s16x8*>(pair + 8 * lane_id());
+    f0.v = __builtin_shufflevector(x, x, 0, 1, 2, 3);
+    f1.v = __builtin_shufflevector(x, x, 4, 5, 6, 7);
 }
-__device__ __forceinline__ void st_gk4(void* base, int64_t elem_off, int is_f32, f32x4 x) {
-    if (is_f32) *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(base) + elem_off) = x;
+__device__ __forceinline__ void ld_pair(const float* pair, Frag<float>& f0, Frag<float>& f1) {
+    f0.v = *reinterpret_cast<const f32x4*>(pair + 8 * lane_id());
+    f1.v = *reinterpret_cast<const f32x4*>(pair + 8 * lane_id() + 4);
+}
+template <typename T> __device__ __forceinline__ Frag<T> ld_pair_one(const T* pair, int which) {
+    return ld_frag(pair + 8 * lane_id() + 4 * which);
+}
+template <typename T> __device__ __forceinline__ void st_pair(T* pair, int which, Frag<T> f) {
+    st_frag(pair + 8 * lane_id() + 4 * which, f);
+}
+
+// gk may be stored as bf16 or fp32 independently of the other inputs (compile-time switch GKF32);
+// same contract as ld_frag_sel: the address is readable on every lane, masked lanes read zero.
+template <bool GKF32> __device__ __forceinline__ f32x4 ld_gk4(const void* base, int64_t elem_off, bool ok) {
+    f32x4 x;
+    if (GKF32) x = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(base) + elem_off);
+    else x = to_f32(ld_frag(reinterpret_cast<const bf16*>(base) + elem_off));
+    return ok ? x : zero4();
+}
+template <bool GKF32> __device__ __forceinline__ void st_gk4(void* base, int64_t elem_off, f32x4 x) {
+    if (GKF32) *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(base) + elem_off) = x;
     else st_frag(reinterpret_cast<bf16*>(base) + elem_off, to_frag<bf16>(x));
 }
 
@@ -152,6 +190,12 @@ __device__ __forceinline__ bool locate_chunk(const SeqTab& st, int cid, ChunkPos
 __device__ __forceinline__ void seq_chunks(const SeqTab& st, int n, int& c0, int& c1) {
     if (st.cu == nullptr) { c0 = n * st.NT; c1 = c0 + st.NT; }
     else { c0 = st.chunk_off[n]; c1 = st.chunk_off[n + 1]; }
+}
+
+// token rows [bos, eos) of sequence n on the flattened axis
+__device__ __forceinline__ void seq_bounds(const SeqTab& st, int n, int64_t& bos, int64_t& eos) {
+    if (st.cu == nullptr) { bos = (int64_t)n * st.T; eos = bos + st.T; }
+    else { bos = st.cu[n]; eos = st.cu[n + 1]; }
 }
 
 // ---- per-chunk decay quantities in fragment layout ---------------------------------------------------------

@@ -12,9 +12,9 @@ namespace hdla {
 
 constexpr int LDP = 36;   // padded row length of the 32x32 LDS matrices (keeps 16-byte row alignment)
 
-template <typename T, int K, int V, bool BWD>
+template <typename T, bool GKF32, int K, int V, bool BWD>
 __global__ __launch_bounds__(64) void prep_kernel(ChunkArgs<T> p) {
-    constexpr int KT = K / 16, VT = V / 16;
+    constexpr int KT = K / 16, VT = V / 16, KT2 = KT / 2;
     __shared__ __attribute__((aligned(16))) float sN[32 * LDP];   // A_ab, rank-major
     __shared__ __attribute__((aligned(16))) float sT[32 * LDP];   // (I - A_ab)^-1
 
@@ -24,13 +24,15 @@ __global__ __launch_bounds__(64) void prep_kernel(ChunkArgs<T> p) {
     const int l = lane_id(), g = l >> 4, c = l & 15;
     const int H = p.H;
     const bool rowok = c < cp.len;
-    const int64_t tok = cp.tok0 + c;
+    const int64_t tok = cp.tok0 + min(c, cp.len - 1);   // rows past the end alias the last valid row, masked by rowok
     const int64_t qoff = (tok * H + h) * K + 4 * g;                 // + 16*kt
     const int64_t aoff0 = ((tok * RANK + 0) * H + h) * K + 4 * g;
     const int64_t aoff1 = ((tok * RANK + 1) * H + h) * K + 4 * g;
     const int64_t voff = (tok * H + h) * V + 4 * g;
     const int64_t chw = (int64_t)h * p.st.nch + cid;                // chunk-head slot in the workspace
     const float scale = p.scale;
+    const int blk = blockIdx.y * gridDim.x + blockIdx.x;
+    PHASE_CLOCK(p, blk, 0);
 
     // ---- phase A: cumulative decays and the score tiles (rows i, inner j) -----------------------------------
     f32x4 gi[KT], ge[KT];
@@ -39,17 +41,17 @@ __global__ __launch_bounds__(64) void prep_kernel(ChunkArgs<T> p) {
     f32x4 aqbT[2] = {zero4(), zero4()};
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
-        const f32x4 g4 = ld_gk4(p.gk, qoff + 16 * kt, p.gk_f32, rowok);
+        const f32x4 g4 = ld_gk4<GKF32>(p.gk, qoff + 16 * kt, rowok);
         gi[kt] = scan16_incl(g4);
         ge[kt] = gi[kt] - g4;
         const f32x4 m = bcast16(gi[kt], MID);
         const f32x4 eq = exp4<T>(gi[kt] - m), ek = exp4<T>(m - gi[kt]), ea = exp4<T>(ge[kt] - m);
-        const f32x4 q4 = to_f32(ld_frag_if(p.q + qoff + 16 * kt, rowok));
-        const f32x4 k4 = to_f32(ld_frag_if(p.k + qoff + 16 * kt, rowok));
-        const f32x4 a0 = to_f32(ld_frag_if(p.a + aoff0 + 16 * kt, rowok));
-        const f32x4 a1 = to_f32(ld_frag_if(p.a + aoff1 + 16 * kt, rowok));
-        const f32x4 b0 = to_f32(ld_frag_if(p.b + aoff0 + 16 * kt, rowok));
-        const f32x4 b1 = to_f32(ld_frag_if(p.b + aoff1 + 16 * kt, rowok));
+        const f32x4 q4 = to_f32(ld_frag_sel(p.q + qoff + 16 * kt, rowok));
+        const f32x4 k4 = to_f32(ld_frag_sel(p.k + qoff + 16 * kt, rowok));
+        const f32x4 a0 = to_f32(ld_frag_sel(p.a + aoff0 + 16 * kt, rowok));
+        const f32x4 a1 = to_f32(ld_frag_sel(p.a + aoff1 + 16 * kt, rowok));
+        const f32x4 b0 = to_f32(ld_frag_sel(p.b + aoff0 + 16 * kt, rowok));
+        const f32x4 b1 = to_f32(ld_frag_sel(p.b + aoff1 + 16 * kt, rowok));
         const Frag<T> qh = to_frag<T>(q4 * eq * scale), kh = to_frag<T>(k4 * ek);
         const Frag<T> ah[2] = {to_frag<T>(a0 * ea), to_frag<T>(a1 * ea)};
         const Frag<T> bh[2] = {to_frag<T>(b0 * ek), to_frag<T>(b1 * ek)};
@@ -74,11 +76,11 @@ __global__ __launch_bounds__(64) void prep_kernel(ChunkArgs<T> p) {
     }
     if (!BWD) {
         st_tile(p.ws.AQK + chw * TILE, to_frag<T>(aqk));
-        st_tile(p.ws.AQB + (chw * 2 + 0) * TILE, to_frag<T>(aqb[0]));
-        st_tile(p.ws.AQB + (chw * 2 + 1) * TILE, to_frag<T>(aqb[1]));
+        st_pair(p.ws.AQB + chw * PAIR, 0, to_frag<T>(aqb[0]));
+        st_pair(p.ws.AQB + chw * PAIR, 1, to_frag<T>(aqb[1]));
     } else {
-        st_tile(p.ws.AQBT + (chw * 2 + 0) * TILE, to_frag<T>(aqbT[0]));
-        st_tile(p.ws.AQBT + (chw * 2 + 1) * TILE, to_frag<T>(aqbT[1]));
+        st_pair(p.ws.AQBT + chw * PAIR, 0, to_frag<T>(aqbT[0]));
+        st_pair(p.ws.AQBT + chw * PAIR, 1, to_frag<T>(aqbT[1]));
     }
 #pragma unroll
     for (int r = 0; r < 2; ++r)
@@ -86,6 +88,7 @@ __global__ __launch_bounds__(64) void prep_kernel(ChunkArgs<T> p) {
         for (int s = 0; s < 2; ++s)
             *reinterpret_cast<f32x4*>(&sN[(16 * r + c) * LDP + 16 * s + 4 * g]) = aab[r][s];
     __syncthreads();
+    PHASE_CLOCK(p, blk, 1);
 
     // ---- phase B: (I - A_ab)^-1 by forward substitution over tokens, two rank rows x 32 columns per step ----
     {
@@ -101,6 +104,7 @@ __global__ __launch_bounds__(64) void prep_kernel(ChunkArgs<T> p) {
             __syncthreads();
         }
     }
+    PHASE_CLOCK(p, blk, 2);
     Frag<T> tm[2][2];   // F(Tm^{s s'}): rows i, inner j
 #pragma unroll
     for (int s = 0; s < 2; ++s)
@@ -122,47 +126,48 @@ __global__ __launch_bounds__(64) void prep_kernel(ChunkArgs<T> p) {
     for (int kt = 0; kt < KT; ++kt) {
         const f32x4 gl = bcast16(gi[kt], CH - 1);
         const f32x4 egi = exp4<T>(gi[kt]), ege = exp4<T>(ge[kt]), edn = exp4<T>(gl - gi[kt]);
-        const f32x4 q4 = to_f32(ld_frag_if(p.q + qoff + 16 * kt, rowok));
-        const f32x4 k4 = to_f32(ld_frag_if(p.k + qoff + 16 * kt, rowok));
-        const f32x4 a0 = to_f32(ld_frag_if(p.a + aoff0 + 16 * kt, rowok));
-        const f32x4 a1 = to_f32(ld_frag_if(p.a + aoff1 + 16 * kt, rowok));
-        const f32x4 b0 = to_f32(ld_frag_if(p.b + aoff0 + 16 * kt, rowok));
-        const f32x4 b1 = to_f32(ld_frag_if(p.b + aoff1 + 16 * kt, rowok));
+        const f32x4 q4 = to_f32(ld_frag_sel(p.q + qoff + 16 * kt, rowok));
+        const f32x4 k4 = to_f32(ld_frag_sel(p.k + qoff + 16 * kt, rowok));
+        const f32x4 a0 = to_f32(ld_frag_sel(p.a + aoff0 + 16 * kt, rowok));
+        const f32x4 a1 = to_f32(ld_frag_sel(p.a + aoff1 + 16 * kt, rowok));
+        const f32x4 b0 = to_f32(ld_frag_sel(p.b + aoff0 + 16 * kt, rowok));
+        const f32x4 b1 = to_f32(ld_frag_sel(p.b + aoff1 + 16 * kt, rowok));
         const Frag<T> agT[2] = {transpose(to_frag<T>(a0 * ege), ident), transpose(to_frag<T>(a1 * ege), ident)};
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
             f32x4 w = zero4();
             w = mm(tm[s][0], agT[0], w);
             w = mm(tm[s][1], agT[1], w);
-            st_tile(p.ws.W + ((chw * 2 + s) * KT + kt) * TILE, to_frag<T>(w));
+            st_pair(p.ws.W + ((chw * 2 + s) * KT2 + kt / 2) * PAIR, kt & 1, to_frag<T>(w));
             if (BWD) {
                 f32x4 wT = zero4();
                 wT = mm(agT[0], tm[s][0], wT);
                 wT = mm(agT[1], tm[s][1], wT);
-                st_tile(p.ws.WT + ((chw * 2 + s) * KT + kt) * TILE, to_frag<T>(wT));
+                st_pair(p.ws.WT + ((chw * 2 + s) * KT2 + kt / 2) * PAIR, kt & 1, to_frag<T>(wT));
             }
         }
         const Frag<T> qg = to_frag<T>(q4 * egi * scale);
         const Frag<T> kg = to_frag<T>(k4 * edn);
         const Frag<T> bg[2] = {to_frag<T>(b0 * edn), to_frag<T>(b1 * edn)};
-        st_tile(p.ws.KGT + (chw * KT + kt) * TILE, transpose(kg, ident));
-        st_tile(p.ws.BGT + ((chw * 2 + 0) * KT + kt) * TILE, transpose(bg[0], ident));
-        st_tile(p.ws.BGT + ((chw * 2 + 1) * KT + kt) * TILE, transpose(bg[1], ident));
+        st_pair(p.ws.KGT + (chw * KT2 + kt / 2) * PAIR, kt & 1, transpose(kg, ident));
+        st_pair(p.ws.BGT + ((chw * 2 + 0) * KT2 + kt / 2) * PAIR, kt & 1, transpose(bg[0], ident));
+        st_pair(p.ws.BGT + ((chw * 2 + 1) * KT2 + kt / 2) * PAIR, kt & 1, transpose(bg[1], ident));
         if (!BWD) {
-            st_tile(p.ws.QG + (chw * KT + kt) * TILE, qg);
+            st_pair(p.ws.QG + (chw * KT2 + kt / 2) * PAIR, kt & 1, qg);
         } else {
-            st_tile(p.ws.QGT + (chw * KT + kt) * TILE, transpose(qg, ident));
-            st_tile(p.ws.BG + ((chw * 2 + 0) * KT + kt) * TILE, bg[0]);
-            st_tile(p.ws.BG + ((chw * 2 + 1) * KT + kt) * TILE, bg[1]);
+            st_pair(p.ws.QGT + (chw * KT2 + kt / 2) * PAIR, kt & 1, transpose(qg, ident));
+            st_pair(p.ws.BG + ((chw * 2 + 0) * KT2 + kt / 2) * PAIR, kt & 1, bg[0]);
+            st_pair(p.ws.BG + ((chw * 2 + 1) * KT2 + kt / 2) * PAIR, kt & 1, bg[1]);
         }
         if (c == 0) *reinterpret_cast<f32x4*>(p.ws.EGL + chw * K + 16 * kt + 4 * g) = exp4<T>(gl);
     }
 
+    PHASE_CLOCK(p, blk, 3);
     // ---- phase D: u = Tm (A_ak v), kept transposed (rows value, inner token) ---------------------------------
     const Frag<T> aakf[2] = {to_frag<T>(aak[0]), to_frag<T>(aak[1])};
 #pragma unroll
     for (int vt = 0; vt < VT; ++vt) {
-        const Frag<T> vT = transpose(ld_frag_if(p.v + voff + 16 * vt, rowok), ident);
+        const Frag<T> vT = transpose(ld_frag_sel(p.v + voff + 16 * vt, rowok), ident);
         st_tile(p.ws.VTT + (chw * VT + vt) * TILE, vT);
         const Frag<T> mT[2] = {to_frag<T>(mm(vT, aakf[0], zero4())), to_frag<T>(mm(vT, aakf[1], zero4()))};
 #pragma unroll
@@ -170,9 +175,10 @@ __global__ __launch_bounds__(64) void prep_kernel(ChunkArgs<T> p) {
             f32x4 uT = zero4();
             uT = mm(mT[0], tm[s][0], uT);
             uT = mm(mT[1], tm[s][1], uT);
-            st_tile(p.ws.UT + ((chw * 2 + s) * VT + vt) * TILE, to_frag<T>(uT));
+            st_pair(p.ws.UT + (chw * VT + vt) * PAIR, s, to_frag<T>(uT));
         }
     }
+    PHASE_CLOCK(p, blk, 4);
 }
 
 // ---- chunk table for packed variable-length batches ----------------------------------------------------------
@@ -204,8 +210,14 @@ __global__ void build_chunk_table_kernel(const int64_t* cu, int N, int nch, int3
 template <typename T, int K, int V>
 static hipError_t launch_prep_kv(const ChunkArgs<T>& a, bool bwd, hipStream_t stream) {
     dim3 grid(a.st.nch, a.H), block(64);
-    if (bwd) hipLaunchKernelGGL((prep_kernel<T, K, V, true>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((prep_kernel<T, K, V, false>), grid, block, 0, stream, a);
+    constexpr bool kAlwaysF32 = sizeof(T) == 4;
+    if (kAlwaysF32 || a.gk_f32) {
+        if (bwd) hipLaunchKernelGGL((prep_kernel<T, true, K, V, true>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((prep_kernel<T, true, K, V, false>), grid, block, 0, stream, a);
+    } else {
+        if (bwd) hipLaunchKernelGGL((prep_kernel<T, kAlwaysF32, K, V, true>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((prep_kernel<T, kAlwaysF32, K, V, false>), grid, block, 0, stream, a);
+    }
     return hipGetLastError();
 }
 

@@ -9,8 +9,8 @@
 // The block lives in MFMA accumulators as the row fragment of S^T (rows = value column, inner = channel), which
 // is at once the operand layout of the next product: w S, qg S and the rank updates chain through registers
 // with no LDS traffic and no cross-lane movement.  All per-chunk operands were written by the prep kernel in
-// fragment order, so each is one coalesced 512-byte (bf16) load per tile; the loads of chunk c+1 are issued
-// before the products of chunk c.
+// fragment order, so each is one coalesced 512-byte (bf16) load per tile; the loads of the next few chunks are
+// in flight while one chunk is computed.
 #include "hdla_common.cuh"
 #include "hdla_launch.h"
 
@@ -25,25 +25,24 @@ struct FwdOps {
     f32x4 egl[KT];
 
     __device__ __forceinline__ void load(const Ws<T>& ws, int64_t chw, int vt) {
-        constexpr int VT = V / 16;
+        constexpr int VT = V / 16, KT2 = KT / 2;
         const int l = lane_id(), g = l >> 4;
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) {
-            w[0][kt] = ld_tile(ws.W + ((chw * 2 + 0) * KT + kt) * TILE);
-            w[1][kt] = ld_tile(ws.W + ((chw * 2 + 1) * KT + kt) * TILE);
-            kgt[kt] = ld_tile(ws.KGT + (chw * KT + kt) * TILE);
-            bgt[0][kt] = ld_tile(ws.BGT + ((chw * 2 + 0) * KT + kt) * TILE);
-            bgt[1][kt] = ld_tile(ws.BGT + ((chw * 2 + 1) * KT + kt) * TILE);
-            egl[kt] = *reinterpret_cast<const f32x4*>(ws.EGL + chw * K + 16 * kt + 4 * g);
-            if (WRITE_O) qg[kt] = ld_tile(ws.QG + (chw * KT + kt) * TILE);
+        for (int kp = 0; kp < KT2; ++kp) {
+            ld_pair(ws.W + ((chw * 2 + 0) * KT2 + kp) * PAIR, w[0][2 * kp], w[0][2 * kp + 1]);
+            ld_pair(ws.W + ((chw * 2 + 1) * KT2 + kp) * PAIR, w[1][2 * kp], w[1][2 * kp + 1]);
+            ld_pair(ws.KGT + (chw * KT2 + kp) * PAIR, kgt[2 * kp], kgt[2 * kp + 1]);
+            ld_pair(ws.BGT + ((chw * 2 + 0) * KT2 + kp) * PAIR, bgt[0][2 * kp], bgt[0][2 * kp + 1]);
+            ld_pair(ws.BGT + ((chw * 2 + 1) * KT2 + kp) * PAIR, bgt[1][2 * kp], bgt[1][2 * kp + 1]);
+            if (WRITE_O) ld_pair(ws.QG + (chw * KT2 + kp) * PAIR, qg[2 * kp], qg[2 * kp + 1]);
         }
-        ut[0] = ld_tile(ws.UT + ((chw * 2 + 0) * VT + vt) * TILE);
-        ut[1] = ld_tile(ws.UT + ((chw * 2 + 1) * VT + vt) * TILE);
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) egl[kt] = *reinterpret_cast<const f32x4*>(ws.EGL + chw * K + 16 * kt + 4 * g);
+        ld_pair(ws.UT + (chw * VT + vt) * PAIR, ut[0], ut[1]);
         vtt = ld_tile(ws.VTT + (chw * VT + vt) * TILE);
         if (WRITE_O) {
             aqk = ld_tile(ws.AQK + chw * TILE);
-            aqb[0] = ld_tile(ws.AQB + (chw * 2 + 0) * TILE);
-            aqb[1] = ld_tile(ws.AQB + (chw * 2 + 1) * TILE);
+            ld_pair(ws.AQB + chw * PAIR, aqb[0], aqb[1]);
         }
     }
 };
@@ -56,38 +55,43 @@ __global__ __launch_bounds__(64) void scan_fwd_kernel(ChunkArgs<T> p) {
     const int H = p.H;
     int c0, c1;
     seq_chunks(p.st, n, c0, c1);
+    int64_t bos, eos;
+    seq_bounds(p.st, n, bos, eos);
+    const int blk = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+    PHASE_CLOCK(p, blk, 0);
 
     // state block: lane (g,c) reg i of tile kt = S[16kt + 4g + i][16vt + c]
     f32x4 S[KT];
     const int64_t soff = ((int64_t)n * H + h) * K * V + 16 * vt + c;
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt) {
+    for (int kt = 0; kt < KT; ++kt) S[kt] = zero4();
+    if (p.h0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) S[kt][i] = p.h0 ? p.h0[soff + (int64_t)(16 * kt + 4 * g + i) * V] : 0.f;
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) S[kt][i] = p.h0[soff + (int64_t)(16 * kt + 4 * g + i) * V];
     }
 
-    // Operands of chunk c+1 are fetched while chunk c is computed when two sets fit the register file
-    // (bf16 operands, or fp32 with K = 64); otherwise one set is loaded per step.
-    constexpr bool PF = sizeof(T) == 2 || K == 64;
-    FwdOps<T, K, V, WRITE_O> cur, nxt;
-    if (PF && c0 < c1) cur.load(p.ws, (int64_t)h * p.st.nch + c0, vt);
-#pragma unroll 1
-    for (int cid = c0; cid < c1; ++cid) {
-        const int64_t chw = (int64_t)h * p.st.nch + cid;
-        if (PF) { if (cid + 1 < c1) nxt.load(p.ws, chw + 1, vt); }
-        else cur.load(p.ws, chw, vt);
-        ChunkPos cp;
-        locate_chunk(p.st, cid, cp);
+    // Operand sets of the next NBUF-1 chunks are in flight while one chunk is computed: each step of the scan
+    // would otherwise wait a full memory round trip.  NBUF is what the register file holds without spilling.
+    constexpr int NBUF = sizeof(T) == 2 ? (K == 64 ? 4 : 2) : (K == 64 ? 2 : 1);
+    FwdOps<T, K, V, WRITE_O> buf[NBUF];
+    const Frag<T> ident = ident_frag<T>();
+    const int64_t chw0 = (int64_t)h * p.st.nch;
 
+    auto step = [&](const FwdOps<T, K, V, WRITE_O>& cur, int cid) __attribute__((always_inline)) {
+        const int64_t chw = chw0 + cid;
+        const int64_t tok0 = bos + (int64_t)(cid - c0) * CH;
+        const int len = (int)min((int64_t)CH, eos - tok0);
         Frag<T> sb[KT];
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt) sb[kt] = to_frag<T>(S[kt]);
         if (!WRITE_O) {
-            T* hc = p.ws.HC + chw * (K * V) + 16 * vt + c;
+            // checkpoint of the entering state, row-major [K][V]: one transposing product per tile turns the
+            // register layout (4 channels of one value column per lane) into 4 consecutive values of one channel
+            T* hc = p.ws.HC + chw * (K * V) + 16 * vt + 4 * g;
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) st_elem(hc + (16 * kt + 4 * g + i) * V, S[kt][i]);
+            for (int kt = 0; kt < KT; ++kt) st_frag(hc + (16 * kt + c) * V, transpose(sb[kt], ident));
         }
         // v_new^T (rows value, inner token) = u^T + S^T w^T
         f32x4 vn[2] = {to_f32(cur.ut[0]), to_f32(cur.ut[1])};
@@ -98,11 +102,9 @@ __global__ __launch_bounds__(64) void scan_fwd_kernel(ChunkArgs<T> p) {
         }
         const Frag<T> vnb[2] = {to_frag<T>(vn[0]), to_frag<T>(vn[1])};
         if (!WRITE_O) {
-            T* vnp = p.ws.VN + chw * (2 * CH * V) + 16 * vt + c;
+            T* vnp = p.ws.VN + chw * (2 * CH * V) + 16 * vt + 4 * g;
 #pragma unroll
-            for (int s = 0; s < 2; ++s)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) st_elem(vnp + (s * CH + 4 * g + i) * V, vn[s][i]);
+            for (int s = 0; s < 2; ++s) st_frag(vnp + (s * CH + c) * V, transpose(vnb[s], ident));
         }
         if (WRITE_O) {
             // o (rows token, inner value) = qg S + A_qk v + sum_s A_qb^s v_new_s
@@ -112,7 +114,7 @@ __global__ __launch_bounds__(64) void scan_fwd_kernel(ChunkArgs<T> p) {
             o = mm(cur.aqk, cur.vtt, o);
             o = mm(cur.aqb[0], vnb[0], o);
             o = mm(cur.aqb[1], vnb[1], o);
-            if (c < cp.len) st_frag(p.o + ((cp.tok0 + c) * H + h) * V + 16 * vt + 4 * g, to_frag<T>(o));
+            if (c < len) st_frag(p.o + ((tok0 + c) * H + h) * V + 16 * vt + 4 * g, to_frag<T>(o));
         }
         // S <- exp(g_last) S + kg^T v + sum_s bg_s^T v_new_s
 #pragma unroll
@@ -123,8 +125,31 @@ __global__ __launch_bounds__(64) void scan_fwd_kernel(ChunkArgs<T> p) {
             x = mm(vnb[1], cur.bgt[1][kt], x);
             S[kt] = x;
         }
-        if (PF) cur = nxt;
+    };
+
+    // Every load of the main loop is unconditional (prefetch indices are clamped to the last chunk): a load or
+    // store that may or may not have been issued would force the compiler to wait for all outstanding memory
+    // operations instead of only those of the oldest operand set.
+    const int nfull = (c1 - c0) / NBUF;
+    if (c0 < c1) {
+#pragma unroll
+        for (int j = 0; j < NBUF - 1; ++j) buf[j].load(p.ws, chw0 + min(c0 + j, c1 - 1), vt);
+#pragma unroll 1
+        for (int gi = 0; gi < nfull; ++gi) {
+            const int base = c0 + gi * NBUF;
+#pragma unroll
+            for (int j = 0; j < NBUF; ++j) {
+                buf[(j + NBUF - 1) % NBUF].load(p.ws, chw0 + min(base + j + NBUF - 1, c1 - 1), vt);
+                step(buf[j], base + j);
+            }
+        }
+#pragma unroll 1
+        for (int cid = c0 + nfull * NBUF; cid < c1; ++cid) {      // fewer than NBUF chunks left
+            buf[0].load(p.ws, chw0 + cid, vt);
+            step(buf[0], cid);
+        }
     }
+    PHASE_CLOCK(p, blk, 1);
     if (p.ht) {
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
@@ -140,24 +165,27 @@ struct BwdOps {
     Frag<T> aqbt[2], bg[2][KT], wt[2][KT], qgt[KT], don;
     f32x4 egl[KT];
 
-    __device__ __forceinline__ void load(const ChunkArgs<T>& p, int cid, int h, int vt) {
+    __device__ __forceinline__ void load(const ChunkArgs<T>& p, int cid, int c0, int64_t bos, int64_t eos, int h, int vt) {
+        constexpr int KT2 = KT / 2;
         const int l = lane_id(), g = l >> 4, c = l & 15;
         const int64_t chw = (int64_t)h * p.st.nch + cid;
         const Ws<T>& ws = p.ws;
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) {
-            bg[0][kt] = ld_tile(ws.BG + ((chw * 2 + 0) * KT + kt) * TILE);
-            bg[1][kt] = ld_tile(ws.BG + ((chw * 2 + 1) * KT + kt) * TILE);
-            wt[0][kt] = ld_tile(ws.WT + ((chw * 2 + 0) * KT + kt) * TILE);
-            wt[1][kt] = ld_tile(ws.WT + ((chw * 2 + 1) * KT + kt) * TILE);
-            qgt[kt] = ld_tile(ws.QGT + (chw * KT + kt) * TILE);
-            egl[kt] = *reinterpret_cast<const f32x4*>(ws.EGL + chw * K + 16 * kt + 4 * g);
+        for (int kp = 0; kp < KT2; ++kp) {
+            ld_pair(ws.BG + ((chw * 2 + 0) * KT2 + kp) * PAIR, bg[0][2 * kp], bg[0][2 * kp + 1]);
+            ld_pair(ws.BG + ((chw * 2 + 1) * KT2 + kp) * PAIR, bg[1][2 * kp], bg[1][2 * kp + 1]);
+            ld_pair(ws.WT + ((chw * 2 + 0) * KT2 + kp) * PAIR, wt[0][2 * kp], wt[0][2 * kp + 1]);
+            ld_pair(ws.WT + ((chw * 2 + 1) * KT2 + kp) * PAIR, wt[1][2 * kp], wt[1][2 * kp + 1]);
+            ld_pair(ws.QGT + (chw * KT2 + kp) * PAIR, qgt[2 * kp], qgt[2 * kp + 1]);
         }
-        aqbt[0] = ld_tile(ws.AQBT + (chw * 2 + 0) * TILE);
-        aqbt[1] = ld_tile(ws.AQBT + (chw * 2 + 1) * TILE);
-        ChunkPos cp;
-        locate_chunk(p.st, cid, cp);
-        don = ld_frag_if(p.dout + ((cp.tok0 + c) * p.H + h) * V + 16 * vt + 4 * g, c < cp.len);
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) egl[kt] = *reinterpret_cast<const f32x4*>(ws.EGL + chw * K + 16 * kt + 4 * g);
+        ld_pair(ws.AQBT + chw * PAIR, aqbt[0], aqbt[1]);
+        // rows past the end of a ragged chunk alias its last row here and are zeroed where the value is used:
+        // a select right after the load would make the wave wait for this (youngest) load at once
+        const int64_t tok0 = bos + (int64_t)(cid - c0) * CH;
+        const int len = (int)min((int64_t)CH, eos - tok0);
+        don = ld_frag(p.dout + ((tok0 + min(c, len - 1)) * p.H + h) * V + 16 * vt + 4 * g);
     }
 };
 
@@ -169,34 +197,39 @@ __global__ __launch_bounds__(64) void scan_bwd_kernel(ChunkArgs<T> p) {
     const int H = p.H;
     int c0, c1;
     seq_chunks(p.st, n, c0, c1);
+    int64_t bos, eos;
+    seq_bounds(p.st, n, bos, eos);
+    const int blk = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+    PHASE_CLOCK(p, blk, 0);
 
     f32x4 dS[KT];   // lane (g,c) reg i of tile kt = dS[16kt + 4g + i][16vt + c]
     const int64_t soff = ((int64_t)n * H + h) * K * V + 16 * vt + c;
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt) {
+    for (int kt = 0; kt < KT; ++kt) dS[kt] = zero4();
+    if (p.dht) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dS[kt][i] = p.dht ? p.dht[soff + (int64_t)(16 * kt + 4 * g + i) * V] : 0.f;
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dS[kt][i] = p.dht[soff + (int64_t)(16 * kt + 4 * g + i) * V];
     }
     const Frag<T> ident = ident_frag<T>();
 
-    constexpr bool PF = sizeof(T) == 2 || K == 64;
-    BwdOps<T, K, V> cur, nxt;
-    if (PF && c0 < c1) cur.load(p, c1 - 1, h, vt);
-#pragma unroll 1
-    for (int cid = c1 - 1; cid >= c0; --cid) {
-        const int64_t chw = (int64_t)h * p.st.nch + cid;
-        if (PF) { if (cid > c0) nxt.load(p, cid - 1, h, vt); }
-        else cur.load(p, cid, h, vt);
+    constexpr int NBUF = sizeof(T) == 2 ? (K == 64 ? 4 : 2) : (K == 64 ? 2 : 1);
+    BwdOps<T, K, V> buf[NBUF];
 
+    auto step = [&](const BwdOps<T, K, V>& cur, int cid) __attribute__((always_inline)) {
+        const int64_t chw = (int64_t)h * p.st.nch + cid;
         Frag<T> dsb[KT];
-        T* dhc = p.ws.DHC + chw * (K * V) + 16 * vt + c;
+        T* dhc = p.ws.DHC + chw * (K * V) + 16 * vt + 4 * g;
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt) {
             dsb[kt] = to_frag<T>(dS[kt]);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) st_elem(dhc + (16 * kt + 4 * g + i) * V, dS[kt][i]);
+            st_frag(dhc + (16 * kt + c) * V, transpose(dsb[kt], ident));     // row-major [K][V], 8-byte stores
         }
-        const Frag<T> doT = transpose(cur.don, ident);      // rows value, inner token
+        const int len = (int)min((int64_t)CH, eos - (bos + (int64_t)(cid - c0) * CH));
+        Frag<T> don = cur.don;
+        if (c >= len) don = zero_frag<T>();
+        const Frag<T> doT = transpose(don, ident);          // rows value, inner token
         // dv_new_s^T (rows value, inner token) = do^T A_qb^s + dS^T bg_s^T
         f32x4 dvn[2];
         dvn[0] = mm(doT, cur.aqbt[0], zero4());
@@ -206,12 +239,10 @@ __global__ __launch_bounds__(64) void scan_bwd_kernel(ChunkArgs<T> p) {
             dvn[0] = mm(dsb[kt], cur.bg[0][kt], dvn[0]);
             dvn[1] = mm(dsb[kt], cur.bg[1][kt], dvn[1]);
         }
-        T* dvp = p.ws.DVN + chw * (2 * CH * V) + 16 * vt + c;
-#pragma unroll
-        for (int s = 0; s < 2; ++s)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) st_elem(dvp + (s * CH + 4 * g + i) * V, dvn[s][i]);
         const Frag<T> dvb[2] = {to_frag<T>(dvn[0]), to_frag<T>(dvn[1])};
+        T* dvp = p.ws.DVN + chw * (2 * CH * V) + 16 * vt + 4 * g;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) st_frag(dvp + (s * CH + c) * V, transpose(dvb[s], ident));
         // dS <- exp(g_last) dS + qg^T do + sum_s w_s^T dv_new_s
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt) {
@@ -221,8 +252,28 @@ __global__ __launch_bounds__(64) void scan_bwd_kernel(ChunkArgs<T> p) {
             x = mm(dvb[1], cur.wt[1][kt], x);
             dS[kt] = x;
         }
-        if (PF) cur = nxt;
+    };
+
+    const int nfull = (c1 - c0) / NBUF;
+    if (c0 < c1) {
+#pragma unroll
+        for (int j = 0; j < NBUF - 1; ++j) buf[j].load(p, max(c1 - 1 - j, c0), c0, bos, eos, h, vt);
+#pragma unroll 1
+        for (int gi = 0; gi < nfull; ++gi) {
+            const int base = c1 - 1 - gi * NBUF;
+#pragma unroll
+            for (int j = 0; j < NBUF; ++j) {
+                buf[(j + NBUF - 1) % NBUF].load(p, max(base - j - (NBUF - 1), c0), c0, bos, eos, h, vt);
+                step(buf[j], base - j);
+            }
+        }
+#pragma unroll 1
+        for (int cid = c1 - 1 - nfull * NBUF; cid >= c0; --cid) {
+            buf[0].load(p, cid, c0, bos, eos, h, vt);
+            step(buf[0], cid);
+        }
     }
+    PHASE_CLOCK(p, blk, 1);
     if (p.dh0) {
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)

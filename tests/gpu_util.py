@@ -20,6 +20,22 @@ def tiles(ws, off, dtype, H, nch, *lead):
     return t.reshape(H, nch, *lead, 16, 16).cpu()
 
 
+def pair_tiles(ws, off, dtype, H, nch, *lead):
+    """Like tiles(), for buffers whose tiles are stored interleaved in pairs along the last lead dimension:
+    element 8*lane + 4*which + i of a 512-element pair block belongs to tile `which` of the pair."""
+    n = 1
+    for x in lead:
+        n *= x
+    assert lead[-1] % 2 == 0
+    t = _raw(ws, off, H * nch * n * 256, dtype).double().reshape(H, nch, *lead[:-1], lead[-1] // 2, 64, 2, 4)
+    nd = t.dim()
+    t = t.transpose(nd - 3, nd - 2)                                   # [npairs, 2, 64, 4]
+    t = t.reshape(H, nch, *lead, 4, 16, 4)
+    nd = t.dim()
+    t = t.transpose(nd - 3, nd - 2)
+    return t.reshape(H, nch, *lead, 16, 16).cpu()
+
+
 def rows(ws, off, dtype, H, nch, *shape):
     n = 1
     for x in shape:

@@ -37,16 +37,16 @@ def test_workspace_buffers_backward_pass(B, T, H, K, V):
         return x.permute(1, 0, 2, *range(3, x.dim())).reshape(H, B * NT, *x.shape[3:])
 
     got = {
-        "W": (G.cat_tiles(G.tiles(ws, L["W"], dtype, H, nch, 2, KT), 3), bh(p["w"])),
-        "UT": (G.cat_tiles(G.tiles(ws, L["UT"], dtype, H, nch, 2, VT), 3, transpose=True), bh(p["u"])),
-        "KGT": (G.cat_tiles(G.tiles(ws, L["KGT"], dtype, H, nch, KT), 2, transpose=True), bh(p["kg"])),
-        "BGT": (G.cat_tiles(G.tiles(ws, L["BGT"], dtype, H, nch, 2, KT), 3, transpose=True), bh(p["bg"])),
+        "W": (G.cat_tiles(G.pair_tiles(ws, L["W"], dtype, H, nch, 2, KT), 3), bh(p["w"])),
+        "UT": (G.cat_tiles(G.pair_tiles(ws, L["UT"], dtype, H, nch, VT, 2).transpose(2, 3), 3, transpose=True), bh(p["u"])),
+        "KGT": (G.cat_tiles(G.pair_tiles(ws, L["KGT"], dtype, H, nch, KT), 2, transpose=True), bh(p["kg"])),
+        "BGT": (G.cat_tiles(G.pair_tiles(ws, L["BGT"], dtype, H, nch, 2, KT), 3, transpose=True), bh(p["bg"])),
         "VTT": (G.cat_tiles(G.tiles(ws, L["VTT"], dtype, H, nch, VT), 2, transpose=True), bh(p["v"])),
         "EGL": (G.rows(ws, L["EGL"], torch.float32, H, nch, K), bh(torch.exp(p["gl"]))[..., 0, :]),
-        "AQBT": (G.tiles(ws, L["AQBT"], dtype, H, nch, 2), bh(p["Aqb"]).transpose(-1, -2)),
-        "BG": (G.cat_tiles(G.tiles(ws, L["BG"], dtype, H, nch, 2, KT), 3), bh(p["bg"])),
-        "WT": (G.cat_tiles(G.tiles(ws, L["WT"], dtype, H, nch, 2, KT), 3, transpose=True), bh(p["w"])),
-        "QGT": (G.cat_tiles(G.tiles(ws, L["QGT"], dtype, H, nch, KT), 2, transpose=True), bh(p["qg"])),
+        "AQBT": (G.pair_tiles(ws, L["AQBT"], dtype, H, nch, 2), bh(p["Aqb"]).transpose(-1, -2)),
+        "BG": (G.cat_tiles(G.pair_tiles(ws, L["BG"], dtype, H, nch, 2, KT), 3), bh(p["bg"])),
+        "WT": (G.cat_tiles(G.pair_tiles(ws, L["WT"], dtype, H, nch, 2, KT), 3, transpose=True), bh(p["w"])),
+        "QGT": (G.cat_tiles(G.pair_tiles(ws, L["QGT"], dtype, H, nch, KT), 2, transpose=True), bh(p["qg"])),
         "TM": (G.rows(ws, L["TM"], torch.float32, H, nch, 2, 16, 2, 16), bh(p["Tm"]).permute(0, 1, 2, 4, 3, 5)),
         "HC": (G.rows(ws, L["HC"], dtype, H, nch, K, V), bh(f["h"])),
         "VN": (G.rows(ws, L["VN"], dtype, H, nch, 2, 16, V), bh(f["vn"])),
@@ -80,9 +80,9 @@ def test_workspace_buffers_forward_pass(K, V):
     NT = p["q"].shape[2]
     bh = lambda x: x.permute(1, 0, 2, *range(3, x.dim())).reshape(H, B * NT, *x.shape[3:])
     errs = {
-        "QG": O.rel_l2(G.cat_tiles(G.tiles(ws, L["QG"], dtype, H, nch, KT), 2), bh(p["qg"])),
+        "QG": O.rel_l2(G.cat_tiles(G.pair_tiles(ws, L["QG"], dtype, H, nch, KT), 2), bh(p["qg"])),
         "AQK": O.rel_l2(G.tiles(ws, L["AQK"], dtype, H, nch), bh(p["Aqk"])),
-        "AQB": O.rel_l2(G.tiles(ws, L["AQB"], dtype, H, nch, 2), bh(p["Aqb"])),
+        "AQB": O.rel_l2(G.pair_tiles(ws, L["AQB"], dtype, H, nch, 2), bh(p["Aqb"])),
         "o": O.rel_l2(o, CS._unchunk(f["o"], T)),
         "ht": O.rel_l2(ht, f["ht"]),
     }
