@@ -5,7 +5,8 @@
 // scan_bwd replaces HRDPLR/bwd_triton.py:127-222 (reverse recurrence of the state gradient, dh checkpoints,
 // dh0) fused with the dv_new part of HRDPLR/bwd_triton.py:30-105.
 //
-// One wavefront owns a K x 16 column block of the fp32 state of one (sequence, head) for the whole sequence.
+// One wavefront owns a K x 16 column block of the fp32 state of one (sequence, head) for the whole sequence;
+// one single-wave workgroup each, numbered so that the blocks of one (sequence, head) share an XCD's L2.
 // The block lives in MFMA accumulators as the row fragment of S^T (rows = value column, inner = channel), which
 // is at once the operand layout of the next product: w S, qg S and the rank updates chain through registers
 // with no LDS traffic and no cross-lane movement.  All per-chunk operands were written by the prep kernel in
@@ -15,6 +16,25 @@
 #include "hdla_launch.h"
 
 namespace hdla {
+
+// ---- block numbering ------------------------------------------------------------------------------------------
+// The V/16 column blocks of one (sequence, head) read the same w/kg/bg/qg tiles.  Workgroups are handed to the
+// eight XCDs round-robin by their linear index and each XCD has its own L2, so the linear index is decoded as
+// (pair mod 8) + 8 * (column block + V/16 * (pair / 8)): all column blocks of a pair land on one XCD (shared
+// tiles come from HBM once per pair instead of V/16 times) but on different compute units (each wave keeps a
+// whole register file and its own L1 bandwidth).
+constexpr int XCDS = 8;
+static inline unsigned scan_grid(int H, int N, int VT) { return (unsigned)(XCDS * VT * ((H * N + XCDS - 1) / XCDS)); }
+template <typename T>
+__device__ __forceinline__ bool scan_block(const ChunkArgs<T>& p, int VT, int& vt, int& h, int& n) {
+    const int L = blockIdx.x, xcd = L % XCDS, idx = L / XCDS;
+    vt = idx % VT;
+    const int pair = (idx / VT) * XCDS + xcd;
+    if (pair >= p.H * p.st.N) return false;
+    n = pair / p.H;
+    h = pair - n * p.H;
+    return true;
+}
 
 // ---- forward -------------------------------------------------------------------------------------------------
 template <typename T, int K, int V, bool WRITE_O>
@@ -50,14 +70,15 @@ struct FwdOps {
 template <typename T, int K, int V, bool WRITE_O>
 __global__ __launch_bounds__(64) void scan_fwd_kernel(ChunkArgs<T> p) {
     constexpr int KT = K / 16;
-    const int vt = blockIdx.x, h = blockIdx.y, n = blockIdx.z;
+    int vt, h, n;
+    if (!scan_block(p, V / 16, vt, h, n)) return;
     const int l = lane_id(), g = l >> 4, c = l & 15;
     const int H = p.H;
     int c0, c1;
     seq_chunks(p.st, n, c0, c1);
     int64_t bos, eos;
     seq_bounds(p.st, n, bos, eos);
-    const int blk = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+    const int blk = blockIdx.x;
     PHASE_CLOCK(p, blk, 0);
 
     // state block: lane (g,c) reg i of tile kt = S[16kt + 4g + i][16vt + c]
@@ -192,14 +213,15 @@ struct BwdOps {
 template <typename T, int K, int V>
 __global__ __launch_bounds__(64) void scan_bwd_kernel(ChunkArgs<T> p) {
     constexpr int KT = K / 16;
-    const int vt = blockIdx.x, h = blockIdx.y, n = blockIdx.z;
+    int vt, h, n;
+    if (!scan_block(p, V / 16, vt, h, n)) return;
     const int l = lane_id(), g = l >> 4, c = l & 15;
     const int H = p.H;
     int c0, c1;
     seq_chunks(p.st, n, c0, c1);
     int64_t bos, eos;
     seq_bounds(p.st, n, bos, eos);
-    const int blk = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+    const int blk = blockIdx.x;
     PHASE_CLOCK(p, blk, 0);
 
     f32x4 dS[KT];   // lane (g,c) reg i of tile kt = dS[16kt + 4g + i][16vt + c]
@@ -285,14 +307,14 @@ __global__ __launch_bounds__(64) void scan_bwd_kernel(ChunkArgs<T> p) {
 // ---- launchers -----------------------------------------------------------------------------------------------
 template <typename T, int K, int V>
 static hipError_t launch_scan_fwd_kv(const ChunkArgs<T>& a, bool write_o, hipStream_t stream) {
-    dim3 grid(V / 16, a.H, a.st.N), block(64);
+    dim3 grid(scan_grid(a.H, a.st.N, V / 16)), block(64);
     if (write_o) hipLaunchKernelGGL((scan_fwd_kernel<T, K, V, true>), grid, block, 0, stream, a);
     else hipLaunchKernelGGL((scan_fwd_kernel<T, K, V, false>), grid, block, 0, stream, a);
     return hipGetLastError();
 }
 template <typename T, int K, int V>
 static hipError_t launch_scan_bwd_kv(const ChunkArgs<T>& a, hipStream_t stream) {
-    dim3 grid(V / 16, a.H, a.st.N), block(64);
+    dim3 grid(scan_grid(a.H, a.st.N, V / 16)), block(64);
     hipLaunchKernelGGL((scan_bwd_kernel<T, K, V>), grid, block, 0, stream, a);
     return hipGetLastError();
 }
