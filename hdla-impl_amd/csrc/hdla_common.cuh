@@ -199,28 +199,34 @@ __device__ __forceinline__ void seq_bounds(const SeqTab& st, int n, int64_t& bos
 }
 
 // ---- per-chunk decay quantities in fragment layout ---------------------------------------------------------
-// lane (g,c) holds token c of the chunk and channels 16*kt + 4g + i.  An inclusive prefix sum over the 16 lanes
-// of a group gives the cumulative log-decay gi; ge = gi - g is the exclusive one.
-__device__ __forceinline__ f32x4 scan16_incl(f32x4 x) {
-    const int c = lane_id() & 15;
-#pragma unroll
-    for (int off = 1; off < 16; off <<= 1) {
-        f32x4 t;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) t[i] = __shfl_up(x[i], off, 16);
-        if (c >= off) x += t;
-    }
+// lane (g,c) holds token c of the chunk and channels 16*kt + 4g + i.  The 16 lanes of a group are one DPP "row",
+// so prefix sums, suffix sums and sums over the tokens of a chunk are row_shr / row_shl / mirror additions on
+// the vector ALU (out-of-row lanes read 0), with no LDS round trips.
+template <int CTRL> __device__ __forceinline__ float dpp0(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+template <int CTRL> __device__ __forceinline__ f32x4 dpp0(f32x4 x) {
+    f32x4 r; r[0] = dpp0<CTRL>(x[0]); r[1] = dpp0<CTRL>(x[1]); r[2] = dpp0<CTRL>(x[2]); r[3] = dpp0<CTRL>(x[3]); return r;
+}
+__device__ __forceinline__ f32x4 scan16_incl(f32x4 x) {     // inclusive prefix sum over the 16 lanes of a group
+    x += dpp0<0x111>(x);    // row_shr:1
+    x += dpp0<0x112>(x);    // row_shr:2
+    x += dpp0<0x114>(x);    // row_shr:4
+    x += dpp0<0x118>(x);    // row_shr:8
     return x;
 }
-__device__ __forceinline__ f32x4 rscan16_incl(f32x4 x) {   // suffix sum over the 16 lanes of a group
-    const int c = lane_id() & 15;
-#pragma unroll
-    for (int off = 1; off < 16; off <<= 1) {
-        f32x4 t;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) t[i] = __shfl_down(x[i], off, 16);
-        if (c + off < 16) x += t;
-    }
+__device__ __forceinline__ f32x4 rscan16_incl(f32x4 x) {    // inclusive suffix sum over the 16 lanes of a group
+    x += dpp0<0x101>(x);    // row_shl:1
+    x += dpp0<0x102>(x);
+    x += dpp0<0x104>(x);
+    x += dpp0<0x108>(x);
+    return x;
+}
+__device__ __forceinline__ f32x4 sum16(f32x4 x) {           // sum over the 16 lanes of a group, on all of them
+    x += dpp0<0xB1>(x);     // quad_perm:[1,0,3,2]
+    x += dpp0<0x4E>(x);     // quad_perm:[2,3,0,1]
+    x += dpp0<0x141>(x);    // row_half_mirror
+    x += dpp0<0x140>(x);    // row_mirror
     return x;
 }
 __device__ __forceinline__ f32x4 bcast16(f32x4 x, int src) {  // value of lane `src` of the own 16-lane group
@@ -229,15 +235,11 @@ __device__ __forceinline__ f32x4 bcast16(f32x4 x, int src) {  // value of lane `
     for (int i = 0; i < 4; ++i) r[i] = __shfl(x[i], src, 16);
     return r;
 }
-__device__ __forceinline__ f32x4 sum16(f32x4 x) {             // sum over the 16 lanes of a group, on all of them
-#pragma unroll
-    for (int off = 1; off < 16; off <<= 1) {
-        f32x4 t;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) t[i] = __shfl_xor(x[i], off, 16);
-        x += t;
-    }
-    return x;
+// value held by the lane 32 positions away (v_permlane32_swap exchanges the two halves of the wave)
+__device__ __forceinline__ float xor32(float x) {
+    const int xi = __float_as_int(x);
+    auto r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+    return __int_as_float(lane_id() < 32 ? r[1] : r[0]);
 }
 
 }  // namespace hdla

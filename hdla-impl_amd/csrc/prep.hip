@@ -90,19 +90,33 @@ __global__ __launch_bounds__(64) void prep_kernel(ChunkArgs<T> p) {
     __syncthreads();
     PHASE_CLOCK(p, blk, 1);
 
-    // ---- phase B: (I - A_ab)^-1 by forward substitution over tokens, two rank rows x 32 columns per step ----
+    // ---- phase B: (I - A_ab)^-1 by forward substitution over tokens, in registers -----------------------------
+    // Lane (r, col) builds column `col` of the rows (r, i), i = 0..15, one token per step; the entries of the
+    // other rank's rows come from the lane 32 positions away.  The coefficients N[(r,i)][*] are uniform per
+    // half-wave (LDS broadcast reads, off the dependency chain); entries with j >= i are zero by the mask.
     {
         const int r = l >> 5, col = l & 31;
+        float x[16], y[16];                      // own rows (r, j) and the partner's rows (1-r, j) of column col
+#pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const int row = 16 * r + i;
-            float acc = (col == row) ? 1.f : 0.f;
-            for (int j = 0; j < i; ++j) {
-                acc = fmaf(sN[row * LDP + j], sT[j * LDP + col], acc);
-                acc = fmaf(sN[row * LDP + 16 + j], sT[(16 + j) * LDP + col], acc);
+            const float* nrow = &sN[(16 * r + i) * LDP];
+            float acc0 = (col == 16 * r + i) ? 1.f : 0.f, acc1 = 0.f;
+#pragma unroll
+            for (int j4 = 0; j4 < (i + 3) / 4; ++j4) {
+                const f32x4 co = *reinterpret_cast<const f32x4*>(nrow + 16 * r + 4 * j4);         // own rank block
+                const f32x4 cx = *reinterpret_cast<const f32x4*>(nrow + 16 * (1 - r) + 4 * j4);   // other rank block
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) {
+                    const int j = 4 * j4 + jj;
+                    if (j < i) { acc0 = fmaf(co[jj], x[j], acc0); acc1 = fmaf(cx[jj], y[j], acc1); }
+                }
             }
-            sT[row * LDP + col] = acc;
-            __syncthreads();
+            x[i] = acc0 + acc1;
+            y[i] = xor32(x[i]);
         }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sT[(16 * r + i) * LDP + col] = x[i];
+        __syncthreads();
     }
     PHASE_CLOCK(p, blk, 2);
     Frag<T> tm[2][2];   // F(Tm^{s s'}): rows i, inner j
