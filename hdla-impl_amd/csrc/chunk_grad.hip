@@ -20,7 +20,8 @@ namespace hdla {
 constexpr int LDG = 36;
 
 template <typename T, bool GKF32, int K, int V>
-__global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 2 && K == 64 && V == 64 ? 2 : 1, sizeof(T) == 2 && K == 64 && V == 64 ? 2 : 1)))
+void chunk_grad_kernel(ChunkArgs<T> p) {
     constexpr int KT = K / 16, VT = V / 16;
     __shared__ __attribute__((aligned(16))) float sT[32 * LDG];   // (I - A_ab)^-1, rank-major
 
@@ -66,15 +67,15 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     const Frag<T> ident = ident_frag<T>();
 
     // ---- cumulative decays; A_qk^T and A_ak^T (rows j, inner i) -----------------------------------------------
-    f32x4 gi[KT], ge[KT];
+    // (the decays are recomputed per channel tile wherever they are needed: a load and four DPP additions cost
+    // less than keeping 2*K/16 vector registers alive across the kernel)
     f32x4 aqkT = zero4(), aakT[2] = {zero4(), zero4()};
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
         const f32x4 g4 = ld_gk4<GKF32>(p.gk, qoff + 16 * kt, rowok);
-        gi[kt] = scan16_incl(g4);
-        ge[kt] = gi[kt] - g4;
-        const f32x4 m = bcast16(gi[kt], MID);
-        const f32x4 eq = exp4<T>(gi[kt] - m), ek = exp4<T>(m - gi[kt]), ea = exp4<T>(ge[kt] - m);
+        const f32x4 gi = scan16_incl(g4), ge = gi - g4;
+        const f32x4 m = bcast16(gi, MID);
+        const f32x4 eq = exp4<T>(gi - m), ek = exp4<T>(m - gi), ea = exp4<T>(ge - m);
         const f32x4 q4 = to_f32(ld_frag_sel(p.q + qoff + 16 * kt, rowok));
         const f32x4 k4 = to_f32(ld_frag_sel(p.k + qoff + 16 * kt, rowok));
         const f32x4 a0 = to_f32(ld_frag_sel(p.a + aoff0 + 16 * kt, rowok));
@@ -134,8 +135,7 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     }
 
     PHASE_CLOCK(p, blk, 2);
-    // ---- first pass over channel tiles: dw -> dag, and the w part of dA_ab ------------------------------------
-    f32x4 dag[2][KT];
+    // ---- first pass over channel tiles: dw -> dag -> the w part of dA_ab (dag itself is rebuilt in pass two) ----
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
         f32x4 dwT[2] = {zero4(), zero4()};                // rows channel, inner token
@@ -149,8 +149,7 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
             f32x4 x = mm(tmT[0][r], dwTf[0], zero4());
-            x = mm(tmT[1][r], dwTf[1], x);
-            dag[r][kt] = x;                               // rows token, inner channel
+            x = mm(tmT[1][r], dwTf[1], x);                // dag_r: rows token, inner channel
             const Frag<T> dagf = to_frag<T>(x);
             dAab[r][0] = mm(dagf, ld_pair_one(p.ws.W + ((chw * 2 + 0) * (KT / 2) + kt / 2) * PAIR, kt & 1), dAab[r][0]);
             dAab[r][1] = mm(dagf, ld_pair_one(p.ws.W + ((chw * 2 + 1) * (KT / 2) + kt / 2) * PAIR, kt & 1), dAab[r][1]);
@@ -177,23 +176,19 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
 
     PHASE_CLOCK(p, blk, 4);
     // ---- second pass over channel tiles: state products, score backward, final gradients ----------------------
-#pragma unroll
+#pragma unroll 1
     for (int kt = 0; kt < KT; ++kt) {
-        const f32x4 m = bcast16(gi[kt], MID), gl = bcast16(gi[kt], CH - 1);
-        const f32x4 eq = exp4<T>(gi[kt] - m), ek = exp4<T>(m - gi[kt]), ea = exp4<T>(ge[kt] - m);
-        const f32x4 egi = exp4<T>(gi[kt]), ege = exp4<T>(ge[kt]), edn = exp4<T>(gl - gi[kt]);
-        const f32x4 q4 = to_f32(ld_frag_sel(p.q + qoff + 16 * kt, rowok));
+        // (a) what the loop over value tiles needs: only kg of this channel tile
+        const f32x4 g4 = ld_gk4<GKF32>(p.gk, qoff + 16 * kt, rowok);
+        const f32x4 gi = scan16_incl(g4);
+        const f32x4 gl = bcast16(gi, CH - 1);
+        const f32x4 edn = exp4<T>(gl - gi);
         const f32x4 k4 = to_f32(ld_frag_sel(p.k + qoff + 16 * kt, rowok));
-        const f32x4 a4[2] = {to_f32(ld_frag_sel(p.a + aoff0 + 16 * kt, rowok)), to_f32(ld_frag_sel(p.a + aoff1 + 16 * kt, rowok))};
-        const f32x4 b4[2] = {to_f32(ld_frag_sel(p.b + aoff0 + 16 * kt, rowok)), to_f32(ld_frag_sel(p.b + aoff1 + 16 * kt, rowok))};
-        const Frag<T> qhT = transpose(to_frag<T>(q4 * eq * scale), ident), khT = transpose(to_frag<T>(k4 * ek), ident);
-        const Frag<T> ahT[2] = {transpose(to_frag<T>(a4[0] * ea), ident), transpose(to_frag<T>(a4[1] * ea), ident)};
-        const Frag<T> bhT[2] = {transpose(to_frag<T>(b4[0] * ek), ident), transpose(to_frag<T>(b4[1] * ek), ident)};
         const f32x4 kg4 = k4 * edn;
-        const f32x4 bg4[2] = {b4[0] * edn, b4[1] * edn};
         const Frag<T> kgf = to_frag<T>(kg4);
 
         f32x4 dqg = zero4(), dkg = zero4(), dbg[2] = {zero4(), zero4()};
+        f32x4 dwT[2] = {zero4(), zero4()};                 // dw_s^T for this channel tile (rows channel, inner token)
         float hh = 0.f;                                    // partial of sum_v S * dS for channel 16kt + c
 #pragma unroll
         for (int vt = 0; vt < VT; ++vt) {
@@ -202,6 +197,8 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
             const Frag<T> doN = ld_frag_sel(p.dout + voff + 16 * vt, rowok);
             const Frag<T> vN = ld_frag_sel(p.v + voff + 16 * vt, rowok);
             dqg = mm(doN, Sf, dqg);
+            dwT[0] = mm(Sf, ld_frag(DVN + (0 * CH + c) * V + 16 * vt + 4 * g), dwT[0]);
+            dwT[1] = mm(Sf, ld_frag(DVN + (1 * CH + c) * V + 16 * vt + 4 * g), dwT[1]);
             dkg = mm(vN, dSf, dkg);
             dbg[0] = mm(ld_frag(VN + (0 * CH + c) * V + 16 * vt + 4 * g), dSf, dbg[0]);
             dbg[1] = mm(ld_frag(VN + (1 * CH + c) * V + 16 * vt + 4 * g), dSf, dbg[1]);
@@ -215,6 +212,25 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) hh4[i] = __shfl(hh, 4 * g + i);
 
+        const Frag<T> dwTf[2] = {to_frag<T>(dwT[0]), to_frag<T>(dwT[1])};
+        f32x4 dag[2];                                      // dag_r = sum_s (Tm^{s r})^T dw_s, rows token, inner channel
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            dag[r] = mm(tmT[0][r], dwTf[0], zero4());
+            dag[r] = mm(tmT[1][r], dwTf[1], dag[r]);
+        }
+        // (b) the factorised operands and decay factors of this channel tile, for the score backward
+        const f32x4 ge = gi - g4;
+        const f32x4 m = bcast16(gi, MID);
+        const f32x4 eq = exp4<T>(gi - m), ek = exp4<T>(m - gi), ea = exp4<T>(ge - m);
+        const f32x4 egi = exp4<T>(gi), ege = exp4<T>(ge);
+        const f32x4 q4 = to_f32(ld_frag_sel(p.q + qoff + 16 * kt, rowok));
+        const f32x4 a4[2] = {to_f32(ld_frag_sel(p.a + aoff0 + 16 * kt, rowok)), to_f32(ld_frag_sel(p.a + aoff1 + 16 * kt, rowok))};
+        const f32x4 b4[2] = {to_f32(ld_frag_sel(p.b + aoff0 + 16 * kt, rowok)), to_f32(ld_frag_sel(p.b + aoff1 + 16 * kt, rowok))};
+        const Frag<T> qhT = transpose(to_frag<T>(q4 * eq * scale), ident), khT = transpose(to_frag<T>(k4 * ek), ident);
+        const Frag<T> ahT[2] = {transpose(to_frag<T>(a4[0] * ea), ident), transpose(to_frag<T>(a4[1] * ea), ident)};
+        const Frag<T> bhT[2] = {transpose(to_frag<T>(b4[0] * ek), ident), transpose(to_frag<T>(b4[1] * ek), ident)};
+        const f32x4 bg4[2] = {b4[0] * edn, b4[1] * edn};
         f32x4 dqh = mm(fAqk, khT, zero4());
         dqh = mm(fAqb[0], bhT[0], dqh);
         dqh = mm(fAqb[1], bhT[1], dqh);
@@ -235,7 +251,7 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         }
         const f32x4 dq = (dqh * eq + dqg * egi) * scale;
         const f32x4 dk = dkh * ek + dkg * edn;
-        const f32x4 da[2] = {dah[0] * ea + dag[0][kt] * ege, dah[1] * ea + dag[1][kt] * ege};
+        const f32x4 da[2] = {dah[0] * ea + dag[0] * ege, dah[1] * ea + dag[1] * ege};
         const f32x4 db[2] = {dbh[0] * ek + dbg[0] * edn, dbh[1] * ek + dbg[1] * edn};
         const f32x4 Dge = da[0] * a4[0] + da[1] * a4[1];
         const f32x4 Dgi = dq * q4 - dk * k4 - db[0] * b4[0] - db[1] * b4[1];

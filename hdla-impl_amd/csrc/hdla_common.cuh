@@ -52,15 +52,26 @@ __device__ __forceinline__ uint16_t f2bf(float f) {
 
 template <typename T> __device__ __forceinline__ Frag<T> to_frag(f32x4 a);
 template <> __device__ __forceinline__ Frag<bf16> to_frag<bf16>(f32x4 a) {
+    // two v_cvt_pk_bf16_f32 (round to nearest even), results already packed in operand order
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+    const f32x2 lo = {a[0], a[1]}, hi = {a[2], a[3]};
+    u32x2 w;
+    w[0] = __builtin_bit_cast(unsigned, __builtin_convertvector(lo, bf16x2));
+    w[1] = __builtin_bit_cast(unsigned, __builtin_convertvector(hi, bf16x2));
     Frag<bf16> r;
-    r.v[0] = (short)f2bf(a[0]); r.v[1] = (short)f2bf(a[1]); r.v[2] = (short)f2bf(a[2]); r.v[3] = (short)f2bf(a[3]);
+    r.v = __builtin_bit_cast(s16x4, w);
     return r;
 }
 template <> __device__ __forceinline__ Frag<float> to_frag<float>(f32x4 a) { Frag<float> r; r.v = a; return r; }
 
 __device__ __forceinline__ f32x4 to_f32(Frag<bf16> a) {
+    typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 w = __builtin_bit_cast(u32x2, a.v);
     f32x4 r;
-    r[0] = bf2f((uint16_t)a.v[0]); r[1] = bf2f((uint16_t)a.v[1]); r[2] = bf2f((uint16_t)a.v[2]); r[3] = bf2f((uint16_t)a.v[3]);
+    r[0] = __uint_as_float(w[0] << 16); r[1] = __uint_as_float(w[0] & 0xffff0000u);
+    r[2] = __uint_as_float(w[1] << 16); r[3] = __uint_as_float(w[1] & 0xffff0000u);
     return r;
 }
 __device__ __forceinline__ f32x4 to_f32(Frag<float> a) { return a.v; }
