@@ -89,6 +89,24 @@ __device__ __forceinline__ f32x4 mm(Frag<float> frows, Frag<float> finner, f32x4
     return acc;
 }
 
+// Split operands for the score products of the bf16 path: x = hi + lo with both halves bf16, and
+// P Q^T ~ Ph Qh^T + Ph Ql^T + Pl Qh^T, which removes the rounding of the decayed operands (the largest single
+// contribution to the forward error) at the price of two more MFMAs per product.  fp32 operands need no split.
+template <typename T> struct Split;
+template <> struct Split<bf16> { Frag<bf16> hi, lo; };
+template <> struct Split<float> { Frag<float> hi; };
+__device__ __forceinline__ void split(f32x4 x, Split<bf16>& s) {
+    s.hi = to_frag<bf16>(x);
+    s.lo = to_frag<bf16>(x - to_f32(s.hi));
+}
+__device__ __forceinline__ void split(f32x4 x, Split<float>& s) { s.hi.v = x; }
+__device__ __forceinline__ f32x4 mm3(const Split<bf16>& p, const Split<bf16>& q, f32x4 acc) {
+    acc = mm(p.lo, q.hi, acc);
+    acc = mm(p.hi, q.lo, acc);
+    return mm(p.hi, q.hi, acc);
+}
+__device__ __forceinline__ f32x4 mm3(const Split<float>& p, const Split<float>& q, f32x4 acc) { return mm(p.hi, q.hi, acc); }
+
 // F(I16): used to transpose a tile with one product, F(X^T) = mm(F(I), F(X)).
 template <typename T> __device__ __forceinline__ Frag<T> ident_frag() {
     const int l = lane_id(), g = l >> 4, c = l & 15;

@@ -52,17 +52,21 @@ __global__ __launch_bounds__(64) void prep_kernel(ChunkArgs<T> p) {
         const f32x4 a1 = to_f32(ld_frag_sel(p.a + aoff1 + 16 * kt, rowok));
         const f32x4 b0 = to_f32(ld_frag_sel(p.b + aoff0 + 16 * kt, rowok));
         const f32x4 b1 = to_f32(ld_frag_sel(p.b + aoff1 + 16 * kt, rowok));
-        const Frag<T> qh = to_frag<T>(q4 * eq * scale), kh = to_frag<T>(k4 * ek);
-        const Frag<T> ah[2] = {to_frag<T>(a0 * ea), to_frag<T>(a1 * ea)};
-        const Frag<T> bh[2] = {to_frag<T>(b0 * ek), to_frag<T>(b1 * ek)};
-        aqk = mm(qh, kh, aqk);
+        Split<T> qh, kh, ah[2], bh[2];
+        split(q4 * eq * scale, qh);
+        split(k4 * ek, kh);
+        split(a0 * ea, ah[0]);
+        split(a1 * ea, ah[1]);
+        split(b0 * ek, bh[0]);
+        split(b1 * ek, bh[1]);
+        aqk = mm3(qh, kh, aqk);
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            aqb[s] = mm(qh, bh[s], aqb[s]);
-            aak[s] = mm(ah[s], kh, aak[s]);
-            if (BWD) aqbT[s] = mm(bh[s], qh, aqbT[s]);
+            aqb[s] = mm3(qh, bh[s], aqb[s]);
+            aak[s] = mm3(ah[s], kh, aak[s]);
+            if (BWD) aqbT[s] = mm3(bh[s], qh, aqbT[s]);
 #pragma unroll
-            for (int r = 0; r < 2; ++r) aab[r][s] = mm(ah[r], bh[s], aab[r][s]);
+            for (int r = 0; r < 2; ++r) aab[r][s] = mm3(ah[r], bh[s], aab[r][s]);
         }
     }
     // causal masks: lane (g,c) reg i is entry (row c, inner 4g+i)
