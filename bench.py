@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the HDLA rank-2 DPLR delta-rule hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload train|fwd|varlen|decode] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload train|fwd|varlen|decode|copy] [--no-cpu-baseline]
 
 Default workload ("train") is the headline configuration: chunked forward + backward at B=4, T=2048, H=16,
 K=V=64, bf16 inputs, fp32 state, random fp32 initial state, upstream gradients do and dht (configuration 2).
@@ -35,7 +35,7 @@ def _args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="train", choices=["train", "fwd", "varlen", "decode"])
+    ap.add_argument("--workload", default="train", choices=["train", "fwd", "varlen", "decode", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
 
@@ -160,6 +160,16 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     wl = args.workload
+    if wl == "copy":
+        # calibration workload for the HBM traffic counters: a plain device-to-device copy of known size
+        # (reads n bytes, writes n bytes per launch); not a benchmark of this library
+        n = 1 << 30
+        x = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
+        y = torch.empty_like(x)
+        sec = time_steps(lambda: y.copy_(x), args.steps, args.warmup)
+        print(json.dumps({"metric": "copy calibration", "bytes_read_per_launch": n, "bytes_written_per_launch": n,
+                          "ms_per_step": sec * 1e3, "GB/s": 2 * n / sec / 1e9}))
+        return
     cfg = {"train": 2, "fwd": 1, "varlen": 3, "decode": 4}[wl]
     B, T, H, K, V = CONFIG_SHAPES[cfg]
     inp = make_config(cfg)

@@ -20,10 +20,14 @@ namespace hdla {
 constexpr int LDG = 36;
 
 template <typename T, bool GKF32, int K, int V>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 2 && K == 64 && V == 64 ? 2 : 1, sizeof(T) == 2 && K == 64 && V == 64 ? 2 : 1)))
-void chunk_grad_kernel(ChunkArgs<T> p) {
+__global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     constexpr int KT = K / 16, VT = V / 16;
     __shared__ __attribute__((aligned(16))) float sT[32 * LDG];   // (I - A_ab)^-1, rank-major
+    // do, v, v_new (2 ranks) and dv_new (2 ranks) of the chunk, [matrix][token][value], staged once: every one of
+    // them is an operand of several products in every pass, and the working set of the resident waves is far
+    // larger than the L2, so repeated global loads would mostly be repeated HBM reads
+    constexpr int VP = V + 16 / (int)sizeof(T);                    // padded row, keeps 16-byte alignment
+    __shared__ __attribute__((aligned(16))) T sTok[6 * CH * VP];
 
     const int cid = blockIdx.x, h = blockIdx.y;
     ChunkPos cp;
@@ -45,6 +49,33 @@ void chunk_grad_kernel(ChunkArgs<T> p) {
     const int blk = blockIdx.y * gridDim.x + blockIdx.x;
     PHASE_CLOCK(p, blk, 0);
 
+    {
+        constexpr int EPL = 16 / (int)sizeof(T), LPR = V / EPL, RPI = 64 / LPR;    // elements/lane, lanes/row, rows/instr
+        const int rr = l / LPR, e = (l % LPR) * EPL;
+        typedef int i32x4 __attribute__((ext_vector_type(4)));
+        auto stage = [&](int m) __attribute__((always_inline)) {
+#pragma unroll
+            for (int r0 = 0; r0 < CH; r0 += RPI) {
+                const int r = r0 + rr;
+                const T* src;
+                if (m == 0) src = p.dout + ((cp.tok0 + min(r, cp.len - 1)) * H + h) * V + e;
+                else if (m == 1) src = p.v + ((cp.tok0 + min(r, cp.len - 1)) * H + h) * V + e;
+                else if (m < 4) src = VN + ((m - 2) * CH + r) * V + e;
+                else src = DVN + ((m - 4) * CH + r) * V + e;
+                i32x4 x = *reinterpret_cast<const i32x4*>(src);
+                if (m < 2 && r >= cp.len) x = (i32x4){0, 0, 0, 0};
+                *reinterpret_cast<i32x4*>(&sTok[(m * CH + r) * VP + e]) = x;
+            }
+        };
+        if (sizeof(T) * V >= 512) {          // 48 wide loads in flight would not fit the register file: one matrix at a time
+#pragma unroll 1
+            for (int m = 0; m < 6; ++m) stage(m);
+        } else {
+#pragma unroll
+            for (int m = 0; m < 6; ++m) stage(m);
+        }
+    }
+    auto tokf = [&](int m, int vt) __attribute__((always_inline)) { return ld_frag(&sTok[(m * CH + c) * VP + 16 * vt + 4 * g]); };
     {
         const float* tmw = p.ws.TM + chw * 1024;
         const int row = l >> 1, c0 = (l & 1) * 16;
@@ -101,10 +132,10 @@ void chunk_grad_kernel(ChunkArgs<T> p) {
     f32x4 dv[VT];
 #pragma unroll
     for (int vt = 0; vt < VT; ++vt) {
-        const Frag<T> doN = ld_frag_sel(p.dout + voff + 16 * vt, rowok);
-        const Frag<T> vN = ld_frag_sel(p.v + voff + 16 * vt, rowok);
-        const Frag<T> vnN[2] = {ld_frag(VN + (0 * CH + c) * V + 16 * vt + 4 * g), ld_frag(VN + (1 * CH + c) * V + 16 * vt + 4 * g)};
-        const Frag<T> dvnN[2] = {ld_frag(DVN + (0 * CH + c) * V + 16 * vt + 4 * g), ld_frag(DVN + (1 * CH + c) * V + 16 * vt + 4 * g)};
+        const Frag<T> doN = tokf(0, vt);
+        const Frag<T> vN = tokf(1, vt);
+        const Frag<T> vnN[2] = {tokf(2, vt), tokf(3, vt)};
+        const Frag<T> dvnN[2] = {tokf(4, vt), tokf(5, vt)};
         dAqk = mm(doN, vN, dAqk);
         dAqb[0] = mm(doN, vnN[0], dAqb[0]);
         dAqb[1] = mm(doN, vnN[1], dAqb[1]);
@@ -142,8 +173,8 @@ void chunk_grad_kernel(ChunkArgs<T> p) {
 #pragma unroll
         for (int vt = 0; vt < VT; ++vt) {
             const Frag<T> Sf = ld_frag(HC + (16 * kt + c) * V + 16 * vt + 4 * g);
-            dwT[0] = mm(Sf, ld_frag(DVN + (0 * CH + c) * V + 16 * vt + 4 * g), dwT[0]);
-            dwT[1] = mm(Sf, ld_frag(DVN + (1 * CH + c) * V + 16 * vt + 4 * g), dwT[1]);
+            dwT[0] = mm(Sf, tokf(4, vt), dwT[0]);
+            dwT[1] = mm(Sf, tokf(5, vt), dwT[1]);
         }
         const Frag<T> dwTf[2] = {to_frag<T>(dwT[0]), to_frag<T>(dwT[1])};
 #pragma unroll
@@ -190,18 +221,18 @@ void chunk_grad_kernel(ChunkArgs<T> p) {
         f32x4 dqg = zero4(), dkg = zero4(), dbg[2] = {zero4(), zero4()};
         f32x4 dwT[2] = {zero4(), zero4()};                 // dw_s^T for this channel tile (rows channel, inner token)
         float hh = 0.f;                                    // partial of sum_v S * dS for channel 16kt + c
-#pragma unroll
+#pragma unroll(sizeof(T) == 2 ? VT : 2)
         for (int vt = 0; vt < VT; ++vt) {
             const Frag<T> Sf = ld_frag(HC + (16 * kt + c) * V + 16 * vt + 4 * g);
             const Frag<T> dSf = ld_frag(DHC + (16 * kt + c) * V + 16 * vt + 4 * g);
-            const Frag<T> doN = ld_frag_sel(p.dout + voff + 16 * vt, rowok);
-            const Frag<T> vN = ld_frag_sel(p.v + voff + 16 * vt, rowok);
+            const Frag<T> doN = tokf(0, vt);
+            const Frag<T> vN = tokf(1, vt);
             dqg = mm(doN, Sf, dqg);
-            dwT[0] = mm(Sf, ld_frag(DVN + (0 * CH + c) * V + 16 * vt + 4 * g), dwT[0]);
-            dwT[1] = mm(Sf, ld_frag(DVN + (1 * CH + c) * V + 16 * vt + 4 * g), dwT[1]);
+            dwT[0] = mm(Sf, tokf(4, vt), dwT[0]);
+            dwT[1] = mm(Sf, tokf(5, vt), dwT[1]);
             dkg = mm(vN, dSf, dkg);
-            dbg[0] = mm(ld_frag(VN + (0 * CH + c) * V + 16 * vt + 4 * g), dSf, dbg[0]);
-            dbg[1] = mm(ld_frag(VN + (1 * CH + c) * V + 16 * vt + 4 * g), dSf, dbg[1]);
+            dbg[0] = mm(tokf(2, vt), dSf, dbg[0]);
+            dbg[1] = mm(tokf(3, vt), dSf, dbg[1]);
             const f32x4 s4 = to_f32(Sf), d4 = to_f32(dSf);
             hh += s4[0] * d4[0] + s4[1] * d4[1] + s4[2] * d4[2] + s4[3] * d4[3];
             dv[vt] = mm(kgf, transpose(dSf, ident), dv[vt]);

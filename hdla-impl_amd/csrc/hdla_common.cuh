@@ -168,6 +168,15 @@ template <typename T> __device__ __forceinline__ Frag<T> ld_pair_one(const T* pa
 template <typename T> __device__ __forceinline__ void st_pair(T* pair, int which, Frag<T> f) {
     st_frag(pair + 8 * lane_id() + 4 * which, f);
 }
+// both tiles of a pair at once: whole 16-byte pieces, so no cache line is ever written in two halves
+__device__ __forceinline__ void st_pair2(bf16* pair, Frag<bf16> f0, Frag<bf16> f1) {
+    const s16x8 x = __builtin_shufflevector(f0.v, f1.v, 0, 1, 2, 3, 4, 5, 6, 7);
+    *reinterpret_cast<s16x8*>(pair + 8 * lane_id()) = x;
+}
+__device__ __forceinline__ void st_pair2(float* pair, Frag<float> f0, Frag<float> f1) {
+    *reinterpret_cast<f32x4*>(pair + 8 * lane_id()) = f0.v;
+    *reinterpret_cast<f32x4*>(pair + 8 * lane_id() + 4) = f1.v;
+}
 
 // gk may be stored as bf16 or fp32 independently of the other inputs (compile-time switch GKF32);
 // same contract as ld_frag_sel: the address is readable on every lane, masked lanes read zero.

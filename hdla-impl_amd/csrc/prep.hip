@@ -13,7 +13,7 @@ namespace hdla {
 constexpr int LDP = 36;   // padded row length of the 32x32 LDS matrices (keeps 16-byte row alignment)
 
 template <typename T, bool GKF32, int K, int V, bool BWD>
-__global__ __launch_bounds__(64) void prep_kernel(ChunkArgs<T> p) {
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 : 1, K == 64 ? 2 : 1))) void prep_kernel(ChunkArgs<T> p) {
     constexpr int KT = K / 16, VT = V / 16, KT2 = KT / 2;
     __shared__ __attribute__((aligned(16))) float sN[32 * LDP];   // A_ab, rank-major
     __shared__ __attribute__((aligned(16))) float sT[32 * LDP];   // (I - A_ab)^-1
@@ -39,19 +39,24 @@ __global__ __launch_bounds__(64) void prep_kernel(ChunkArgs<T> p) {
     f32x4 aqk = zero4(), aqb[2] = {zero4(), zero4()}, aak[2] = {zero4(), zero4()};
     f32x4 aab[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
     f32x4 aqbT[2] = {zero4(), zero4()};
+    // the inputs of the chunk stay in registers (as loaded) for the second use in phase C: the working set of the
+    // resident waves is larger than the L2, so a second load would come from HBM again
+    Frag<T> rq[KT], rk[KT], ra[2][KT], rb[2][KT];
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
         const f32x4 g4 = ld_gk4<GKF32>(p.gk, qoff + 16 * kt, rowok);
+        rq[kt] = ld_frag_sel(p.q + qoff + 16 * kt, rowok);
+        rk[kt] = ld_frag_sel(p.k + qoff + 16 * kt, rowok);
+        ra[0][kt] = ld_frag_sel(p.a + aoff0 + 16 * kt, rowok);
+        ra[1][kt] = ld_frag_sel(p.a + aoff1 + 16 * kt, rowok);
+        rb[0][kt] = ld_frag_sel(p.b + aoff0 + 16 * kt, rowok);
+        rb[1][kt] = ld_frag_sel(p.b + aoff1 + 16 * kt, rowok);
         gi[kt] = scan16_incl(g4);
         ge[kt] = gi[kt] - g4;
         const f32x4 m = bcast16(gi[kt], MID);
         const f32x4 eq = exp4<T>(gi[kt] - m), ek = exp4<T>(m - gi[kt]), ea = exp4<T>(ge[kt] - m);
-        const f32x4 q4 = to_f32(ld_frag_sel(p.q + qoff + 16 * kt, rowok));
-        const f32x4 k4 = to_f32(ld_frag_sel(p.k + qoff + 16 * kt, rowok));
-        const f32x4 a0 = to_f32(ld_frag_sel(p.a + aoff0 + 16 * kt, rowok));
-        const f32x4 a1 = to_f32(ld_frag_sel(p.a + aoff1 + 16 * kt, rowok));
-        const f32x4 b0 = to_f32(ld_frag_sel(p.b + aoff0 + 16 * kt, rowok));
-        const f32x4 b1 = to_f32(ld_frag_sel(p.b + aoff1 + 16 * kt, rowok));
+        const f32x4 q4 = to_f32(rq[kt]), k4 = to_f32(rk[kt]);
+        const f32x4 a0 = to_f32(ra[0][kt]), a1 = to_f32(ra[1][kt]), b0 = to_f32(rb[0][kt]), b1 = to_f32(rb[1][kt]);
         Split<T> qh, kh, ah[2], bh[2];
         split(q4 * eq * scale, qh);
         split(k4 * ek, kh);
@@ -80,11 +85,9 @@ __global__ __launch_bounds__(64) void prep_kernel(ChunkArgs<T> p) {
     }
     if (!BWD) {
         st_tile(p.ws.AQK + chw * TILE, to_frag<T>(aqk));
-        st_pair(p.ws.AQB + chw * PAIR, 0, to_frag<T>(aqb[0]));
-        st_pair(p.ws.AQB + chw * PAIR, 1, to_frag<T>(aqb[1]));
+        st_pair2(p.ws.AQB + chw * PAIR, to_frag<T>(aqb[0]), to_frag<T>(aqb[1]));
     } else {
-        st_pair(p.ws.AQBT + chw * PAIR, 0, to_frag<T>(aqbT[0]));
-        st_pair(p.ws.AQBT + chw * PAIR, 1, to_frag<T>(aqbT[1]));
+        st_pair2(p.ws.AQBT + chw * PAIR, to_frag<T>(aqbT[0]), to_frag<T>(aqbT[1]));
     }
 #pragma unroll
     for (int r = 0; r < 2; ++r)
@@ -139,45 +142,50 @@ __global__ __launch_bounds__(64) void prep_kernel(ChunkArgs<T> p) {
 
     const Frag<T> ident = ident_frag<T>();
 
-    // ---- phase C: w = Tm ag and the gated copies, one channel tile at a time ---------------------------------
+    // ---- phase C: w = Tm ag and the gated copies, two channel tiles (one stored pair) at a time -----------------
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt) {
-        const f32x4 gl = bcast16(gi[kt], CH - 1);
-        const f32x4 egi = exp4<T>(gi[kt]), ege = exp4<T>(ge[kt]), edn = exp4<T>(gl - gi[kt]);
-        const f32x4 q4 = to_f32(ld_frag_sel(p.q + qoff + 16 * kt, rowok));
-        const f32x4 k4 = to_f32(ld_frag_sel(p.k + qoff + 16 * kt, rowok));
-        const f32x4 a0 = to_f32(ld_frag_sel(p.a + aoff0 + 16 * kt, rowok));
-        const f32x4 a1 = to_f32(ld_frag_sel(p.a + aoff1 + 16 * kt, rowok));
-        const f32x4 b0 = to_f32(ld_frag_sel(p.b + aoff0 + 16 * kt, rowok));
-        const f32x4 b1 = to_f32(ld_frag_sel(p.b + aoff1 + 16 * kt, rowok));
-        const Frag<T> agT[2] = {transpose(to_frag<T>(a0 * ege), ident), transpose(to_frag<T>(a1 * ege), ident)};
+    for (int kp = 0; kp < KT2; ++kp) {
+        Frag<T> fw[2][2], fwT[2][2], fkgT[2], fbgT[2][2], fqg[2], fqgT[2], fbg[2][2];   // [..][tile of the pair]
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int kt = 2 * kp + e;
+            const f32x4 gl = bcast16(gi[kt], CH - 1);
+            const f32x4 egi = exp4<T>(gi[kt]), ege = exp4<T>(ge[kt]), edn = exp4<T>(gl - gi[kt]);
+            const Frag<T> agT[2] = {transpose(to_frag<T>(to_f32(ra[0][kt]) * ege), ident),
+                                    transpose(to_frag<T>(to_f32(ra[1][kt]) * ege), ident)};
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                f32x4 w = mm(tm[s][0], agT[0], zero4());
+                w = mm(tm[s][1], agT[1], w);
+                fw[s][e] = to_frag<T>(w);
+                if (BWD) {
+                    f32x4 wT = mm(agT[0], tm[s][0], zero4());
+                    wT = mm(agT[1], tm[s][1], wT);
+                    fwT[s][e] = to_frag<T>(wT);
+                }
+            }
+            fqg[e] = to_frag<T>(to_f32(rq[kt]) * egi * scale);
+            const Frag<T> kg = to_frag<T>(to_f32(rk[kt]) * edn);
+            fbg[0][e] = to_frag<T>(to_f32(rb[0][kt]) * edn);
+            fbg[1][e] = to_frag<T>(to_f32(rb[1][kt]) * edn);
+            fkgT[e] = transpose(kg, ident);
+            fbgT[0][e] = transpose(fbg[0][e], ident);
+            fbgT[1][e] = transpose(fbg[1][e], ident);
+            if (BWD) fqgT[e] = transpose(fqg[e], ident);
+            if (c == 0) *reinterpret_cast<f32x4*>(p.ws.EGL + chw * K + 16 * kt + 4 * g) = exp4<T>(gl);
+        }
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            f32x4 w = zero4();
-            w = mm(tm[s][0], agT[0], w);
-            w = mm(tm[s][1], agT[1], w);
-            st_pair(p.ws.W + ((chw * 2 + s) * KT2 + kt / 2) * PAIR, kt & 1, to_frag<T>(w));
+            st_pair2(p.ws.W + ((chw * 2 + s) * KT2 + kp) * PAIR, fw[s][0], fw[s][1]);
+            st_pair2(p.ws.BGT + ((chw * 2 + s) * KT2 + kp) * PAIR, fbgT[s][0], fbgT[s][1]);
             if (BWD) {
-                f32x4 wT = zero4();
-                wT = mm(agT[0], tm[s][0], wT);
-                wT = mm(agT[1], tm[s][1], wT);
-                st_pair(p.ws.WT + ((chw * 2 + s) * KT2 + kt / 2) * PAIR, kt & 1, to_frag<T>(wT));
+                st_pair2(p.ws.WT + ((chw * 2 + s) * KT2 + kp) * PAIR, fwT[s][0], fwT[s][1]);
+                st_pair2(p.ws.BG + ((chw * 2 + s) * KT2 + kp) * PAIR, fbg[s][0], fbg[s][1]);
             }
         }
-        const Frag<T> qg = to_frag<T>(q4 * egi * scale);
-        const Frag<T> kg = to_frag<T>(k4 * edn);
-        const Frag<T> bg[2] = {to_frag<T>(b0 * edn), to_frag<T>(b1 * edn)};
-        st_pair(p.ws.KGT + (chw * KT2 + kt / 2) * PAIR, kt & 1, transpose(kg, ident));
-        st_pair(p.ws.BGT + ((chw * 2 + 0) * KT2 + kt / 2) * PAIR, kt & 1, transpose(bg[0], ident));
-        st_pair(p.ws.BGT + ((chw * 2 + 1) * KT2 + kt / 2) * PAIR, kt & 1, transpose(bg[1], ident));
-        if (!BWD) {
-            st_pair(p.ws.QG + (chw * KT2 + kt / 2) * PAIR, kt & 1, qg);
-        } else {
-            st_pair(p.ws.QGT + (chw * KT2 + kt / 2) * PAIR, kt & 1, transpose(qg, ident));
-            st_pair(p.ws.BG + ((chw * 2 + 0) * KT2 + kt / 2) * PAIR, kt & 1, bg[0]);
-            st_pair(p.ws.BG + ((chw * 2 + 1) * KT2 + kt / 2) * PAIR, kt & 1, bg[1]);
-        }
-        if (c == 0) *reinterpret_cast<f32x4*>(p.ws.EGL + chw * K + 16 * kt + 4 * g) = exp4<T>(gl);
+        st_pair2(p.ws.KGT + (chw * KT2 + kp) * PAIR, fkgT[0], fkgT[1]);
+        if (!BWD) st_pair2(p.ws.QG + (chw * KT2 + kp) * PAIR, fqg[0], fqg[1]);
+        else st_pair2(p.ws.QGT + (chw * KT2 + kp) * PAIR, fqgT[0], fqgT[1]);
     }
 
     PHASE_CLOCK(p, blk, 3);
@@ -188,13 +196,14 @@ __global__ __launch_bounds__(64) void prep_kernel(ChunkArgs<T> p) {
         const Frag<T> vT = transpose(ld_frag_sel(p.v + voff + 16 * vt, rowok), ident);
         st_tile(p.ws.VTT + (chw * VT + vt) * TILE, vT);
         const Frag<T> mT[2] = {to_frag<T>(mm(vT, aakf[0], zero4())), to_frag<T>(mm(vT, aakf[1], zero4()))};
+        Frag<T> fu[2];
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            f32x4 uT = zero4();
-            uT = mm(mT[0], tm[s][0], uT);
+            f32x4 uT = mm(mT[0], tm[s][0], zero4());
             uT = mm(mT[1], tm[s][1], uT);
-            st_pair(p.ws.UT + (chw * VT + vt) * PAIR, s, to_frag<T>(uT));
+            fu[s] = to_frag<T>(uT);
         }
+        st_pair2(p.ws.UT + (chw * VT + vt) * PAIR, fu[0], fu[1]);
     }
     PHASE_CLOCK(p, blk, 4);
 }
