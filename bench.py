@@ -63,6 +63,26 @@ def interface_bytes(kernel, pass_, K, V, es, gs):
     raise ValueError(kernel)
 
 
+def measured_traffic(workload, kernel_key, K, V):
+    """HBM bytes per launch of one kernel from the committed rocprofv3 counter summary (profiles/hbm_traffic.json:
+    FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the same counter reads for a plain 1 GiB copy), or
+    None when that summary does not cover the kernel.  The counters cannot be collected from inside this script."""
+    try:
+        table = json.load(open(os.path.join(ROOT, "profiles", "hbm_traffic.json"))).get(workload, {})
+    except (OSError, ValueError):
+        return None
+    pass_, name = kernel_key.split(".") if "." in kernel_key else ("", kernel_key)
+    for k, rec in table.items():
+        if not k.startswith(name + "_kernel<") or f" {K}, {V}" not in k:
+            continue
+        if name in ("prep", "scan_fwd"):
+            forward_variant = k.endswith("false>") if name == "prep" else k.endswith("true>")
+            if forward_variant != (pass_ == "fwd"):
+                continue
+        return rec["hbm_bytes_per_launch"]
+    return None
+
+
 def time_steps(fn, steps, warmup):
     for _ in range(warmup):
         fn()
@@ -211,7 +231,7 @@ def main():
                                        "persistent fp32 state", "batch": B, "heads": H, "K": K, "V": V},
                    roofline={"bound": "hbm", "kernel": "recurrent_kernel", "achieved": nbytes / (kms * 1e-3) / 1e9,
                              "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                             "traffic": None, "bytes_per_launch": nbytes, "ms_per_launch": kms})
+                             "traffic": measured_traffic("decode", "recurrent", K, V), "bytes_per_launch": nbytes, "ms_per_launch": kms})
         if not args.no_cpu_baseline:
             res["cpu_baseline"] = cpu_baseline_decode()
         print(json.dumps(res))
@@ -261,7 +281,8 @@ def main():
                                     "varlen": "config 3: chunked fwd+bwd, packed 2048/4096/4096/6144, H=16 K=V=128"}[wl],
                        "global_batch": B, "seq_len": T, "heads": H, "K": K, "V": V, "chunk": 16},
                roofline={"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS,
-                         "unit": "GB/s", "frac": dom["frac_hbm"], "traffic": None,
+                         "unit": "GB/s", "frac": dom["frac_hbm"],
+                         "traffic": measured_traffic("train", dom["kernel"], K, V) if wl == "train" else None,
                          "bytes_per_launch": dom["bytes"], "ms_per_launch": dom["ms"]},
                kernels=klist,
                whole_step={"compulsory_bytes": whole, "GB/s": whole / sec / 1e9, "frac_hbm": whole / sec / 1e9 / HBM_PEAK_GBS,

@@ -207,7 +207,8 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
 
     PHASE_CLOCK(p, blk, 4);
     // ---- second pass over channel tiles: state products, score backward, final gradients ----------------------
-#pragma unroll 1
+    // (two tiles per trip: the two 32-byte pieces a row gets from them leave together as one 64-byte burst)
+#pragma unroll 2
     for (int kt = 0; kt < KT; ++kt) {
         // (a) what the loop over value tiles needs: only kg of this channel tile
         const f32x4 g4 = ld_gk4<GKF32>(p.gk, qoff + 16 * kt, rowok);
