@@ -101,16 +101,21 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     // (the decays are recomputed per channel tile wherever they are needed: a load and four DPP additions cost
     // less than keeping 2*K/16 vector registers alive across the kernel)
     f32x4 aqkT = zero4(), aakT[2] = {zero4(), zero4()};
+    // q, k, a and gk of the chunk stay in registers for their second use in the last pass (a second load would
+    // mostly be a second HBM read); bf16 operands only, fp32 ones would not fit next to the accumulators
+    constexpr bool KEEP = sizeof(T) == 2;
+    Frag<T> rq[KEEP ? KT : 1], rk[KEEP ? KT : 1], ra[2][KEEP ? KT : 1];
+    f32x4 rg[KEEP ? KT : 1];
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
         const f32x4 g4 = ld_gk4<GKF32>(p.gk, qoff + 16 * kt, rowok);
         const f32x4 gi = scan16_incl(g4), ge = gi - g4;
         const f32x4 m = bcast16(gi, MID);
         const f32x4 eq = exp4<T>(gi - m), ek = exp4<T>(m - gi), ea = exp4<T>(ge - m);
-        const f32x4 q4 = to_f32(ld_frag_sel(p.q + qoff + 16 * kt, rowok));
-        const f32x4 k4 = to_f32(ld_frag_sel(p.k + qoff + 16 * kt, rowok));
-        const f32x4 a0 = to_f32(ld_frag_sel(p.a + aoff0 + 16 * kt, rowok));
-        const f32x4 a1 = to_f32(ld_frag_sel(p.a + aoff1 + 16 * kt, rowok));
+        const Frag<T> fq = ld_frag_sel(p.q + qoff + 16 * kt, rowok), fk = ld_frag_sel(p.k + qoff + 16 * kt, rowok);
+        const Frag<T> fa0 = ld_frag_sel(p.a + aoff0 + 16 * kt, rowok), fa1 = ld_frag_sel(p.a + aoff1 + 16 * kt, rowok);
+        if (KEEP) { rq[kt] = fq; rk[kt] = fk; ra[0][kt] = fa0; ra[1][kt] = fa1; rg[kt] = g4; }
+        const f32x4 q4 = to_f32(fq), k4 = to_f32(fk), a0 = to_f32(fa0), a1 = to_f32(fa1);
         const Frag<T> qh = to_frag<T>(q4 * eq * scale), kh = to_frag<T>(k4 * ek);
         aqkT = mm(kh, qh, aqkT);
         aakT[0] = mm(kh, to_frag<T>(a0 * ea), aakT[0]);
@@ -207,15 +212,14 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
 
     PHASE_CLOCK(p, blk, 4);
     // ---- second pass over channel tiles: state products, score backward, final gradients ----------------------
-    // (two tiles per trip: the two 32-byte pieces a row gets from them leave together as one 64-byte burst)
-#pragma unroll 2
+#pragma unroll(KEEP ? KT : 1)
     for (int kt = 0; kt < KT; ++kt) {
         // (a) what the loop over value tiles needs: only kg of this channel tile
-        const f32x4 g4 = ld_gk4<GKF32>(p.gk, qoff + 16 * kt, rowok);
+        const f32x4 g4 = KEEP ? rg[KEEP ? kt : 0] : ld_gk4<GKF32>(p.gk, qoff + 16 * kt, rowok);
         const f32x4 gi = scan16_incl(g4);
         const f32x4 gl = bcast16(gi, CH - 1);
         const f32x4 edn = exp4<T>(gl - gi);
-        const f32x4 k4 = to_f32(ld_frag_sel(p.k + qoff + 16 * kt, rowok));
+        const f32x4 k4 = to_f32(KEEP ? rk[KEEP ? kt : 0] : ld_frag_sel(p.k + qoff + 16 * kt, rowok));
         const f32x4 kg4 = k4 * edn;
         const Frag<T> kgf = to_frag<T>(kg4);
 
@@ -256,8 +260,9 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         const f32x4 m = bcast16(gi, MID);
         const f32x4 eq = exp4<T>(gi - m), ek = exp4<T>(m - gi), ea = exp4<T>(ge - m);
         const f32x4 egi = exp4<T>(gi), ege = exp4<T>(ge);
-        const f32x4 q4 = to_f32(ld_frag_sel(p.q + qoff + 16 * kt, rowok));
-        const f32x4 a4[2] = {to_f32(ld_frag_sel(p.a + aoff0 + 16 * kt, rowok)), to_f32(ld_frag_sel(p.a + aoff1 + 16 * kt, rowok))};
+        const f32x4 q4 = to_f32(KEEP ? rq[KEEP ? kt : 0] : ld_frag_sel(p.q + qoff + 16 * kt, rowok));
+        const f32x4 a4[2] = {to_f32(KEEP ? ra[0][KEEP ? kt : 0] : ld_frag_sel(p.a + aoff0 + 16 * kt, rowok)),
+                             to_f32(KEEP ? ra[1][KEEP ? kt : 0] : ld_frag_sel(p.a + aoff1 + 16 * kt, rowok))};
         const f32x4 b4[2] = {to_f32(ld_frag_sel(p.b + aoff0 + 16 * kt, rowok)), to_f32(ld_frag_sel(p.b + aoff1 + 16 * kt, rowok))};
         const Frag<T> qhT = transpose(to_frag<T>(q4 * eq * scale), ident), khT = transpose(to_frag<T>(k4 * ek), ident);
         const Frag<T> ahT[2] = {transpose(to_frag<T>(a4[0] * ea), ident), transpose(to_frag<T>(a4[1] * ea), ident)};
