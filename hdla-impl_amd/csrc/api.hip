@@ -47,21 +47,19 @@ int make_layout(const hdla_dims* d, int pass, WsLayout& L, int& nch) {
     size_t off = 0;
     auto take = [&](size_t bytes) { const size_t o = off; off += up256(bytes); return o; };
     L = WsLayout{};
-    L.W = take(chw * 2 * K * 16 * es);
+    const BlkF bf = blk_fwd(d->K, (int)es, pass == 0);
+    const size_t sa = take(chw * (size_t)bf.SIZE);
+    L.SA_STRIDE = bf.SIZE;
+    L.W = sa + bf.W; L.BGT = sa + bf.BGT; L.KGT = sa + bf.KGT; L.EGL = sa + bf.EGL;
     L.UT = take(chw * 2 * V * 16 * es);
-    L.KGT = take(chw * K * 16 * es);
-    L.BGT = take(chw * 2 * K * 16 * es);
     L.VTT = take(chw * V * 16 * es);
-    L.EGL = take(chw * K * 4);
     if (pass == 0) {
-        L.QG = take(chw * K * 16 * es);
-        L.AQK = take(chw * 256 * es);
-        L.AQB = take(chw * 2 * 256 * es);
+        L.QG = sa + bf.QG; L.AQB = sa + bf.AQB; L.AQK = sa + bf.AQK;
     } else {
-        L.AQBT = take(chw * 2 * 256 * es);
-        L.BG = take(chw * 2 * K * 16 * es);
-        L.WT = take(chw * 2 * K * 16 * es);
-        L.QGT = take(chw * K * 16 * es);
+        const BlkB bb = blk_bwd(d->K, (int)es);
+        const size_t sb = take(chw * (size_t)bb.SIZE);
+        L.SB_STRIDE = bb.SIZE;
+        L.BG = sb + bb.BG; L.WT = sb + bb.WT; L.QGT = sb + bb.QGT; L.AQBT = sb + bb.AQBT; L.EGLB = sb + bb.EGL;
         L.TM = take(chw * 1024 * 4);
         L.HC = take(chw * K * V * es);
         L.DHC = take(chw * K * V * es);
@@ -85,6 +83,7 @@ void bind_ws(ChunkArgs<T>& a, const hdla_dims* d, const WsLayout& L, int nch, vo
     a.ws.AQBT = at(L.AQBT); a.ws.BG = at(L.BG); a.ws.WT = at(L.WT); a.ws.QGT = at(L.QGT);
     a.ws.HC = at(L.HC); a.ws.DHC = at(L.DHC); a.ws.VN = at(L.VN); a.ws.DVN = at(L.DVN);
     a.ws.EGL = reinterpret_cast<float*>(base + L.EGL);
+    a.ws.EGLB = reinterpret_cast<float*>(base + L.EGLB);
     a.ws.TM = reinterpret_cast<float*>(base + L.TM);
     a.st.cu = d->cu_seqlens;
     a.st.chunk_off = d->cu_seqlens ? reinterpret_cast<const int32_t*>(base + L.CHUNK_OFF) : nullptr;
@@ -185,6 +184,7 @@ int hdla_workspace_layout(const hdla_dims* dims, int pass, hdla_ws_layout* out) 
     out->W = L.W; out->UT = L.UT; out->KGT = L.KGT; out->BGT = L.BGT; out->VTT = L.VTT; out->EGL = L.EGL;
     out->QG = L.QG; out->AQK = L.AQK; out->AQB = L.AQB;
     out->AQBT = L.AQBT; out->BG = L.BG; out->WT = L.WT; out->QGT = L.QGT; out->TM = L.TM;
+    out->EGLB = L.EGLB; out->SA_STRIDE = L.SA_STRIDE; out->SB_STRIDE = L.SB_STRIDE;
     out->HC = L.HC; out->DHC = L.DHC; out->VN = L.VN; out->DVN = L.DVN;
     out->CHUNK_OFF = L.CHUNK_OFF; out->CHUNK_SEQ = L.CHUNK_SEQ;
     out->total = L.total;

@@ -22,6 +22,7 @@ constexpr int LDG = 36;
 template <typename T, bool GKF32, int K, int V>
 __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     constexpr int KT = K / 16, VT = V / 16;
+    constexpr int SFS = blk_fwd(K, sizeof(T), false).SIZE / (int)sizeof(T);   // elements between slots of the scan block
     __shared__ __attribute__((aligned(16))) float sT[32 * LDG];   // (I - A_ab)^-1, rank-major
     // do, v, v_new (2 ranks) and dv_new (2 ranks) of the chunk, [matrix][token][value], staged once: every one of
     // them is an operand of several products in every pass, and the working set of the resident waves is far
@@ -49,30 +50,34 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     const int blk = blockIdx.y * gridDim.x + blockIdx.x;
     PHASE_CLOCK(p, blk, 0);
 
+    const Frag<T> ident = ident_frag<T>();
     {
+        // do and v: rows of the original tensors, 16 bytes per lane
         constexpr int EPL = 16 / (int)sizeof(T), LPR = V / EPL, RPI = 64 / LPR;    // elements/lane, lanes/row, rows/instr
         const int rr = l / LPR, e = (l % LPR) * EPL;
         typedef int i32x4 __attribute__((ext_vector_type(4)));
-        auto stage = [&](int m) __attribute__((always_inline)) {
+#pragma unroll
+        for (int m = 0; m < 2; ++m)
 #pragma unroll
             for (int r0 = 0; r0 < CH; r0 += RPI) {
                 const int r = r0 + rr;
-                const T* src;
-                if (m == 0) src = p.dout + ((cp.tok0 + min(r, cp.len - 1)) * H + h) * V + e;
-                else if (m == 1) src = p.v + ((cp.tok0 + min(r, cp.len - 1)) * H + h) * V + e;
-                else if (m < 4) src = VN + ((m - 2) * CH + r) * V + e;
-                else src = DVN + ((m - 4) * CH + r) * V + e;
+                const T* src = (m == 0 ? p.dout : p.v) + ((cp.tok0 + min(r, cp.len - 1)) * H + h) * V + e;
                 i32x4 x = *reinterpret_cast<const i32x4*>(src);
-                if (m < 2 && r >= cp.len) x = (i32x4){0, 0, 0, 0};
+                if (r >= cp.len) x = (i32x4){0, 0, 0, 0};
                 *reinterpret_cast<i32x4*>(&sTok[(m * CH + r) * VP + e]) = x;
             }
-        };
-        if (sizeof(T) * V >= 512) {          // 48 wide loads in flight would not fit the register file: one matrix at a time
-#pragma unroll 1
-            for (int m = 0; m < 6; ++m) stage(m);
-        } else {
-#pragma unroll
-            for (int m = 0; m < 6; ++m) stage(m);
+        // v_new and dv_new: the scans left them as fragments of the transposed tiles (rows value, inner token), the
+        // two ranks of a value tile paired; one transposing product each gives the rows
+#pragma unroll(sizeof(T) * V >= 512 ? 1 : VT)
+        for (int vt = 0; vt < VT; ++vt) {
+            Frag<T> x0, x1, y0, y1;
+            ld_pair(VN + vt * PAIR, x0, x1);
+            ld_pair(DVN + vt * PAIR, y0, y1);
+            T* dst = &sTok[c * VP + 16 * vt + 4 * g];
+            st_frag(dst + 2 * CH * VP, transpose(x0, ident));
+            st_frag(dst + 3 * CH * VP, transpose(x1, ident));
+            st_frag(dst + 4 * CH * VP, transpose(y0, ident));
+            st_frag(dst + 5 * CH * VP, transpose(y1, ident));
         }
     }
     auto tokf = [&](int m, int vt) __attribute__((always_inline)) { return ld_frag(&sTok[(m * CH + c) * VP + 16 * vt + 4 * g]); };
@@ -95,7 +100,6 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
             for (int i = 0; i < 4; ++i) t[i] = sT[(16 * s + 4 * g + i) * LDG + 16 * r + c];
             tmT[s][r] = to_frag<T>(t);
         }
-    const Frag<T> ident = ident_frag<T>();
 
     // ---- cumulative decays; A_qk^T and A_ak^T (rows j, inner i) -----------------------------------------------
     // (the decays are recomputed per channel tile wherever they are needed: a load and four DPP additions cost
@@ -140,12 +144,12 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         const Frag<T> doN = tokf(0, vt);
         const Frag<T> vN = tokf(1, vt);
         const Frag<T> vnN[2] = {tokf(2, vt), tokf(3, vt)};
-        const Frag<T> dvnN[2] = {tokf(4, vt), tokf(5, vt)};
         dAqk = mm(doN, vN, dAqk);
         dAqb[0] = mm(doN, vnN[0], dAqb[0]);
         dAqb[1] = mm(doN, vnN[1], dAqb[1]);
         const Frag<T> doT = transpose(doN, ident);
-        const Frag<T> dvnT[2] = {transpose(dvnN[0], ident), transpose(dvnN[1], ident)};
+        Frag<T> dvnT[2];                                  // as the reverse scan left them: rows value, inner token
+        ld_pair(DVN + vt * PAIR, dvnT[0], dvnT[1]);
         Frag<T> dMf[2], dMTf[2];
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
@@ -177,7 +181,7 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         f32x4 dwT[2] = {zero4(), zero4()};                // rows channel, inner token
 #pragma unroll
         for (int vt = 0; vt < VT; ++vt) {
-            const Frag<T> Sf = ld_frag(HC + (16 * kt + c) * V + 16 * vt + 4 * g);
+            const Frag<T> Sf = transpose(ld_pair_one(HC + ((kt / 2) * VT + vt) * PAIR, kt & 1), ident);
             dwT[0] = mm(Sf, tokf(4, vt), dwT[0]);
             dwT[1] = mm(Sf, tokf(5, vt), dwT[1]);
         }
@@ -187,8 +191,8 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
             f32x4 x = mm(tmT[0][r], dwTf[0], zero4());
             x = mm(tmT[1][r], dwTf[1], x);                // dag_r: rows token, inner channel
             const Frag<T> dagf = to_frag<T>(x);
-            dAab[r][0] = mm(dagf, ld_pair_one(p.ws.W + ((chw * 2 + 0) * (KT / 2) + kt / 2) * PAIR, kt & 1), dAab[r][0]);
-            dAab[r][1] = mm(dagf, ld_pair_one(p.ws.W + ((chw * 2 + 1) * (KT / 2) + kt / 2) * PAIR, kt & 1), dAab[r][1]);
+            dAab[r][0] = mm(dagf, ld_pair_one(p.ws.W + chw * SFS + (0 * (KT / 2) + kt / 2) * PAIR, kt & 1), dAab[r][0]);
+            dAab[r][1] = mm(dagf, ld_pair_one(p.ws.W + chw * SFS + (1 * (KT / 2) + kt / 2) * PAIR, kt & 1), dAab[r][1]);
         }
     }
 
@@ -228,8 +232,10 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         float hh = 0.f;                                    // partial of sum_v S * dS for channel 16kt + c
 #pragma unroll(sizeof(T) == 2 ? VT : 2)
         for (int vt = 0; vt < VT; ++vt) {
-            const Frag<T> Sf = ld_frag(HC + (16 * kt + c) * V + 16 * vt + 4 * g);
-            const Frag<T> dSf = ld_frag(DHC + (16 * kt + c) * V + 16 * vt + 4 * g);
+            // the scans checkpoint S and dS as fragments of the transposed tiles (rows value, inner channel)
+            const Frag<T> dST = ld_pair_one(DHC + ((kt / 2) * VT + vt) * PAIR, kt & 1);
+            const Frag<T> Sf = transpose(ld_pair_one(HC + ((kt / 2) * VT + vt) * PAIR, kt & 1), ident);
+            const Frag<T> dSf = transpose(dST, ident);
             const Frag<T> doN = tokf(0, vt);
             const Frag<T> vN = tokf(1, vt);
             dqg = mm(doN, Sf, dqg);
@@ -240,7 +246,7 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
             dbg[1] = mm(tokf(3, vt), dSf, dbg[1]);
             const f32x4 s4 = to_f32(Sf), d4 = to_f32(dSf);
             hh += s4[0] * d4[0] + s4[1] * d4[1] + s4[2] * d4[2] + s4[3] * d4[3];
-            dv[vt] = mm(kgf, transpose(dSf, ident), dv[vt]);
+            dv[vt] = mm(kgf, dST, dv[vt]);
         }
         hh += __shfl_xor(hh, 16);
         hh += __shfl_xor(hh, 32);

@@ -23,7 +23,35 @@ struct SeqTab {
     int nch;                  // chunk slots the workspace is laid out for (an upper bound with cu_seqlens)
 };
 
-// Byte offsets into the caller's workspace; 0-sized entries are unused in the given pass.
+// Operands of the state scans that all value-column blocks of a (chunk, head) share are kept in ONE contiguous
+// block per (chunk, head), so that a workgroup can copy a block into LDS with a few whole-kilobyte loads.
+// Byte offsets inside a block, by head size K, element size es and pass:
+//   forward-scan block:  W [2][K/16] | BGT [2][K/16] | KGT [K/16] | (QG [K/16] | AQB [2] | AQK [1]) | EGL fp32[K]
+//   reverse-scan block:  BG [2][K/16] | WT [2][K/16] | QGT [K/16] | AQBT [2] | EGL fp32[K]
+// (tiles of 256 elements in fragment order, consecutive tile pairs interleaved; the part in parentheses only in
+// the forward pass, where the scan also produces the output)
+struct BlkF { int W, BGT, KGT, QG, AQB, AQK, EGL, SIZE; };
+struct BlkB { int BG, WT, QGT, AQBT, EGL, SIZE; };
+constexpr BlkF blk_fwd(int K, int es, bool with_o) {
+    const int tb = 256 * es, KT = K / 16;
+    BlkF b{};
+    b.W = 0; b.BGT = 2 * KT * tb; b.KGT = 4 * KT * tb;
+    if (with_o) { b.QG = 5 * KT * tb; b.AQB = 6 * KT * tb; b.AQK = (6 * KT + 2) * tb; b.EGL = (6 * KT + 3) * tb; }
+    else { b.QG = 0; b.AQB = 0; b.AQK = 0; b.EGL = 5 * KT * tb; }
+    b.SIZE = (b.EGL + 4 * K + 1023) & ~1023;
+    return b;
+}
+constexpr BlkB blk_bwd(int K, int es) {
+    const int tb = 256 * es, KT = K / 16;
+    BlkB b{};
+    b.BG = 0; b.WT = 2 * KT * tb; b.QGT = 4 * KT * tb; b.AQBT = 5 * KT * tb; b.EGL = (5 * KT + 2) * tb;
+    b.SIZE = (b.EGL + 4 * K + 1023) & ~1023;
+    return b;
+}
+
+// Byte offsets into the caller's workspace; 0-sized entries are unused in the given pass.  The entries of the
+// two scan blocks (W .. EGL and BG .. EGLB) are the offsets of that part for (chunk, head) slot 0; consecutive
+// slots are SA_STRIDE / SB_STRIDE bytes apart.
 struct WsLayout {
     // written by prep, read by the scans
     size_t W;      // tiles  [2][K/16]   F(w_s)        rows token, inner channel
@@ -41,6 +69,8 @@ struct WsLayout {
     size_t BG;     // tiles  [2][K/16]   F(bg_s)       rows token, inner channel
     size_t WT;     // tiles  [2][K/16]   F(w_s^T)      rows channel, inner token
     size_t QGT;    // tiles  [K/16]      F(qg^T)       rows channel, inner token
+    size_t EGLB;   // fp32   [K]         exp(g_last), copy inside the reverse-scan block
+    size_t SA_STRIDE, SB_STRIDE;   // bytes between consecutive (chunk, head) slots of the two scan blocks
     size_t TM;     // fp32   [32][32]    (I - A_ab)^-1 in rank-major order (row r*16+i, column s*16+j)
     size_t HC;     // rows   [K][V]      state entering the chunk
     size_t DHC;    // rows   [K][V]      gradient of the state leaving the chunk
@@ -55,7 +85,7 @@ struct WsLayout {
 template <typename T>
 struct Ws {
     T *W, *UT, *KGT, *BGT, *VTT, *QG, *AQK, *AQB, *AQBT, *BG, *WT, *QGT, *HC, *DHC, *VN, *DVN;
-    float *EGL, *TM;
+    float *EGL, *EGLB, *TM;
 };
 
 template <typename T>

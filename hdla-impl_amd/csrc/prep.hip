@@ -15,6 +15,8 @@ constexpr int LDP = 36;   // padded row length of the 32x32 LDS matrices (keeps 
 template <typename T, bool GKF32, int K, int V, bool BWD>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 : 1, K == 64 ? 2 : 1))) void prep_kernel(ChunkArgs<T> p) {
     constexpr int KT = K / 16, VT = V / 16, KT2 = KT / 2;
+    constexpr int SAS = blk_fwd(K, sizeof(T), !BWD).SIZE / (int)sizeof(T);   // elements between (chunk, head) slots
+    constexpr int SBS = blk_bwd(K, sizeof(T)).SIZE / (int)sizeof(T);
     __shared__ __attribute__((aligned(16))) float sN[32 * LDP];   // A_ab, rank-major
     __shared__ __attribute__((aligned(16))) float sT[32 * LDP];   // (I - A_ab)^-1
 
@@ -84,10 +86,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 
         if (!tle) { aqbT[0][i] = 0.f; aqbT[1][i] = 0.f; }
     }
     if (!BWD) {
-        st_tile(p.ws.AQK + chw * TILE, to_frag<T>(aqk));
-        st_pair2(p.ws.AQB + chw * PAIR, to_frag<T>(aqb[0]), to_frag<T>(aqb[1]));
+        st_tile(p.ws.AQK + chw * SAS, to_frag<T>(aqk));
+        st_pair2(p.ws.AQB + chw * SAS, to_frag<T>(aqb[0]), to_frag<T>(aqb[1]));
     } else {
-        st_pair2(p.ws.AQBT + chw * PAIR, to_frag<T>(aqbT[0]), to_frag<T>(aqbT[1]));
+        st_pair2(p.ws.AQBT + chw * SBS, to_frag<T>(aqbT[0]), to_frag<T>(aqbT[1]));
     }
 #pragma unroll
     for (int r = 0; r < 2; ++r)
@@ -172,20 +174,24 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 
             fbgT[0][e] = transpose(fbg[0][e], ident);
             fbgT[1][e] = transpose(fbg[1][e], ident);
             if (BWD) fqgT[e] = transpose(fqg[e], ident);
-            if (c == 0) *reinterpret_cast<f32x4*>(p.ws.EGL + chw * K + 16 * kt + 4 * g) = exp4<T>(gl);
+            if (c == 0) {
+                const f32x4 egl = exp4<T>(gl);
+                *reinterpret_cast<f32x4*>(p.ws.EGL + chw * (SAS * (int)sizeof(T) / 4) + 16 * kt + 4 * g) = egl;
+                if (BWD) *reinterpret_cast<f32x4*>(p.ws.EGLB + chw * (SBS * (int)sizeof(T) / 4) + 16 * kt + 4 * g) = egl;
+            }
         }
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            st_pair2(p.ws.W + ((chw * 2 + s) * KT2 + kp) * PAIR, fw[s][0], fw[s][1]);
-            st_pair2(p.ws.BGT + ((chw * 2 + s) * KT2 + kp) * PAIR, fbgT[s][0], fbgT[s][1]);
+            st_pair2(p.ws.W + chw * SAS + (s * KT2 + kp) * PAIR, fw[s][0], fw[s][1]);
+            st_pair2(p.ws.BGT + chw * SAS + (s * KT2 + kp) * PAIR, fbgT[s][0], fbgT[s][1]);
             if (BWD) {
-                st_pair2(p.ws.WT + ((chw * 2 + s) * KT2 + kp) * PAIR, fwT[s][0], fwT[s][1]);
-                st_pair2(p.ws.BG + ((chw * 2 + s) * KT2 + kp) * PAIR, fbg[s][0], fbg[s][1]);
+                st_pair2(p.ws.WT + chw * SBS + (s * KT2 + kp) * PAIR, fwT[s][0], fwT[s][1]);
+                st_pair2(p.ws.BG + chw * SBS + (s * KT2 + kp) * PAIR, fbg[s][0], fbg[s][1]);
             }
         }
-        st_pair2(p.ws.KGT + (chw * KT2 + kp) * PAIR, fkgT[0], fkgT[1]);
-        if (!BWD) st_pair2(p.ws.QG + (chw * KT2 + kp) * PAIR, fqg[0], fqg[1]);
-        else st_pair2(p.ws.QGT + (chw * KT2 + kp) * PAIR, fqgT[0], fqgT[1]);
+        st_pair2(p.ws.KGT + chw * SAS + kp * PAIR, fkgT[0], fkgT[1]);
+        if (!BWD) st_pair2(p.ws.QG + chw * SAS + kp * PAIR, fqg[0], fqg[1]);
+        else st_pair2(p.ws.QGT + chw * SBS + kp * PAIR, fqgT[0], fqgT[1]);
     }
 
     PHASE_CLOCK(p, blk, 3);

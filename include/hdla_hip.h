@@ -62,11 +62,15 @@ typedef struct hdla_dims {
 
 /* Byte offsets of the named intermediates inside the workspace (0 = not part of this pass); for tests and
  * debugging: after hdla_chunk_bwd every stage's output is still there.  "tiles" are 16x16 blocks in MFMA
- * fragment order (element 4*lane + i of a block is row lane%16, inner index 4*(lane/16) + i), laid out
- * [H][nch][...]; "rows" are row-major. */
+ * fragment order (element 4*lane + i of a block is row lane%16, inner index 4*(lane/16) + i; consecutive
+ * tile pairs are stored interleaved, element 8*lane + 4*which + i), "rows" are row-major, all laid out
+ * [H][nch][...].  W, BGT, KGT, QG, AQB, AQK, EGL are parts of one block per (head, chunk) slot: the value given
+ * is the offset for slot 0 and consecutive slots are SA_STRIDE bytes apart; likewise BG, WT, QGT, AQBT, EGLB
+ * with SB_STRIDE. */
 typedef struct hdla_ws_layout {
     int64_t nch;               /* chunk slots per head */
     int64_t W, UT, KGT, BGT, VTT, EGL, QG, AQK, AQB, AQBT, BG, WT, QGT, TM, HC, DHC, VN, DVN;
+    int64_t EGLB, SA_STRIDE, SB_STRIDE;
     int64_t CHUNK_OFF, CHUNK_SEQ;
     int64_t total;
 } hdla_ws_layout;

@@ -2,32 +2,38 @@
 import torch
 
 
-def _raw(ws: torch.Tensor, off: int, count: int, dtype: torch.dtype) -> torch.Tensor:
+def _raw(ws: torch.Tensor, off: int, count: int, dtype: torch.dtype, stride: int = 0, slots: int = 1) -> torch.Tensor:
+    """`count` elements at byte offset `off`; with `stride`, they are `slots` equal pieces `stride` bytes apart
+    (the parts of the scan operand blocks, one block per (head, chunk) slot)."""
     nbytes = count * torch.empty((), dtype=dtype).element_size()
-    return ws[off:off + nbytes].view(dtype)
+    if not stride:
+        return ws[off:off + nbytes].view(dtype)
+    assert nbytes % slots == 0 and nbytes // slots <= stride
+    return torch.as_strided(ws, (slots, nbytes // slots), (stride, 1), off).contiguous().view(-1).view(dtype)
 
 
-def tiles(ws, off, dtype, H, nch, *lead):
+def tiles(ws, off, dtype, H, nch, *lead, stride=0):
     """Buffer of 16x16 tiles in fragment order -> float64 tensor [H, nch, *lead, 16 (row), 16 (inner)].
 
     Element 4*lane + i of a tile is row lane % 16, inner index 4*(lane // 16) + i."""
     n = 1
     for x in lead:
         n *= x
-    t = _raw(ws, off, H * nch * n * 256, dtype).double().reshape(H, nch, *lead, 4, 16, 4)   # [g][c][i]
+    t = _raw(ws, off, H * nch * n * 256, dtype, stride, H * nch).double().reshape(H, nch, *lead, 4, 16, 4)   # [g][c][i]
     nd = t.dim()
     t = t.transpose(nd - 3, nd - 2)                                                          # [c][g][i]
     return t.reshape(H, nch, *lead, 16, 16).cpu()
 
 
-def pair_tiles(ws, off, dtype, H, nch, *lead):
+def pair_tiles(ws, off, dtype, H, nch, *lead, stride=0):
     """Like tiles(), for buffers whose tiles are stored interleaved in pairs along the last lead dimension:
     element 8*lane + 4*which + i of a 512-element pair block belongs to tile `which` of the pair."""
     n = 1
     for x in lead:
         n *= x
     assert lead[-1] % 2 == 0
-    t = _raw(ws, off, H * nch * n * 256, dtype).double().reshape(H, nch, *lead[:-1], lead[-1] // 2, 64, 2, 4)
+    t = _raw(ws, off, H * nch * n * 256, dtype, stride, H * nch).double()
+    t = t.reshape(H, nch, *lead[:-1], lead[-1] // 2, 64, 2, 4)
     nd = t.dim()
     t = t.transpose(nd - 3, nd - 2)                                   # [npairs, 2, 64, 4]
     t = t.reshape(H, nch, *lead, 4, 16, 4)
@@ -36,11 +42,11 @@ def pair_tiles(ws, off, dtype, H, nch, *lead):
     return t.reshape(H, nch, *lead, 16, 16).cpu()
 
 
-def rows(ws, off, dtype, H, nch, *shape):
+def rows(ws, off, dtype, H, nch, *shape, stride=0):
     n = 1
     for x in shape:
         n *= x
-    return _raw(ws, off, H * nch * n, dtype).double().reshape(H, nch, *shape).cpu()
+    return _raw(ws, off, H * nch * n, dtype, stride, H * nch).double().reshape(H, nch, *shape).cpu()
 
 
 def cat_tiles(t, dim_tiles, transpose=False):
