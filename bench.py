@@ -57,6 +57,8 @@ def interface_bytes(kernel, pass_, K, V, es, gs):
         return rd + (QG + AQK + AQB + 16 * V * es if pass_ == 0 else HC + VN)
     if kernel == "scan_bwd":
         return AQBT + BG + WT + QGT + EGL + 16 * V * es + DHC + DVN
+    if kernel == "scan_pair":           # both scans of the backward pass in one launch
+        return interface_bytes("scan_fwd", 1, K, V, es, gs) + interface_bytes("scan_bwd", 1, K, V, es, gs)
     if kernel == "chunk_grad":
         outs = 2 * 16 * K * es + 16 * K * gs + 2 * 32 * K * es + 16 * V * es
         return inputs + 16 * V * es + TM + W + UT + HC + DHC + VN + DVN + outs
@@ -102,8 +104,8 @@ def stage_times(inp_dev, dims_kw, pass_, steps, outputs):
     dims = _lib.make_dims(**dims_kw)
     ws = _lib.workspace(dims, pass_, q.device)
     P = _lib.ptr
-    names = {1: "prep", 2: "scan_fwd", 4: "scan_bwd", 8: "chunk_grad"}
-    masks = [1, 2] if pass_ == 0 else [1, 2, 4, 8]
+    names = {1: "prep", 2: "scan_fwd", 6: "scan_pair", 8: "chunk_grad"}
+    masks = [1, 2] if pass_ == 0 else [1, 6, 8]            # the library runs the two backward scans as one launch
     o, ht, dq, dk, dv, da, db, dgk, dh0 = outputs
     stream = _lib.current_stream(q.device)
     acc = {m: 0.0 for m in masks}

@@ -128,12 +128,17 @@ int run_chunk(const hdla_dims* d, int pass, const void* q, const void* k, const 
         e = launch_prep<T>(a, d->K, d->V, pass == 1, stream);
         if (e != hipSuccess) return (int)e;
     }
-    if (stages & HDLA_STAGE_SCAN_FWD) {
+    // the two scans of the backward pass are independent of each other: one launch when both are asked for
+    const bool pair = pass == 1 && (stages & HDLA_STAGE_SCAN_FWD) && (stages & HDLA_STAGE_SCAN_BWD);
+    if (pair) {
+        e = launch_scan_pair<T>(a, d->K, d->V, stream);
+        if (e != hipSuccess) return (int)e;
+    } else if (stages & HDLA_STAGE_SCAN_FWD) {
         e = launch_scan_fwd<T>(a, d->K, d->V, pass == 0, stream);
         if (e != hipSuccess) return (int)e;
     }
     if (pass == 1) {
-        if (stages & HDLA_STAGE_SCAN_BWD) {
+        if (!pair && (stages & HDLA_STAGE_SCAN_BWD)) {
             e = launch_scan_bwd<T>(a, d->K, d->V, stream);
             if (e != hipSuccess) return (int)e;
         }

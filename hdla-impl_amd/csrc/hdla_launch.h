@@ -12,6 +12,8 @@ hipError_t launch_chunk_table(const int64_t* cu, int N, int nch, int32_t* chunk_
 template <typename T> hipError_t launch_prep(const ChunkArgs<T>& a, int K, int V, bool bwd, hipStream_t stream);
 template <typename T> hipError_t launch_scan_fwd(const ChunkArgs<T>& a, int K, int V, bool write_o, hipStream_t stream);
 template <typename T> hipError_t launch_scan_bwd(const ChunkArgs<T>& a, int K, int V, hipStream_t stream);
+// both scans of the backward pass (scan_fwd without the output, scan_bwd) in one launch
+template <typename T> hipError_t launch_scan_pair(const ChunkArgs<T>& a, int K, int V, hipStream_t stream);
 template <typename T> hipError_t launch_chunk_grad(const ChunkArgs<T>& a, int K, int V, hipStream_t stream);
 template <typename T> hipError_t launch_recurrent(const RecurrentArgs<T>& a, int K, int V, hipStream_t stream);
 

@@ -6,16 +6,33 @@
 // dh0) fused with the dv_new part of HRDPLR/bwd_triton.py:30-105.
 //
 // One workgroup per (sequence, head), one wavefront per 16-column block of the fp32 state.  A wave keeps its
-// K x 16 block in MFMA accumulators as the row fragment of S^T (rows = value column, inner = channel), which is
-// at once the operand layout of the next product: w S, qg S and the rank updates chain through registers with
-// no cross-lane movement.
+// K x 16 block in registers as the row fragment of S^T (rows = value column, inner = channel), which is at once
+// the operand layout of the next product: w S, qg S and the rank updates chain through registers with no
+// cross-lane movement.
 //
 // What bounds a step is not arithmetic but operand delivery: a wave may have at most 63 memory instructions in
 // flight, and every wave of a head needs the same w / kg / bg / qg tiles.  So the waves of a workgroup split the
 // chunk's shared operand block (one contiguous block per chunk, written by the prep kernel) between them:
-// each wave fetches its share of the block of chunk c+6 into registers (16 bytes per lane, a few instructions),
-// hands the share of chunk c+1 to LDS, and all waves read the operands of chunk c from LDS.  One LDS-only
-// barrier per chunk; global loads stay in flight across it.
+// each wave fetches its share of the blocks of the next few chunks into registers (16 bytes per lane, a few
+// instructions per chunk) and hands them to LDS two chunks ahead of their use; all waves read their operands
+// from LDS.  Three LDS slots rotate, with ONE LDS-only barrier per chunk (global loads stay in flight across it):
+//
+//   step t:  barrier                      block t+1 (written during step t-1) becomes visible
+//            share of block t+2 -> slot (t+2) % 3          (its last readers finished before the barrier)
+//            read the operands of the state update of chunk t from slot t % 3
+//            phase 1: v_new (operands already in registers, read during step t-1)
+//            read the phase-1 operands of chunk t+1 from slot (t+1) % 3
+//            phase 2: state update
+//
+// so every LDS read has a phase of matrix products between its issue and its first use.
+//
+// Stores go through LDS as well, to waves that do nothing else ("store waves").  Memory instructions of one wave
+// complete in order, and the acknowledgement of a store takes several times as long as a load takes to return
+// (much longer still right after a kernel that left the L2 full of dirty lines, as the prep kernel does): a wave
+// that both stores its results and waits for prefetched operands ends up waiting for its own stores.  The
+// computing waves therefore leave a chunk's results in an LDS outbox laid out like the chunk's record in global
+// memory, and the store waves copy the outbox of the previous chunk out while the next chunk is computed; they
+// never wait for anything but the per-chunk barrier.
 #include "hdla_common.cuh"
 #include "hdla_launch.h"
 
@@ -30,25 +47,27 @@ __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-// depth of the register ring of operand shares: enough chunks in flight to cover the memory latency
+constexpr int NSLOT = 3;
+
 template <typename T, int K, int V> struct ScanCfg {
-    static constexpr int NW = V / 16;                                            // wavefronts per workgroup
-    static constexpr int DR = (sizeof(T) == 2 && NW == 4 && K == 64) ? 6 : (sizeof(T) == 2 || K == 64) ? 4 : 2;
-    // whether the ring also carries the wave's own u and v tiles; the largest fp32 shape has no registers left
-    // for them and loads them where they are used
-    static constexpr bool RING_OWN = !(sizeof(T) == 4 && K == 128 && V == 128);
-    // When a step reads its shared operands from LDS.  2: all of them before the first product; 1: those of the
-    // state update only once the products of v_new are issued; 0: wherever the compiler puts them (shapes whose
-    // registers allow nothing else).  KB = bytes of one operand row; with_o = the scan also produces the output.
-    static constexpr int read_mode(bool with_o) {
-        constexpr int KB = K * (int)sizeof(T);
-        if (KB <= 128) return 2;
-        if (KB >= 512 || (V == 128 && with_o)) return 0;
-        return 1;
-    }
+    static constexpr int NW = V / 16;                 // computing wavefronts per workgroup
+    static constexpr int KB = K * (int)sizeof(T);     // bytes of one operand row
+    // Store waves.  Only where eight waves leave every computing wave the registers it needs: not at V = 128
+    // (eight computing waves already) and not for operand rows beyond 128 bytes.
+    static constexpr int NH = (V == 64 && KB <= 128) ? 4 : 0;
+    static constexpr int THREADS = 64 * (NW + NH);
+    // Depth of the register ring of block shares and own tiles (chunks in flight from global memory); a multiple
+    // of the number of slots so that slot numbers are static in the unrolled loop; 0: no ring, one chunk at a time.
+    static constexpr int DR = KB <= 128 ? 6 : KB <= 256 ? 3 : 0;
+    // Whether LDS reads are issued a phase ahead of their use as described above, or left where the compiler
+    // puts them (the shapes whose operands would not fit the register file twice over).
+    static constexpr bool pipelined(bool with_o) { return KB <= 128 || (KB <= 256 && !(V == 128 && with_o)); }
+    // ... and whether that includes the operands of the state update (80 registers at KB = 256, too many for the
+    // eight-wave workgroups of V = 128, which have 256 registers per lane)
+    static constexpr bool early_update_reads() { return KB <= 128 || (KB <= 256 && V == 64); }
 };
 
-// one wave's share of a shared operand block: instructions w, w+NW, ... of the NI 1-KiB pieces
+// one wave's share of a shared operand block: the 1-KiB pieces w, w+NW, ... of its NI pieces
 template <int NI, int NW> struct Share {
     static constexpr int CNT = (NI + NW - 1) / NW;
     i32x4 a[CNT];
@@ -70,24 +89,85 @@ template <int NI, int NW> struct Share {
     }
 };
 
+// One store wave's part of copying an outbox record of NP 1-KiB pieces to global memory; piece i goes to dst(i).
+template <int NP, int NH, typename Dst>
+__device__ __forceinline__ void copy_out(const char* outbox, int hw, Dst dst) {
+    const int l = lane_id();
+#pragma unroll
+    for (int j = 0; j < (NP + NH - 1) / NH; ++j) {
+        const int i = hw + j * NH;
+        if (i < NP) *reinterpret_cast<i32x4*>(dst(i) + l * 16) = *reinterpret_cast<const i32x4*>(outbox + i * 1024 + l * 16);
+    }
+}
+
 // ---- forward -------------------------------------------------------------------------------------------------
+// LDS of the forward scan: the three operand slots, then (with store waves) two outboxes.  Backward pass: an
+// outbox is the chunk's checkpoint record, [K/32][V/16] tile pairs of the state then [V/16] tile pairs of v_new,
+// exactly as in global memory.  Forward pass: the 16 x V output rows, padded by 16 bytes a row against bank
+// conflicts.
+template <typename T, int K, int V, bool WRITE_O> struct FwdLds {
+    static constexpr int ES = sizeof(T), NH = ScanCfg<T, K, V>::NH;
+    static constexpr int SLOT = blk_fwd(K, ES, WRITE_O).SIZE;
+    static constexpr int OROW = V * ES + 16;
+    static constexpr int OB_HC = K * V * ES, OB = WRITE_O ? CH * OROW : OB_HC + 2 * CH * V * ES;
+    static constexpr int BYTES = NSLOT * SLOT + (NH ? 2 * OB : 0);
+};
+
 template <typename T, int K, int V, bool WRITE_O>
-__global__ __launch_bounds__(V * 4) void scan_fwd_kernel(ChunkArgs<T> p) {
+__device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem) {
     constexpr int KT = K / 16, KT2 = KT / 2, VT = V / 16, NW = ScanCfg<T, K, V>::NW, DR = ScanCfg<T, K, V>::DR;
+    constexpr int NH = ScanCfg<T, K, V>::NH, ES = sizeof(T);
     constexpr BlkF B = blk_fwd(K, sizeof(T), WRITE_O);
-    constexpr int RM = ScanCfg<T, K, V>::read_mode(WRITE_O);
-    constexpr int ES = sizeof(T), NI = B.SIZE / 1024;
-    __shared__ __attribute__((aligned(16))) char lds[2][B.SIZE];
+    constexpr bool PIPE = ScanCfg<T, K, V>::pipelined(WRITE_O);
+    constexpr bool PIPE_UPD = PIPE && ScanCfg<T, K, V>::early_update_reads();
+    constexpr int NI = B.SIZE / 1024;
+    typedef FwdLds<T, K, V, WRITE_O> L;
+    constexpr int OROW = L::OROW, OB_HC = L::OB_HC, OB = L::OB;
+    char (*lds)[B.SIZE] = reinterpret_cast<char (*)[B.SIZE]>(smem);
+    char (*outbox)[OB] = reinterpret_cast<char (*)[OB]>(smem + NSLOT * B.SIZE);
 
     const int h = blockIdx.x, n = blockIdx.y;
-    const int vt = threadIdx.x >> 6;                      // this wave's column block; also its index for the shares
+    const int vt = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // column block of a computing wave
     const int l = lane_id(), g = l >> 4, c = l & 15;
     const int H = p.H;
     int c0, c1;
     seq_chunks(p.st, n, c0, c1);
     int64_t bos, eos;
     seq_bounds(p.st, n, bos, eos);
-    PHASE_CLOCK(p, (blockIdx.y * gridDim.x + blockIdx.x) * NW + vt, 0);
+    const int64_t chw0 = (int64_t)h * p.st.nch;
+    const int nchunks = c1 - c0;
+
+    if (NH && vt >= NW) {
+        // ---- store wave: one barrier for the computing waves' prologue, one per chunk, one to close; after the
+        // barrier of step t the outbox of chunk t-1 is complete, and it is overwritten only after the barrier of t+1
+        if (nchunks <= 0) return;
+        const int hw = vt - NW;
+        lds_barrier();
+        for (int t = 0; t <= nchunks; ++t) {
+            lds_barrier();
+            if (t == 0) continue;
+            const int cid = c0 + t - 1;
+            const char* ob = outbox[(t - 1) & 1];
+            if (WRITE_O) {
+                // rows of o: 16-byte pieces, LPR lanes a row
+                constexpr int LPR = V * ES / 16, RPI = 64 / LPR;
+                const int64_t tok0 = bos + (int64_t)(cid - c0) * CH;
+                const int len = (int)min((int64_t)CH, eos - tok0);
+#pragma unroll
+                for (int r0 = hw * RPI; r0 < CH; r0 += (NH ? NH : 1) * RPI) {
+                    const int r = r0 + l / LPR, e = (l % LPR) * 16;
+                    if (r < len)
+                        *reinterpret_cast<i32x4*>(reinterpret_cast<char*>(p.o + ((tok0 + r) * H + h) * V) + e) =
+                            *reinterpret_cast<const i32x4*>(ob + r * OROW + e);
+                }
+            } else {
+                char* hc = reinterpret_cast<char*>(p.ws.HC + (chw0 + cid) * (K * V));
+                char* vn = reinterpret_cast<char*>(p.ws.VN + (chw0 + cid) * (2 * CH * V));
+                copy_out<OB / 1024, NH ? NH : 1>(ob, hw, [&](int i) { return i < OB_HC / 1024 ? hc + i * 1024 : vn + (i - OB_HC / 1024) * 1024; });
+            }
+        }
+        return;
+    }
 
     // state block: lane (g,c) reg i of tile kt = S[16kt + 4g + i][16vt + c]
     f32x4 S[KT];
@@ -100,48 +180,41 @@ __global__ __launch_bounds__(V * 4) void scan_fwd_kernel(ChunkArgs<T> p) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) S[kt][i] = p.h0[soff + (int64_t)(16 * kt + 4 * g + i) * V];
     }
-    const int64_t chw0 = (int64_t)h * p.st.nch;
-    const char* blocks = reinterpret_cast<const char*>(p.ws.W);
-
-    struct Stage {
-        Share<NI, NW> sh;
-        Frag<T> ut[2], vtt;
+    const int last = c1 - 1;
+    // block of chunk cid; indices past the end of the sequence are clamped, so every load is unconditional (a load
+    // that may or may not have been issued would make the compiler wait for all outstanding loads)
+    auto blk = [&](int cid) __attribute__((always_inline)) {
+        return reinterpret_cast<const char*>(p.ws.W) + (chw0 + min(cid, last)) * B.SIZE;
     };
-    auto load_share = [&](Stage& st, int cid) __attribute__((always_inline)) {
-        st.sh.load(blocks + (chw0 + cid) * B.SIZE, vt);
-    };
-    auto load_own = [&](Stage& st, int cid) __attribute__((always_inline)) {
-        if (!ScanCfg<T, K, V>::RING_OWN) return;
-        const int64_t chw = chw0 + cid;
-        ld_pair(p.ws.UT + (chw * VT + vt) * PAIR, st.ut[0], st.ut[1]);
-        st.vtt = ld_tile(p.ws.VTT + (chw * VT + vt) * TILE);
-    };
-    auto load_stage = [&](Stage& st, int cid) __attribute__((always_inline)) {
-        load_share(st, cid);
-        load_own(st, cid);
+    struct Own { Frag<T> ut[2], vtt; };                   // the tiles only this wave reads
+    auto load_own = [&](Own& o, int cid) __attribute__((always_inline)) {
+        const int64_t chw = chw0 + min(cid, last);
+        ld_pair(p.ws.UT + (chw * VT + vt) * PAIR, o.ut[0], o.ut[1]);
+        o.vtt = ld_tile(p.ws.VTT + (chw * VT + vt) * TILE);
     };
 
-    // one chunk, shared operands from the LDS slot, own operands in registers
-    auto step = [&](const char* slot, Frag<T> ut0, Frag<T> ut1, Frag<T> vtt, int cid) __attribute__((always_inline)) {
+    Frag<T> w[2][KT];                                     // phase-1 operands; when pipelined, read a step ahead
+    auto read_w = [&](const char* slot, int kp) __attribute__((always_inline)) {
+        const T* sW = reinterpret_cast<const T*>(slot + B.W);
+        ld_pair(sW + (0 * KT2 + kp) * PAIR, w[0][2 * kp], w[0][2 * kp + 1]);
+        ld_pair(sW + (1 * KT2 + kp) * PAIR, w[1][2 * kp], w[1][2 * kp + 1]);
+    };
+    auto read_w_all = [&](const char* slot) __attribute__((always_inline)) {
+#pragma unroll
+        for (int kp = 0; kp < KT2; ++kp) read_w(slot, kp);
+    };
+
+    // one chunk: shared operands from `slot`, the phase-1 operands of the next chunk from `slot_next`, results
+    // that go to global memory into the outbox `ob` (when there are store waves)
+    auto step = [&](const char* slot, const char* slot_next, char* ob, Own own, int cid) __attribute__((always_inline)) {
         const int64_t chw = chw0 + cid;
         const int64_t tok0 = bos + (int64_t)(cid - c0) * CH;
         const int len = (int)min((int64_t)CH, eos - tok0);
-        const T* sW = reinterpret_cast<const T*>(slot + B.W);
         const T* sBGT = reinterpret_cast<const T*>(slot + B.BGT);
         const T* sKGT = reinterpret_cast<const T*>(slot + B.KGT);
         const float* sEGL = reinterpret_cast<const float*>(slot + B.EGL);
-        if (!ScanCfg<T, K, V>::RING_OWN) {
-            ld_pair(p.ws.UT + (chw * VT + vt) * PAIR, ut0, ut1);
-            vtt = ld_tile(p.ws.VTT + (chw * VT + vt) * TILE);
-        }
-        // All LDS reads of the step are issued up front, in the order of use: left to itself the compiler sinks
-        // each read to just before its product and the step pays the LDS latency half a dozen times over.
-        Frag<T> w[2][KT], qg[WRITE_O ? KT : 1], aqk, aqb[2], kgt[KT], bgt[2][KT];
+        Frag<T> qg[WRITE_O ? KT : 1], aqk, aqb[2], kgt[KT], bgt[2][KT];
         f32x4 egl[KT];
-        auto read_w = [&](int kp) __attribute__((always_inline)) {
-            ld_pair(sW + (0 * KT2 + kp) * PAIR, w[0][2 * kp], w[0][2 * kp + 1]);
-            ld_pair(sW + (1 * KT2 + kp) * PAIR, w[1][2 * kp], w[1][2 * kp + 1]);
-        };
         auto read_qg = [&](int kp) __attribute__((always_inline)) {
             ld_pair(reinterpret_cast<const T*>(slot + B.QG) + kp * PAIR, qg[2 * kp], qg[2 * kp + 1]);
         };
@@ -152,126 +225,141 @@ __global__ __launch_bounds__(V * 4) void scan_fwd_kernel(ChunkArgs<T> p) {
             egl[2 * kp] = *reinterpret_cast<const f32x4*>(sEGL + 16 * (2 * kp) + 4 * g);
             egl[2 * kp + 1] = *reinterpret_cast<const f32x4*>(sEGL + 16 * (2 * kp + 1) + 4 * g);
         };
-        if (RM) {
-#pragma unroll
-            for (int kp = 0; kp < KT2; ++kp) read_w(kp);
-            if (WRITE_O) {
+        if (WRITE_O) {
+            if (PIPE) {
 #pragma unroll
                 for (int kp = 0; kp < KT2; ++kp) read_qg(kp);
             }
-        }
-        if (WRITE_O) {
             ld_pair(reinterpret_cast<const T*>(slot + B.AQB), aqb[0], aqb[1]);
             aqk = ld_tile(reinterpret_cast<const T*>(slot + B.AQK));
         }
-        if (RM == 2) {
+        if (PIPE_UPD) {
 #pragma unroll
             for (int kp = 0; kp < KT2; ++kp) read_upd(kp);
         }
-        if (RM) __builtin_amdgcn_sched_barrier(0);
+        if (PIPE) __builtin_amdgcn_sched_barrier(0);      // the reads above stay above the products below
         Frag<T> sb[KT];
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt) sb[kt] = to_frag<T>(S[kt]);
         // v_new^T (rows value, inner token) = u^T + S^T w^T
-        f32x4 vn[2] = {to_f32(ut0), to_f32(ut1)};
+        f32x4 vn[2] = {to_f32(own.ut[0]), to_f32(own.ut[1])};
 #pragma unroll
         for (int kp = 0; kp < KT2; ++kp) {
-            if (!RM) read_w(kp);
-            vn[0] = mm2s<0>(sb[2 * kp], w[0][2 * kp], sb[2 * kp + 1], w[0][2 * kp + 1], vn[0]);
-            vn[1] = mm2s<0>(sb[2 * kp], w[1][2 * kp], sb[2 * kp + 1], w[1][2 * kp + 1], vn[1]);
-        }
-        if (RM == 1) {
+            if (!PIPE) read_w(slot, kp);
 #pragma unroll
-            for (int kp = 0; kp < KT2; ++kp) read_upd(kp);
+            for (int kt = 2 * kp; kt < 2 * kp + 2; ++kt) {
+                vn[0] = mm(sb[kt], w[0][kt], vn[0]);
+                vn[1] = mm(sb[kt], w[1][kt], vn[1]);
+            }
+        }
+        f32x4 o = zero4();
+        if (WRITE_O) {
+            // o (rows token, inner value) = qg S + A_qk v + sum_s A_qb^s v_new_s; the first two terms here
+#pragma unroll
+            for (int kp = 0; kp < KT2; ++kp) {
+                if (!PIPE) read_qg(kp);
+                o = mm(qg[2 * kp], sb[2 * kp], o);
+                o = mm(qg[2 * kp + 1], sb[2 * kp + 1], o);
+            }
+            o = mm(aqk, own.vtt, o);
+        }
+        if (PIPE) {
+            __builtin_amdgcn_sched_barrier(0);
+            read_w_all(slot_next);                        // the products above have taken their operands already
             __builtin_amdgcn_sched_barrier(0);
         }
         const Frag<T> vnb[2] = {to_frag<T>(vn[0]), to_frag<T>(vn[1])};
         if (!WRITE_O) {
             // checkpoint of the entering state and v_new, as the fragments held here (tile pairs, 16 bytes per
             // lane, whole cache lines): the chunk_grad kernel turns them the way it needs them
-            T* hc = p.ws.HC + chw * (K * V) + vt * PAIR;
+            T* hc = (NH ? reinterpret_cast<T*>(ob) : p.ws.HC + chw * (K * V)) + vt * PAIR;
+            T* vnp = (NH ? reinterpret_cast<T*>(ob + OB_HC) : p.ws.VN + chw * (2 * CH * V)) + vt * PAIR;
 #pragma unroll
             for (int kp = 0; kp < KT2; ++kp) st_pair2(hc + kp * VT * PAIR, sb[2 * kp], sb[2 * kp + 1]);
-            st_pair2(p.ws.VN + chw * (2 * CH * V) + vt * PAIR, vnb[0], vnb[1]);
+            st_pair2(vnp, vnb[0], vnb[1]);
         }
         if (WRITE_O) {
-            // o (rows token, inner value) = qg S + A_qk v + sum_s A_qb^s v_new_s
-            f32x4 o = zero4();
-#pragma unroll
-            for (int kp = 0; kp < KT2; ++kp) {
-                if (!RM) read_qg(kp);
-                o = mm2s<1>(qg[2 * kp], sb[2 * kp], qg[2 * kp + 1], sb[2 * kp + 1], o);
-            }
-            o = mm(aqk, vtt, o);
-            o = mm2s<2>(aqb[0], vnb[0], aqb[1], vnb[1], o);
-            if (c < len) st_frag(p.o + ((tok0 + c) * H + h) * V + 16 * vt + 4 * g, to_frag<T>(o));
+            o = mm(aqb[0], vnb[0], o);
+            o = mm(aqb[1], vnb[1], o);
+            if (NH) st_frag(reinterpret_cast<T*>(ob + c * OROW) + 16 * vt + 4 * g, to_frag<T>(o));
+            else if (c < len) st_frag(p.o + ((tok0 + c) * H + h) * V + 16 * vt + 4 * g, to_frag<T>(o));
         }
         // S <- exp(g_last) S + kg^T v + sum_s bg_s^T v_new_s
 #pragma unroll
         for (int kp = 0; kp < KT2; ++kp) {
-            if (!RM) read_upd(kp);
+            if (!PIPE_UPD) read_upd(kp);
 #pragma unroll
             for (int kt = 2 * kp; kt < 2 * kp + 2; ++kt) {
                 f32x4 x = S[kt] * egl[kt];
-                x = mm(vtt, kgt[kt], x);
-                x = mm2s<3>(vnb[0], bgt[0][kt], vnb[1], bgt[1][kt], x);
+                x = mm(own.vtt, kgt[kt], x);
+                x = mm(vnb[0], bgt[0][kt], x);
+                x = mm(vnb[1], bgt[1][kt], x);
                 S[kt] = x;
             }
         }
     };
 
-#ifdef HDLA_PHASE_TIMING
-    long long tacc[3] = {0, 0, 0}, tlast = clock64();
-#define TCK(i) do { long long t_ = clock64(); tacc[((i) + 2) % 3] += t_ - tlast; tlast = t_; } while (0)
-#else
-#define TCK(i) do { } while (0)
-#endif
-    const int nchunks = c1 - c0;
     if (nchunks > 0) {
-        // Every global load of the main loop is unconditional (prefetch indices are clamped to the last chunk): a
-        // load that may or may not have been issued would make the compiler wait for all outstanding loads.
-        Stage ring[DR];
+        int done = 0;
+        if constexpr (DR > 0) {
+            Share<NI, NW> sh[DR];
+            Own own[DR];
 #pragma unroll
-        for (int d = 0; d < DR; ++d) load_stage(ring[d], min(c0 + d, c1 - 1));
-        ring[0].sh.to_lds(lds[0], vt);
-        const int nfull = nchunks / DR;
+            for (int d = 0; d < DR; ++d) {
+                sh[d].load(blk(c0 + d), vt);
+                load_own(own[d], c0 + d);
+            }
+            sh[0].to_lds(lds[0], vt);
+            sh[1].to_lds(lds[1], vt);
+            sh[0].load(blk(c0 + DR), vt);
+            sh[1].load(blk(c0 + DR + 1), vt);
+            lds_barrier();
+            if (PIPE) read_w_all(lds[0]);
+            const int nfull = nchunks / DR;
 #pragma unroll 1
-        for (int gi = 0; gi < nfull; ++gi) {
-            const int base = c0 + gi * DR;
+            for (int gi = 0; gi < nfull; ++gi) {
+                const int base = c0 + gi * DR;
 #pragma unroll
-            for (int j = 0; j < DR; ++j) {                 // DR is even: chunk base+j lives in LDS slot j & 1
-                const int cid = base + j;
-                TCK(0);
-                lds_barrier();                             // block of this chunk complete; other slot free again
-                TCK(1);
-                ring[(j + 1) % DR].sh.to_lds(lds[(j + 1) & 1], vt);                 // hand over the next chunk
-                TCK(2);
-                const int nxt = min(cid + DR, c1 - 1);
-                load_share(ring[j], nxt);                  // this share went to LDS a step ago: refill it now
-                step(lds[j & 1], ring[j].ut[0], ring[j].ut[1], ring[j].vtt, cid);
-                // the own tiles are refilled only after their last use: a register that is loaded while its old
-                // value is still live needs a copy, and the copy would wait for the load just issued
-                load_own(ring[j], nxt);
+                for (int j = 0; j < DR; ++j) {             // DR is a multiple of NSLOT: chunk base+j lives in slot j % 3
+                    const int cid = base + j;
+                    lds_barrier();
+                    sh[(j + 2) % DR].to_lds(lds[(j + 2) % NSLOT], vt);
+                    sh[(j + 2) % DR].load(blk(cid + 2 + DR), vt);
+                    step(lds[j % NSLOT], lds[(j + 1) % NSLOT], outbox[(cid - c0) & 1], own[j], cid);
+                    // refilled only after the last use: a register that is loaded while its old value is still
+                    // live needs a copy, and the copy would wait for the load just issued
+                    load_own(own[j], cid + DR);
+                }
+            }
+            done = nfull * DR;
+        } else {
+            Share<NI, NW> tmp;
+            tmp.load(blk(c0), vt);
+            tmp.to_lds(lds[0], vt);
+            tmp.load(blk(c0 + 1), vt);
+            tmp.to_lds(lds[1], vt);
+            lds_barrier();
+            if (PIPE) read_w_all(lds[0]);
+        }
+        // what is left (fewer than DR chunks, or all of them without a ring): one chunk at a time, same protocol
+        if (done < nchunks) {
+            Own cur;
+            load_own(cur, c0 + done);
+#pragma unroll 1
+            for (int t = done; t < nchunks; ++t) {
+                const int cid = c0 + t;
+                lds_barrier();
+                Share<NI, NW> tmp;
+                tmp.load(blk(cid + 2), vt);
+                Own nxt;
+                load_own(nxt, cid + 1);
+                step(lds[t % NSLOT], lds[(t + 1) % NSLOT], outbox[t & 1], cur, cid);
+                tmp.to_lds(lds[(t + 2) % NSLOT], vt);
+                cur = nxt;
             }
         }
-#pragma unroll 1
-        for (int cid = c0 + nfull * DR; cid < c1; ++cid) {  // fewer than DR chunks left: one at a time
-            Stage st;
-            load_stage(st, cid);
-            lds_barrier();
-            st.sh.to_lds(lds[0], vt);
-            lds_barrier();
-            step(lds[0], st.ut[0], st.ut[1], st.vtt, cid);
-        }
+        if (NH) lds_barrier();                            // hands the last outbox to the store waves
     }
-    PHASE_CLOCK(p, (blockIdx.y * gridDim.x + blockIdx.x) * NW + vt, 1);
-#ifdef HDLA_PHASE_TIMING
-    {
-        const int blk_ = (blockIdx.y * gridDim.x + blockIdx.x) * NW + vt;
-        if (p.phase_clk && blk_ < 64 && lane_id() == 0)
-            for (int i = 0; i < 3; ++i) p.phase_clk[blk_ * 16 + 8 + i] = tacc[i];
-    }
-#endif
     if (p.ht) {
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
@@ -281,23 +369,55 @@ __global__ __launch_bounds__(V * 4) void scan_fwd_kernel(ChunkArgs<T> p) {
 }
 
 // ---- backward ------------------------------------------------------------------------------------------------
+// LDS of the reverse scan: three operand slots, then two outboxes holding the chunk's record of dS ([K/32][V/16]
+// tile pairs) then dv_new ([V/16] tile pairs), as in global memory.
+template <typename T, int K, int V> struct BwdLds {
+    static constexpr int ES = sizeof(T), NH = ScanCfg<T, K, V>::NH;
+    static constexpr int SLOT = blk_bwd(K, ES).SIZE;
+    static constexpr int OB_HC = K * V * ES, OB = OB_HC + 2 * CH * V * ES;
+    static constexpr int BYTES = NSLOT * SLOT + (NH ? 2 * OB : 0);
+};
+
 template <typename T, int K, int V>
-__global__ __launch_bounds__(V * 4) void scan_bwd_kernel(ChunkArgs<T> p) {
+__device__ __forceinline__ void scan_bwd_body(const ChunkArgs<T>& p, char* smem) {
     constexpr int KT = K / 16, KT2 = KT / 2, VT = V / 16, NW = ScanCfg<T, K, V>::NW, DR = ScanCfg<T, K, V>::DR;
+    constexpr int NH = ScanCfg<T, K, V>::NH, ES = sizeof(T);
     constexpr BlkB B = blk_bwd(K, sizeof(T));
-    constexpr int RM = ScanCfg<T, K, V>::read_mode(false);
+    constexpr bool PIPE = ScanCfg<T, K, V>::pipelined(false);
+    constexpr bool PIPE_UPD = PIPE && ScanCfg<T, K, V>::early_update_reads();
     constexpr int NI = B.SIZE / 1024;
-    __shared__ __attribute__((aligned(16))) char lds[2][B.SIZE];
+    typedef BwdLds<T, K, V> L;
+    constexpr int OB_HC = L::OB_HC, OB = L::OB;
+    char (*lds)[B.SIZE] = reinterpret_cast<char (*)[B.SIZE]>(smem);
+    char (*outbox)[OB] = reinterpret_cast<char (*)[OB]>(smem + NSLOT * B.SIZE);
 
     const int h = blockIdx.x, n = blockIdx.y;
-    const int vt = threadIdx.x >> 6;
+    const int vt = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int l = lane_id(), g = l >> 4, c = l & 15;
     const int H = p.H;
     int c0, c1;
     seq_chunks(p.st, n, c0, c1);
     int64_t bos, eos;
     seq_bounds(p.st, n, bos, eos);
-    PHASE_CLOCK(p, (blockIdx.y * gridDim.x + blockIdx.x) * NW + vt, 0);
+    const int64_t chw0 = (int64_t)h * p.st.nch;
+    const int nchunks = c1 - c0;
+
+    if (NH && vt >= NW) {
+        // ---- store wave (see the forward scan); step t handles chunk c1-1-t
+        if (nchunks <= 0) return;
+        const int hw = vt - NW;
+        lds_barrier();
+        for (int t = 0; t <= nchunks; ++t) {
+            lds_barrier();
+            if (t == 0) continue;
+            const int cid = c1 - t;
+            char* hc = reinterpret_cast<char*>(p.ws.DHC + (chw0 + cid) * (K * V));
+            char* vn = reinterpret_cast<char*>(p.ws.DVN + (chw0 + cid) * (2 * CH * V));
+            copy_out<OB / 1024, NH ? NH : 1>(outbox[(t - 1) & 1], hw,
+                                              [&](int i) { return i < OB_HC / 1024 ? hc + i * 1024 : vn + (i - OB_HC / 1024) * 1024; });
+        }
+        return;
+    }
 
     f32x4 dS[KT];   // lane (g,c) reg i of tile kt = dS[16kt + 4g + i][16vt + c]
     const int64_t soff = ((int64_t)n * H + h) * K * V + 16 * vt + c;
@@ -310,39 +430,36 @@ __global__ __launch_bounds__(V * 4) void scan_bwd_kernel(ChunkArgs<T> p) {
             for (int i = 0; i < 4; ++i) dS[kt][i] = p.dht[soff + (int64_t)(16 * kt + 4 * g + i) * V];
     }
     const Frag<T> ident = ident_frag<T>();
-    const int64_t chw0 = (int64_t)h * p.st.nch;
-    const char* blocks = reinterpret_cast<const char*>(p.ws.BG);
-
-    struct Stage {
-        Share<NI, NW> sh;
-        Frag<T> don;      // rows past the end of a ragged chunk alias its last row and are zeroed where used
+    // the scan runs from the last chunk to the first: step t handles chunk c1-1-t; indices before c0 are clamped
+    auto blk = [&](int cid) __attribute__((always_inline)) {
+        return reinterpret_cast<const char*>(p.ws.BG) + (chw0 + max(cid, c0)) * B.SIZE;
     };
-    auto load_share = [&](Stage& st, int cid) __attribute__((always_inline)) {
-        st.sh.load(blocks + (chw0 + cid) * B.SIZE, vt);
-    };
-    auto load_own = [&](Stage& st, int cid) __attribute__((always_inline)) {
-        const int64_t tok0 = bos + (int64_t)(cid - c0) * CH;
+    // rows of do; rows past the end of a ragged chunk alias its last row and are zeroed where used
+    auto load_own = [&](Frag<T>& don, int cid) __attribute__((always_inline)) {
+        const int64_t tok0 = bos + (int64_t)(max(cid, c0) - c0) * CH;
         const int len = (int)min((int64_t)CH, eos - tok0);
-        st.don = ld_frag(p.dout + ((tok0 + min(c, len - 1)) * H + h) * V + 16 * vt + 4 * g);
-    };
-    auto load_stage = [&](Stage& st, int cid) __attribute__((always_inline)) {
-        load_share(st, cid);
-        load_own(st, cid);
+        don = ld_frag(p.dout + ((tok0 + min(c, len - 1)) * H + h) * V + 16 * vt + 4 * g);
     };
 
-    auto step = [&](const char* slot, Frag<T> don, int cid) __attribute__((always_inline)) {
-        const int64_t chw = chw0 + cid;
+    Frag<T> aq[2], bg[2][KT];                             // phase-1 operands; when pipelined, read a step ahead
+    auto read_bg = [&](const char* slot, int kp) __attribute__((always_inline)) {
         const T* sBG = reinterpret_cast<const T*>(slot + B.BG);
+        ld_pair(sBG + (0 * KT2 + kp) * PAIR, bg[0][2 * kp], bg[0][2 * kp + 1]);
+        ld_pair(sBG + (1 * KT2 + kp) * PAIR, bg[1][2 * kp], bg[1][2 * kp + 1]);
+    };
+    auto read_p1_all = [&](const char* slot) __attribute__((always_inline)) {
+        ld_pair(reinterpret_cast<const T*>(slot + B.AQBT), aq[0], aq[1]);
+#pragma unroll
+        for (int kp = 0; kp < KT2; ++kp) read_bg(slot, kp);
+    };
+
+    auto step = [&](const char* slot, const char* slot_next, char* ob, Frag<T> don, int cid) __attribute__((always_inline)) {
+        const int64_t chw = chw0 + cid;
         const T* sWT = reinterpret_cast<const T*>(slot + B.WT);
         const T* sQGT = reinterpret_cast<const T*>(slot + B.QGT);
         const float* sEGL = reinterpret_cast<const float*>(slot + B.EGL);
-        // all LDS reads first, in the order of use (see the forward scan)
-        Frag<T> aq[2], bg[2][KT], qgt[KT], wt[2][KT];
+        Frag<T> qgt[KT], wt[2][KT];
         f32x4 egl[KT];
-        auto read_bg = [&](int kp) __attribute__((always_inline)) {
-            ld_pair(sBG + (0 * KT2 + kp) * PAIR, bg[0][2 * kp], bg[0][2 * kp + 1]);
-            ld_pair(sBG + (1 * KT2 + kp) * PAIR, bg[1][2 * kp], bg[1][2 * kp + 1]);
-        };
         auto read_upd = [&](int kp) __attribute__((always_inline)) {
             ld_pair(sQGT + kp * PAIR, qgt[2 * kp], qgt[2 * kp + 1]);
             ld_pair(sWT + (0 * KT2 + kp) * PAIR, wt[0][2 * kp], wt[0][2 * kp + 1]);
@@ -350,16 +467,12 @@ __global__ __launch_bounds__(V * 4) void scan_bwd_kernel(ChunkArgs<T> p) {
             egl[2 * kp] = *reinterpret_cast<const f32x4*>(sEGL + 16 * (2 * kp) + 4 * g);
             egl[2 * kp + 1] = *reinterpret_cast<const f32x4*>(sEGL + 16 * (2 * kp + 1) + 4 * g);
         };
-        ld_pair(reinterpret_cast<const T*>(slot + B.AQBT), aq[0], aq[1]);
-        if (RM) {
-#pragma unroll
-            for (int kp = 0; kp < KT2; ++kp) read_bg(kp);
-        }
-        if (RM == 2) {
+        if (PIPE_UPD) {
 #pragma unroll
             for (int kp = 0; kp < KT2; ++kp) read_upd(kp);
         }
-        if (RM) __builtin_amdgcn_sched_barrier(0);
+        if (PIPE) __builtin_amdgcn_sched_barrier(0);
+        else ld_pair(reinterpret_cast<const T*>(slot + B.AQBT), aq[0], aq[1]);
         Frag<T> dsb[KT];
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt) dsb[kt] = to_frag<T>(dS[kt]);
@@ -372,67 +485,99 @@ __global__ __launch_bounds__(V * 4) void scan_bwd_kernel(ChunkArgs<T> p) {
         dvn[1] = mm(doT, aq[1], zero4());
 #pragma unroll
         for (int kp = 0; kp < KT2; ++kp) {
-            if (!RM) read_bg(kp);
-            dvn[0] = mm2s<4>(dsb[2 * kp], bg[0][2 * kp], dsb[2 * kp + 1], bg[0][2 * kp + 1], dvn[0]);
-            dvn[1] = mm2s<4>(dsb[2 * kp], bg[1][2 * kp], dsb[2 * kp + 1], bg[1][2 * kp + 1], dvn[1]);
-        }
-        if (RM == 1) {
+            if (!PIPE) read_bg(slot, kp);
 #pragma unroll
-            for (int kp = 0; kp < KT2; ++kp) read_upd(kp);
+            for (int kt = 2 * kp; kt < 2 * kp + 2; ++kt) {
+                dvn[0] = mm(dsb[kt], bg[0][kt], dvn[0]);
+                dvn[1] = mm(dsb[kt], bg[1][kt], dvn[1]);
+            }
+        }
+        if (PIPE) {
+            __builtin_amdgcn_sched_barrier(0);
+            read_p1_all(slot_next);
             __builtin_amdgcn_sched_barrier(0);
         }
         const Frag<T> dvb[2] = {to_frag<T>(dvn[0]), to_frag<T>(dvn[1])};
         // gradient of the state leaving the chunk and of v_new, as the fragments held here (tile pairs)
-        T* dhc = p.ws.DHC + chw * (K * V) + vt * PAIR;
+        T* dhc = (NH ? reinterpret_cast<T*>(ob) : p.ws.DHC + chw * (K * V)) + vt * PAIR;
+        T* dvp = (NH ? reinterpret_cast<T*>(ob + OB_HC) : p.ws.DVN + chw * (2 * CH * V)) + vt * PAIR;
 #pragma unroll
         for (int kp = 0; kp < KT2; ++kp) st_pair2(dhc + kp * VT * PAIR, dsb[2 * kp], dsb[2 * kp + 1]);
-        st_pair2(p.ws.DVN + chw * (2 * CH * V) + vt * PAIR, dvb[0], dvb[1]);
+        st_pair2(dvp, dvb[0], dvb[1]);
         // dS <- exp(g_last) dS + qg^T do + sum_s w_s^T dv_new_s
 #pragma unroll
         for (int kp = 0; kp < KT2; ++kp) {
-            if (!RM) read_upd(kp);
+            if (!PIPE_UPD) read_upd(kp);
 #pragma unroll
             for (int kt = 2 * kp; kt < 2 * kp + 2; ++kt) {
                 f32x4 x = dS[kt] * egl[kt];
                 x = mm(doT, qgt[kt], x);
-                x = mm2s<5>(dvb[0], wt[0][kt], dvb[1], wt[1][kt], x);
+                x = mm(dvb[0], wt[0][kt], x);
+                x = mm(dvb[1], wt[1][kt], x);
                 dS[kt] = x;
             }
         }
     };
 
-    const int nchunks = c1 - c0;
     if (nchunks > 0) {
-        Stage ring[DR];
+        const int first = c1 - 1;
+        int done = 0;
+        if constexpr (DR > 0) {
+            Share<NI, NW> sh[DR];
+            Frag<T> own[DR];
 #pragma unroll
-        for (int d = 0; d < DR; ++d) load_stage(ring[d], max(c1 - 1 - d, c0));
-        ring[0].sh.to_lds(lds[0], vt);
-        const int nfull = nchunks / DR;
+            for (int d = 0; d < DR; ++d) {
+                sh[d].load(blk(first - d), vt);
+                load_own(own[d], first - d);
+            }
+            sh[0].to_lds(lds[0], vt);
+            sh[1].to_lds(lds[1], vt);
+            sh[0].load(blk(first - DR), vt);
+            sh[1].load(blk(first - DR - 1), vt);
+            lds_barrier();
+            if (PIPE) read_p1_all(lds[0]);
+            const int nfull = nchunks / DR;
 #pragma unroll 1
-        for (int gi = 0; gi < nfull; ++gi) {
-            const int base = c1 - 1 - gi * DR;
+            for (int gi = 0; gi < nfull; ++gi) {
+                const int base = first - gi * DR;
 #pragma unroll
-            for (int j = 0; j < DR; ++j) {
-                const int cid = base - j;
+                for (int j = 0; j < DR; ++j) {
+                    const int cid = base - j;
+                    lds_barrier();
+                    sh[(j + 2) % DR].to_lds(lds[(j + 2) % NSLOT], vt);
+                    sh[(j + 2) % DR].load(blk(cid - 2 - DR), vt);
+                    step(lds[j % NSLOT], lds[(j + 1) % NSLOT], outbox[(first - cid) & 1], own[j], cid);
+                    load_own(own[j], cid - DR);            // after the last use of the old value: no copy, no wait
+                }
+            }
+            done = nfull * DR;
+        } else {
+            Share<NI, NW> tmp;
+            tmp.load(blk(first), vt);
+            tmp.to_lds(lds[0], vt);
+            tmp.load(blk(first - 1), vt);
+            tmp.to_lds(lds[1], vt);
+            lds_barrier();
+            if (PIPE) read_p1_all(lds[0]);
+        }
+        if (done < nchunks) {
+            Frag<T> cur;
+            load_own(cur, first - done);
+#pragma unroll 1
+            for (int t = done; t < nchunks; ++t) {
+                const int cid = first - t;
                 lds_barrier();
-                ring[(j + 1) % DR].sh.to_lds(lds[(j + 1) & 1], vt);
-                const int nxt = max(cid - DR, c0);
-                load_share(ring[j], nxt);
-                step(lds[j & 1], ring[j].don, cid);
-                load_own(ring[j], nxt);                    // after the last use of the old value: no copy, no wait
+                Share<NI, NW> tmp;
+                tmp.load(blk(cid - 2), vt);
+                Frag<T> nxt;
+                load_own(nxt, cid - 1);
+                step(lds[t % NSLOT], lds[(t + 1) % NSLOT], outbox[t & 1], cur, cid);
+                tmp.to_lds(lds[(t + 2) % NSLOT], vt);
+                cur = nxt;
             }
         }
-#pragma unroll 1
-        for (int cid = c1 - 1 - nfull * DR; cid >= c0; --cid) {
-            Stage st;
-            load_stage(st, cid);
-            lds_barrier();
-            st.sh.to_lds(lds[0], vt);
-            lds_barrier();
-            step(lds[0], st.don, cid);
-        }
+        if (NH) lds_barrier();
     }
-    PHASE_CLOCK(p, (blockIdx.y * gridDim.x + blockIdx.x) * NW + vt, 1);
     if (p.dh0) {
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
@@ -441,18 +586,45 @@ __global__ __launch_bounds__(V * 4) void scan_bwd_kernel(ChunkArgs<T> p) {
     }
 }
 
+// ---- kernels ---------------------------------------------------------------------------------------------------
+template <typename T, int K, int V, bool WRITE_O>
+__global__ __launch_bounds__((ScanCfg<T, K, V>::THREADS)) void scan_fwd_kernel(ChunkArgs<T> p) {
+    __shared__ __attribute__((aligned(16))) char smem[FwdLds<T, K, V, WRITE_O>::BYTES];
+    scan_fwd_body<T, K, V, WRITE_O>(p, smem);
+}
+template <typename T, int K, int V>
+__global__ __launch_bounds__((ScanCfg<T, K, V>::THREADS)) void scan_bwd_kernel(ChunkArgs<T> p) {
+    __shared__ __attribute__((aligned(16))) char smem[BwdLds<T, K, V>::BYTES];
+    scan_bwd_body<T, K, V>(p, smem);
+}
+// Both scans of the backward pass in one launch: they depend on the prep kernel only, not on each other, and each
+// occupies one workgroup per (sequence, head), a fraction of the machine.  blockIdx.z picks the direction.
+template <typename T, int K, int V>
+__global__ __launch_bounds__((ScanCfg<T, K, V>::THREADS)) void scan_pair_kernel(ChunkArgs<T> p) {
+    constexpr int NF = FwdLds<T, K, V, false>::BYTES, NB = BwdLds<T, K, V>::BYTES;
+    __shared__ __attribute__((aligned(16))) char smem[NF > NB ? NF : NB];
+    if (blockIdx.z == 0) scan_fwd_body<T, K, V, false>(p, smem);
+    else scan_bwd_body<T, K, V>(p, smem);
+}
+
 // ---- launchers -----------------------------------------------------------------------------------------------
 template <typename T, int K, int V>
 static hipError_t launch_scan_fwd_kv(const ChunkArgs<T>& a, bool write_o, hipStream_t stream) {
-    dim3 grid(a.H, a.st.N), block(V * 4);
+    dim3 grid(a.H, a.st.N), block(ScanCfg<T, K, V>::THREADS);
     if (write_o) hipLaunchKernelGGL((scan_fwd_kernel<T, K, V, true>), grid, block, 0, stream, a);
     else hipLaunchKernelGGL((scan_fwd_kernel<T, K, V, false>), grid, block, 0, stream, a);
     return hipGetLastError();
 }
 template <typename T, int K, int V>
 static hipError_t launch_scan_bwd_kv(const ChunkArgs<T>& a, hipStream_t stream) {
-    dim3 grid(a.H, a.st.N), block(V * 4);
+    dim3 grid(a.H, a.st.N), block(ScanCfg<T, K, V>::THREADS);
     hipLaunchKernelGGL((scan_bwd_kernel<T, K, V>), grid, block, 0, stream, a);
+    return hipGetLastError();
+}
+template <typename T, int K, int V>
+static hipError_t launch_scan_pair_kv(const ChunkArgs<T>& a, hipStream_t stream) {
+    dim3 grid(a.H, a.st.N, 2), block(ScanCfg<T, K, V>::THREADS);
+    hipLaunchKernelGGL((scan_pair_kernel<T, K, V>), grid, block, 0, stream, a);
     return hipGetLastError();
 }
 
@@ -472,9 +644,19 @@ hipError_t launch_scan_bwd(const ChunkArgs<T>& a, int K, int V, hipStream_t stre
     if (K == 128 && V == 64) return launch_scan_bwd_kv<T, 128, 64>(a, stream);
     return hipErrorInvalidValue;
 }
+template <typename T>
+hipError_t launch_scan_pair(const ChunkArgs<T>& a, int K, int V, hipStream_t stream) {
+    if (K == 64 && V == 64) return launch_scan_pair_kv<T, 64, 64>(a, stream);
+    if (K == 128 && V == 128) return launch_scan_pair_kv<T, 128, 128>(a, stream);
+    if (K == 64 && V == 128) return launch_scan_pair_kv<T, 64, 128>(a, stream);
+    if (K == 128 && V == 64) return launch_scan_pair_kv<T, 128, 64>(a, stream);
+    return hipErrorInvalidValue;
+}
 template hipError_t launch_scan_fwd<bf16>(const ChunkArgs<bf16>&, int, int, bool, hipStream_t);
 template hipError_t launch_scan_fwd<float>(const ChunkArgs<float>&, int, int, bool, hipStream_t);
 template hipError_t launch_scan_bwd<bf16>(const ChunkArgs<bf16>&, int, int, hipStream_t);
 template hipError_t launch_scan_bwd<float>(const ChunkArgs<float>&, int, int, hipStream_t);
+template hipError_t launch_scan_pair<bf16>(const ChunkArgs<bf16>&, int, int, hipStream_t);
+template hipError_t launch_scan_pair<float>(const ChunkArgs<float>&, int, int, hipStream_t);
 
 }  // namespace hdla
