@@ -29,6 +29,12 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     // larger than the L2, so repeated global loads would mostly be repeated HBM reads
     constexpr int VP = V + 16 / (int)sizeof(T);                    // padded row, keeps 16-byte alignment
     __shared__ __attribute__((aligned(16))) T sTok[6 * CH * VP];
+    // Results of 2-byte elements leave through LDS: a lane holds 8 bytes of a row, and 8-byte stores of four lanes
+    // would write 32-byte pieces of rows, half of what HBM writes at once.  Two adjacent 16-column tiles are put
+    // side by side in LDS and stored 16 bytes a lane, 64 contiguous bytes a row.
+    constexpr bool STAGE_OUT = sizeof(T) == 2;
+    constexpr int OPITCH = 80;                                     // bytes; 64 of data, padded against bank conflicts
+    __shared__ __attribute__((aligned(16))) char sOut[STAGE_OUT ? 7 * CH * OPITCH : 16];
 
     const int cid = blockIdx.x, h = blockIdx.y;
     ChunkPos cp;
@@ -36,11 +42,16 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     const int l = lane_id(), g = l >> 4, c = l & 15;
     const int H = p.H;
     const bool rowok = c < cp.len;
-    const int64_t tok = cp.tok0 + min(c, cp.len - 1);   // rows past the end alias the last valid row, masked by rowok
-    const int64_t qoff = (tok * H + h) * K + 4 * g;
-    const int64_t aoff0 = ((tok * RANK + 0) * H + h) * K + 4 * g;
-    const int64_t aoff1 = ((tok * RANK + 1) * H + h) * K + 4 * g;
-    const int64_t voff = (tok * H + h) * V + 4 * g;
+    // Element offsets of the chunk's first row (uniform) and byte offsets of this lane's four elements in row
+    // min(c, len-1) (rows past the end alias the last valid row and are masked by rowok); a/b rows are rank-minor.
+    constexpr uint32_t ES = sizeof(T), GS = GKF32 ? 4 : 2;
+    const int row = min(c, cp.len - 1);
+    const int64_t qb = (cp.tok0 * H + h) * K, ab = (cp.tok0 * RANK * H + h) * K, vb = (cp.tok0 * H + h) * V;
+    const uint32_t qe = (uint32_t)(row * H * K + 4 * g), ae = (uint32_t)(row * RANK * H * K + 4 * g);
+    const uint32_t qo = qe * ES, go = qe * GS, ao0 = ae * ES, ao1 = ao0 + (uint32_t)(H * K) * ES;
+    const uint32_t vo = (uint32_t)(row * H * V + 4 * g) * ES;
+    const char* gkp = reinterpret_cast<const char*>(p.gk) + qb * GS;
+    char* dgkp = reinterpret_cast<char*>(p.dgk) + qb * GS;
     const int64_t chw = (int64_t)h * p.st.nch + cid;
     const float scale = p.scale;
     const T* HC = p.ws.HC + chw * (K * V);
@@ -61,7 +72,7 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
 #pragma unroll
             for (int r0 = 0; r0 < CH; r0 += RPI) {
                 const int r = r0 + rr;
-                const T* src = (m == 0 ? p.dout : p.v) + ((cp.tok0 + min(r, cp.len - 1)) * H + h) * V + e;
+                const T* src = at((m == 0 ? p.dout : p.v) + vb, (uint32_t)(min(r, cp.len - 1) * H * V + e) * ES);
                 i32x4 x = *reinterpret_cast<const i32x4*>(src);
                 if (r >= cp.len) x = (i32x4){0, 0, 0, 0};
                 *reinterpret_cast<i32x4*>(&sTok[(m * CH + r) * VP + e]) = x;
@@ -112,12 +123,12 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     f32x4 rg[KEEP ? KT : 1];
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
-        const f32x4 g4 = ld_gk4<GKF32>(p.gk, qoff + 16 * kt, rowok);
+        const f32x4 g4 = ld_gk4<GKF32>(gkp + go + 16 * kt * GS, 0, rowok);
         const f32x4 gi = scan16_incl(g4), ge = gi - g4;
         const f32x4 m = bcast16(gi, MID);
         const f32x4 eq = exp4<T>(gi - m), ek = exp4<T>(m - gi), ea = exp4<T>(ge - m);
-        const Frag<T> fq = ld_frag_sel(p.q + qoff + 16 * kt, rowok), fk = ld_frag_sel(p.k + qoff + 16 * kt, rowok);
-        const Frag<T> fa0 = ld_frag_sel(p.a + aoff0 + 16 * kt, rowok), fa1 = ld_frag_sel(p.a + aoff1 + 16 * kt, rowok);
+        const Frag<T> fq = ld_frag_sel(at(p.q + qb, qo + 16 * kt * ES), rowok), fk = ld_frag_sel(at(p.k + qb, qo + 16 * kt * ES), rowok);
+        const Frag<T> fa0 = ld_frag_sel(at(p.a + ab, ao0 + 16 * kt * ES), rowok), fa1 = ld_frag_sel(at(p.a + ab, ao1 + 16 * kt * ES), rowok);
         if (KEEP) { rq[kt] = fq; rk[kt] = fk; ra[0][kt] = fa0; ra[1][kt] = fa1; rg[kt] = g4; }
         const f32x4 q4 = to_f32(fq), k4 = to_f32(fk), a0 = to_f32(fa0), a1 = to_f32(fa1);
         const Frag<T> qh = to_frag<T>(q4 * eq * scale), kh = to_frag<T>(k4 * ek);
@@ -204,26 +215,50 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         if (!(j <= c)) { dAqk[i] = 0.f; dAqb[0][i] = 0.f; dAqb[1][i] = 0.f; }
         if (!(j < c)) { dAak[0][i] = 0.f; dAak[1][i] = 0.f; dAab[0][0][i] = 0.f; dAab[0][1][i] = 0.f; dAab[1][0][i] = 0.f; dAab[1][1][i] = 0.f; }
     }
-    const Frag<T> fAqk = to_frag<T>(dAqk), fAqkT = transpose(fAqk, ident);
-    Frag<T> fAqb[2], fAqbT[2], fAak[2], fAakT[2], fAab[2][2], fAabT[2][2];
+    // The transposed tiles are needed once per channel tile of the second pass.  For 2-byte elements the nine of
+    // them fit exactly into the LDS that held (I - A_ab)^-1 (no longer needed) and are read back where used: 18
+    // registers less across the second pass, which is what lets two waves share a SIMD.
+    constexpr bool STASH = sizeof(T) == 2;
+    T* stash = reinterpret_cast<T*>(sT);
+    const Frag<T> fAqk = to_frag<T>(dAqk);
+    Frag<T> fAqb[2], fAak[2], fAab[2][2];
+    Frag<T> rT[STASH ? 1 : 9];                             // transposes kept in registers otherwise
+    auto putT = [&](int idx, Frag<T> f) __attribute__((always_inline)) {
+        const Frag<T> t = transpose(f, ident);
+        if (STASH) st_tile(stash + idx * TILE, t);
+        else rT[STASH ? 0 : idx] = t;
+    };
+    auto getT = [&](int idx) __attribute__((always_inline)) { return STASH ? ld_tile(stash + idx * TILE) : rT[STASH ? 0 : idx]; };
+    // indices: 0 A_qk, 1+s A_qb^s, 3+s A_ak^s, 5+2r+s A_ab^{r s}
+    putT(0, fAqk);
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-        fAqb[s] = to_frag<T>(dAqb[s]); fAqbT[s] = transpose(fAqb[s], ident);
-        fAak[s] = to_frag<T>(dAak[s]); fAakT[s] = transpose(fAak[s], ident);
+        fAqb[s] = to_frag<T>(dAqb[s]); putT(1 + s, fAqb[s]);
+        fAak[s] = to_frag<T>(dAak[s]); putT(3 + s, fAak[s]);
 #pragma unroll
-        for (int r = 0; r < 2; ++r) { fAab[r][s] = to_frag<T>(dAab[r][s]); fAabT[r][s] = transpose(fAab[r][s], ident); }
+        for (int r = 0; r < 2; ++r) { fAab[r][s] = to_frag<T>(dAab[r][s]); putT(5 + 2 * r + s, fAab[r][s]); }
     }
 
+    // put(m, half, f): tile f of output m into column half `half`; flush(m, base, byte0): the 16 x 32 block out
+    auto put = [&](int m, int half, Frag<T> f) __attribute__((always_inline)) {
+        st_frag(reinterpret_cast<T*>(sOut + (m * CH + c) * OPITCH + half * 32) + 4 * g, f);
+    };
+    auto flush = [&](int m, T* ubase, uint32_t row_pitch_bytes, uint32_t byte0) __attribute__((always_inline)) {
+        typedef int i32x4 __attribute__((ext_vector_type(4)));
+        const int r = l >> 2, piece = l & 3;
+        const i32x4 x = *reinterpret_cast<const i32x4*>(sOut + (m * CH + r) * OPITCH + piece * 16);
+        if (r < cp.len) *reinterpret_cast<i32x4*>(reinterpret_cast<char*>(ubase) + (uint32_t)r * row_pitch_bytes + byte0 + piece * 16) = x;
+    };
     PHASE_CLOCK(p, blk, 4);
     // ---- second pass over channel tiles: state products, score backward, final gradients ----------------------
 #pragma unroll(KEEP ? KT : 1)
     for (int kt = 0; kt < KT; ++kt) {
         // (a) what the loop over value tiles needs: only kg of this channel tile
-        const f32x4 g4 = KEEP ? rg[KEEP ? kt : 0] : ld_gk4<GKF32>(p.gk, qoff + 16 * kt, rowok);
+        const f32x4 g4 = KEEP ? rg[KEEP ? kt : 0] : ld_gk4<GKF32>(gkp + go + 16 * kt * GS, 0, rowok);
         const f32x4 gi = scan16_incl(g4);
         const f32x4 gl = bcast16(gi, CH - 1);
         const f32x4 edn = exp4<T>(gl - gi);
-        const f32x4 k4 = to_f32(KEEP ? rk[KEEP ? kt : 0] : ld_frag_sel(p.k + qoff + 16 * kt, rowok));
+        const f32x4 k4 = to_f32(KEEP ? rk[KEEP ? kt : 0] : ld_frag_sel(at(p.k + qb, qo + 16 * kt * ES), rowok));
         const f32x4 kg4 = k4 * edn;
         const Frag<T> kgf = to_frag<T>(kg4);
 
@@ -266,10 +301,10 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         const f32x4 m = bcast16(gi, MID);
         const f32x4 eq = exp4<T>(gi - m), ek = exp4<T>(m - gi), ea = exp4<T>(ge - m);
         const f32x4 egi = exp4<T>(gi), ege = exp4<T>(ge);
-        const f32x4 q4 = to_f32(KEEP ? rq[KEEP ? kt : 0] : ld_frag_sel(p.q + qoff + 16 * kt, rowok));
-        const f32x4 a4[2] = {to_f32(KEEP ? ra[0][KEEP ? kt : 0] : ld_frag_sel(p.a + aoff0 + 16 * kt, rowok)),
-                             to_f32(KEEP ? ra[1][KEEP ? kt : 0] : ld_frag_sel(p.a + aoff1 + 16 * kt, rowok))};
-        const f32x4 b4[2] = {to_f32(ld_frag_sel(p.b + aoff0 + 16 * kt, rowok)), to_f32(ld_frag_sel(p.b + aoff1 + 16 * kt, rowok))};
+        const f32x4 q4 = to_f32(KEEP ? rq[KEEP ? kt : 0] : ld_frag_sel(at(p.q + qb, qo + 16 * kt * ES), rowok));
+        const f32x4 a4[2] = {to_f32(KEEP ? ra[0][KEEP ? kt : 0] : ld_frag_sel(at(p.a + ab, ao0 + 16 * kt * ES), rowok)),
+                             to_f32(KEEP ? ra[1][KEEP ? kt : 0] : ld_frag_sel(at(p.a + ab, ao1 + 16 * kt * ES), rowok))};
+        const f32x4 b4[2] = {to_f32(ld_frag_sel(at(p.b + ab, ao0 + 16 * kt * ES), rowok)), to_f32(ld_frag_sel(at(p.b + ab, ao1 + 16 * kt * ES), rowok))};
         const Frag<T> qhT = transpose(to_frag<T>(q4 * eq * scale), ident), khT = transpose(to_frag<T>(k4 * ek), ident);
         const Frag<T> ahT[2] = {transpose(to_frag<T>(a4[0] * ea), ident), transpose(to_frag<T>(a4[1] * ea), ident)};
         const Frag<T> bhT[2] = {transpose(to_frag<T>(b4[0] * ek), ident), transpose(to_frag<T>(b4[1] * ek), ident)};
@@ -277,9 +312,9 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         f32x4 dqh = mm(fAqk, khT, zero4());
         dqh = mm(fAqb[0], bhT[0], dqh);
         dqh = mm(fAqb[1], bhT[1], dqh);
-        f32x4 dkh = mm(fAqkT, qhT, zero4());
-        dkh = mm(fAakT[0], ahT[0], dkh);
-        dkh = mm(fAakT[1], ahT[1], dkh);
+        f32x4 dkh = mm(getT(0), qhT, zero4());
+        dkh = mm(getT(3), ahT[0], dkh);
+        dkh = mm(getT(4), ahT[1], dkh);
         f32x4 dah[2], dbh[2];
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
@@ -287,9 +322,9 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
             x = mm(fAab[r][0], bhT[0], x);
             x = mm(fAab[r][1], bhT[1], x);
             dah[r] = x;
-            f32x4 y = mm(fAqbT[r], qhT, zero4());          // here r plays the role of the b rank s
-            y = mm(fAabT[0][r], ahT[0], y);
-            y = mm(fAabT[1][r], ahT[1], y);
+            f32x4 y = mm(getT(1 + r), qhT, zero4());          // here r plays the role of the b rank s
+            y = mm(getT(5 + r), ahT[0], y);
+            y = mm(getT(7 + r), ahT[1], y);
             dbh[r] = y;
         }
         const f32x4 dq = (dqh * eq + dqg * egi) * scale;
@@ -300,19 +335,46 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         const f32x4 Dgi = dq * q4 - dk * k4 - db[0] * b4[0] - db[1] * b4[1];
         const f32x4 dgl = exp4<T>(gl) * hh4 + sum16(dkg * kg4 + dbg[0] * bg4[0] + dbg[1] * bg4[1]);
         const f32x4 dg = rscan16_incl(Dgi + Dge) - Dge + dgl;
-        if (rowok) {
-            st_frag(p.dq + qoff + 16 * kt, to_frag<T>(dq));
-            st_frag(p.dk + qoff + 16 * kt, to_frag<T>(dk));
-            st_frag(p.da + aoff0 + 16 * kt, to_frag<T>(da[0]));
-            st_frag(p.da + aoff1 + 16 * kt, to_frag<T>(da[1]));
-            st_frag(p.db + aoff0 + 16 * kt, to_frag<T>(db[0]));
-            st_frag(p.db + aoff1 + 16 * kt, to_frag<T>(db[1]));
-            st_gk4<GKF32>(p.dgk, qoff + 16 * kt, dg);
+        if (STAGE_OUT) {
+            const int half = kt & 1;
+            put(0, half, to_frag<T>(dq));
+            put(1, half, to_frag<T>(dk));
+            put(2, half, to_frag<T>(da[0]));
+            put(3, half, to_frag<T>(da[1]));
+            put(4, half, to_frag<T>(db[0]));
+            put(5, half, to_frag<T>(db[1]));
+            if (!GKF32) put(6, half, to_frag<T>(dg));
+            else if (rowok) st_gk4<GKF32>(dgkp + go + 16 * kt * GS, 0, dg);
+            if (half) {
+                const uint32_t qpitch = (uint32_t)(H * K) * ES, apitch = qpitch * RANK, b0 = (uint32_t)(16 * (kt - 1)) * ES;
+                flush(0, p.dq + qb, qpitch, b0);
+                flush(1, p.dk + qb, qpitch, b0);
+                flush(2, p.da + ab, apitch, b0);
+                flush(3, p.da + ab, apitch, b0 + qpitch);
+                flush(4, p.db + ab, apitch, b0);
+                flush(5, p.db + ab, apitch, b0 + qpitch);
+                if (!GKF32) flush(6, reinterpret_cast<T*>(dgkp), qpitch, b0);
+            }
+        } else if (rowok) {
+            st_frag(at(p.dq + qb, qo + 16 * kt * ES), to_frag<T>(dq));
+            st_frag(at(p.dk + qb, qo + 16 * kt * ES), to_frag<T>(dk));
+            st_frag(at(p.da + ab, ao0 + 16 * kt * ES), to_frag<T>(da[0]));
+            st_frag(at(p.da + ab, ao1 + 16 * kt * ES), to_frag<T>(da[1]));
+            st_frag(at(p.db + ab, ao0 + 16 * kt * ES), to_frag<T>(db[0]));
+            st_frag(at(p.db + ab, ao1 + 16 * kt * ES), to_frag<T>(db[1]));
+            st_gk4<GKF32>(dgkp + go + 16 * kt * GS, 0, dg);
         }
     }
-    if (rowok) {
+    if (STAGE_OUT) {
 #pragma unroll
-        for (int vt = 0; vt < VT; ++vt) st_frag(p.dv + voff + 16 * vt, to_frag<T>(dv[vt]));
+        for (int vt = 0; vt < VT; vt += 2) {
+            put(0, 0, to_frag<T>(dv[vt]));
+            put(0, 1, to_frag<T>(dv[vt + 1]));
+            flush(0, p.dv + vb, (uint32_t)(H * V) * ES, (uint32_t)(16 * vt) * ES);
+        }
+    } else if (rowok) {
+#pragma unroll
+        for (int vt = 0; vt < VT; ++vt) st_frag(at(p.dv + vb, vo + 16 * vt * ES), to_frag<T>(dv[vt]));
     }
     PHASE_CLOCK(p, blk, 5);
 }

@@ -143,6 +143,15 @@ template <typename T> __device__ __forceinline__ Frag<T> transpose(Frag<T> x, Fr
     return to_frag<T>(mm(ident, x, zero4()));
 }
 
+// Address = uniform base (it stays in scalar registers) + a 32-bit byte offset per lane.  This is the form the
+// global memory instructions take directly: one address register per lane instead of two, no 64-bit vector adds.
+template <typename T> __device__ __forceinline__ T* at(T* ubase, uint32_t byte_off) {
+    return reinterpret_cast<T*>(reinterpret_cast<char*>(ubase) + byte_off);
+}
+template <typename T> __device__ __forceinline__ const T* at(const T* ubase, uint32_t byte_off) {
+    return reinterpret_cast<const T*>(reinterpret_cast<const char*>(ubase) + byte_off);
+}
+
 // ---- fragment loads / stores -------------------------------------------------------------------------------
 // four consecutive elements at p (8-byte aligned for bf16, 16-byte aligned for fp32)
 __device__ __forceinline__ Frag<bf16> ld_frag(const bf16* p) { Frag<bf16> r; r.v = *reinterpret_cast<const s16x4*>(p); return r; }

@@ -323,6 +323,9 @@ __device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem)
                 for (int j = 0; j < DR; ++j) {             // DR is a multiple of NSLOT: chunk base+j lives in slot j % 3
                     const int cid = base + j;
                     lds_barrier();
+#ifdef HDLA_PHASE_TIMING
+                    if (!WRITE_O && p.phase_clk && blockIdx.x == 3 && blockIdx.y == 1 && threadIdx.x == 0 && cid - c0 < 1000) p.phase_clk[cid - c0] = wall_clock64();
+#endif
                     sh[(j + 2) % DR].to_lds(lds[(j + 2) % NSLOT], vt);
                     sh[(j + 2) % DR].load(blk(cid + 2 + DR), vt);
                     step(lds[j % NSLOT], lds[(j + 1) % NSLOT], outbox[(cid - c0) & 1], own[j], cid);
