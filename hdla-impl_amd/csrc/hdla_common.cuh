@@ -89,29 +89,9 @@ __device__ __forceinline__ f32x4 mm(Frag<float> frows, Frag<float> finner, f32x4
     return acc;
 }
 
-// Two products into one accumulator: acc += P0 Q0^T + P1 Q1^T.  For bf16 this is ONE 16x16x32 MFMA, which takes
-// the same time as a 16x16x16 one: its inner index k' = 8g + j is read as (product j / 4, inner index 4g + j % 4)
-// on both operands alike, so the operand registers are simply the two fragments side by side.
-typedef short s16x8_ __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-__device__ __forceinline__ f32x4 mm2(Frag<bf16> frows0, Frag<bf16> finner0, Frag<bf16> frows1, Frag<bf16> finner1, f32x4 acc) {
-    const s16x8_ a = __builtin_shufflevector(finner0.v, finner1.v, 0, 1, 2, 3, 4, 5, 6, 7);
-    const s16x8_ b = __builtin_shufflevector(frows0.v, frows1.v, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
-}
-#ifndef HDLA_X32_SITES
-#define HDLA_X32_SITES 0
-#endif
-template <int SITE> __device__ __forceinline__ f32x4 mm2s(Frag<bf16> frows0, Frag<bf16> finner0, Frag<bf16> frows1, Frag<bf16> finner1, f32x4 acc) {
-    if ((HDLA_X32_SITES >> SITE) & 1) return mm2(frows0, finner0, frows1, finner1, acc);
-    return mm(frows1, finner1, mm(frows0, finner0, acc));
-}
-template <int SITE> __device__ __forceinline__ f32x4 mm2s(Frag<float> frows0, Frag<float> finner0, Frag<float> frows1, Frag<float> finner1, f32x4 acc) {
-    return mm(frows1, finner1, mm(frows0, finner0, acc));
-}
-__device__ __forceinline__ f32x4 mm2(Frag<float> frows0, Frag<float> finner0, Frag<float> frows1, Frag<float> finner1, f32x4 acc) {
-    return mm(frows1, finner1, mm(frows0, finner0, acc));
-}
+// (The 16x16x32 bf16 MFMA of gfx950 would do two of these products in the time of one.  It is not used: this
+// toolchain lets a vector ALU instruction overwrite the accumulator-input registers of such an MFMA a few cycles
+// after its issue, while the hardware still reads them, and results then depend on the register allocation.)
 
 // Split operands for the score products of the bf16 path: x = hi + lo with both halves bf16, and
 // P Q^T ~ Ph Qh^T + Ph Ql^T + Pl Qh^T, which removes the rounding of the decayed operands (the largest single
