@@ -61,6 +61,23 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     const int blk = blockIdx.y * gridDim.x + blockIdx.x;
     PHASE_CLOCK(p, blk, 0);
 
+    // q, k, a and gk of the chunk stay in registers for their second use in the last pass (a second load would
+    // mostly be a second HBM read); bf16 operands only, fp32 ones would not fit next to the accumulators.  Their
+    // loads are the first thing issued, so that they travel together with the staging loads below: a wave spends
+    // most of its time waiting for memory, and every dependent round trip to HBM costs thousands of cycles.
+    constexpr bool KEEP = sizeof(T) == 2;
+    Frag<T> rq[KEEP ? KT : 1], rk[KEEP ? KT : 1], ra[2][KEEP ? KT : 1];
+    f32x4 rg[KEEP ? KT : 1];
+    if (KEEP) {
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            rg[KEEP ? kt : 0] = ld_gk4<GKF32>(gkp + go + 16 * kt * GS, 0, rowok);
+            rq[KEEP ? kt : 0] = ld_frag_sel(at(p.q + qb, qo + 16 * kt * ES), rowok);
+            rk[KEEP ? kt : 0] = ld_frag_sel(at(p.k + qb, qo + 16 * kt * ES), rowok);
+            ra[0][KEEP ? kt : 0] = ld_frag_sel(at(p.a + ab, ao0 + 16 * kt * ES), rowok);
+            ra[1][KEEP ? kt : 0] = ld_frag_sel(at(p.a + ab, ao1 + 16 * kt * ES), rowok);
+        }
+    }
     const Frag<T> ident = ident_frag<T>();
     {
         // do and v: rows of the original tensors, 16 bytes per lane
@@ -116,20 +133,16 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     // (the decays are recomputed per channel tile wherever they are needed: a load and four DPP additions cost
     // less than keeping 2*K/16 vector registers alive across the kernel)
     f32x4 aqkT = zero4(), aakT[2] = {zero4(), zero4()};
-    // q, k, a and gk of the chunk stay in registers for their second use in the last pass (a second load would
-    // mostly be a second HBM read); bf16 operands only, fp32 ones would not fit next to the accumulators
-    constexpr bool KEEP = sizeof(T) == 2;
-    Frag<T> rq[KEEP ? KT : 1], rk[KEEP ? KT : 1], ra[2][KEEP ? KT : 1];
-    f32x4 rg[KEEP ? KT : 1];
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
-        const f32x4 g4 = ld_gk4<GKF32>(gkp + go + 16 * kt * GS, 0, rowok);
+        const f32x4 g4 = KEEP ? rg[KEEP ? kt : 0] : ld_gk4<GKF32>(gkp + go + 16 * kt * GS, 0, rowok);
         const f32x4 gi = scan16_incl(g4), ge = gi - g4;
         const f32x4 m = bcast16(gi, MID);
         const f32x4 eq = exp4<T>(gi - m), ek = exp4<T>(m - gi), ea = exp4<T>(ge - m);
-        const Frag<T> fq = ld_frag_sel(at(p.q + qb, qo + 16 * kt * ES), rowok), fk = ld_frag_sel(at(p.k + qb, qo + 16 * kt * ES), rowok);
-        const Frag<T> fa0 = ld_frag_sel(at(p.a + ab, ao0 + 16 * kt * ES), rowok), fa1 = ld_frag_sel(at(p.a + ab, ao1 + 16 * kt * ES), rowok);
-        if (KEEP) { rq[kt] = fq; rk[kt] = fk; ra[0][kt] = fa0; ra[1][kt] = fa1; rg[kt] = g4; }
+        const Frag<T> fq = KEEP ? rq[KEEP ? kt : 0] : ld_frag_sel(at(p.q + qb, qo + 16 * kt * ES), rowok);
+        const Frag<T> fk = KEEP ? rk[KEEP ? kt : 0] : ld_frag_sel(at(p.k + qb, qo + 16 * kt * ES), rowok);
+        const Frag<T> fa0 = KEEP ? ra[0][KEEP ? kt : 0] : ld_frag_sel(at(p.a + ab, ao0 + 16 * kt * ES), rowok);
+        const Frag<T> fa1 = KEEP ? ra[1][KEEP ? kt : 0] : ld_frag_sel(at(p.a + ab, ao1 + 16 * kt * ES), rowok);
         const f32x4 q4 = to_f32(fq), k4 = to_f32(fk), a0 = to_f32(fa0), a1 = to_f32(fa1);
         const Frag<T> qh = to_frag<T>(q4 * eq * scale), kh = to_frag<T>(k4 * ek);
         aqkT = mm(kh, qh, aqkT);
@@ -145,6 +158,17 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     const Frag<T> aqkTf = to_frag<T>(aqkT);
     const Frag<T> aakTf[2] = {to_frag<T>(aakT[0]), to_frag<T>(aakT[1])};
 
+    // Checkpoints of the state (and, for the second pass, of its gradient) arrive a pair of channel tiles ahead of
+    // their use: [buffer][value tile][tile of the pair].  The first pair is requested here, before the loop over
+    // the value dimension, whose work covers the trip.  2-byte types only (registers).
+    constexpr bool PF = sizeof(T) == 2 && K == 64 && V == 64;
+    constexpr int KT2 = KT / 2;
+    Frag<T> hcp[PF ? 2 : 1][PF ? VT : 1][2], dhp[PF ? 2 : 1][PF ? VT : 1][2];
+    auto fetch_pairs = [&](const T* src, Frag<T> (&dst)[PF ? VT : 1][2], int kp) __attribute__((always_inline)) {
+#pragma unroll
+        for (int vt = 0; vt < VT; ++vt) ld_pair(src + (kp * VT + vt) * PAIR, dst[PF ? vt : 0][0], dst[PF ? vt : 0][1]);
+    };
+    if (PF) fetch_pairs(HC, hcp[0], 0);
     PHASE_CLOCK(p, blk, 1);
     // ---- products over the value dimension -------------------------------------------------------------------
     f32x4 dAqk = zero4(), dAqb[2] = {zero4(), zero4()}, dAak[2] = {zero4(), zero4()};
@@ -189,10 +213,12 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     // ---- first pass over channel tiles: dw -> dag -> the w part of dA_ab (dag itself is rebuilt in pass two) ----
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
+        if (PF && !(kt & 1) && kt / 2 + 1 < KT2) fetch_pairs(HC, hcp[PF ? (kt / 2 + 1) & 1 : 0], kt / 2 + 1);
         f32x4 dwT[2] = {zero4(), zero4()};                // rows channel, inner token
 #pragma unroll
         for (int vt = 0; vt < VT; ++vt) {
-            const Frag<T> Sf = transpose(ld_pair_one(HC + ((kt / 2) * VT + vt) * PAIR, kt & 1), ident);
+            const Frag<T> Sf = transpose(PF ? hcp[PF ? (kt / 2) & 1 : 0][PF ? vt : 0][kt & 1]
+                                            : ld_pair_one(HC + ((kt / 2) * VT + vt) * PAIR, kt & 1), ident);
             dwT[0] = mm(Sf, tokf(4, vt), dwT[0]);
             dwT[1] = mm(Sf, tokf(5, vt), dwT[1]);
         }
@@ -207,6 +233,19 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         }
     }
 
+    // for the second pass: the first pair of S and dS tiles, and all of b (used there only), requested now
+    Frag<T> rb[2][KEEP ? KT : 1];
+    if (PF) {
+        fetch_pairs(HC, hcp[0], 0);
+        fetch_pairs(DHC, dhp[0], 0);
+    }
+    if (KEEP) {
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            rb[0][KEEP ? kt : 0] = ld_frag_sel(at(p.b + ab, ao0 + 16 * kt * ES), rowok);
+            rb[1][KEEP ? kt : 0] = ld_frag_sel(at(p.b + ab, ao1 + 16 * kt * ES), rowok);
+        }
+    }
     PHASE_CLOCK(p, blk, 3);
     // ---- masks; both orientations of the nine score-gradient tiles --------------------------------------------
 #pragma unroll
@@ -253,6 +292,10 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     // ---- second pass over channel tiles: state products, score backward, final gradients ----------------------
 #pragma unroll(KEEP ? KT : 1)
     for (int kt = 0; kt < KT; ++kt) {
+        if (PF && !(kt & 1) && kt / 2 + 1 < KT2) {
+            fetch_pairs(HC, hcp[PF ? (kt / 2 + 1) & 1 : 0], kt / 2 + 1);
+            fetch_pairs(DHC, dhp[PF ? (kt / 2 + 1) & 1 : 0], kt / 2 + 1);
+        }
         // (a) what the loop over value tiles needs: only kg of this channel tile
         const f32x4 g4 = KEEP ? rg[KEEP ? kt : 0] : ld_gk4<GKF32>(gkp + go + 16 * kt * GS, 0, rowok);
         const f32x4 gi = scan16_incl(g4);
@@ -268,8 +311,9 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
 #pragma unroll(sizeof(T) == 2 ? VT : 2)
         for (int vt = 0; vt < VT; ++vt) {
             // the scans checkpoint S and dS as fragments of the transposed tiles (rows value, inner channel)
-            const Frag<T> dST = ld_pair_one(DHC + ((kt / 2) * VT + vt) * PAIR, kt & 1);
-            const Frag<T> Sf = transpose(ld_pair_one(HC + ((kt / 2) * VT + vt) * PAIR, kt & 1), ident);
+            const Frag<T> dST = PF ? dhp[PF ? (kt / 2) & 1 : 0][PF ? vt : 0][kt & 1] : ld_pair_one(DHC + ((kt / 2) * VT + vt) * PAIR, kt & 1);
+            const Frag<T> Sf = transpose(PF ? hcp[PF ? (kt / 2) & 1 : 0][PF ? vt : 0][kt & 1]
+                                            : ld_pair_one(HC + ((kt / 2) * VT + vt) * PAIR, kt & 1), ident);
             const Frag<T> dSf = transpose(dST, ident);
             const Frag<T> doN = tokf(0, vt);
             const Frag<T> vN = tokf(1, vt);
@@ -304,7 +348,8 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         const f32x4 q4 = to_f32(KEEP ? rq[KEEP ? kt : 0] : ld_frag_sel(at(p.q + qb, qo + 16 * kt * ES), rowok));
         const f32x4 a4[2] = {to_f32(KEEP ? ra[0][KEEP ? kt : 0] : ld_frag_sel(at(p.a + ab, ao0 + 16 * kt * ES), rowok)),
                              to_f32(KEEP ? ra[1][KEEP ? kt : 0] : ld_frag_sel(at(p.a + ab, ao1 + 16 * kt * ES), rowok))};
-        const f32x4 b4[2] = {to_f32(ld_frag_sel(at(p.b + ab, ao0 + 16 * kt * ES), rowok)), to_f32(ld_frag_sel(at(p.b + ab, ao1 + 16 * kt * ES), rowok))};
+        const f32x4 b4[2] = {to_f32(KEEP ? rb[0][KEEP ? kt : 0] : ld_frag_sel(at(p.b + ab, ao0 + 16 * kt * ES), rowok)),
+                             to_f32(KEEP ? rb[1][KEEP ? kt : 0] : ld_frag_sel(at(p.b + ab, ao1 + 16 * kt * ES), rowok))};
         const Frag<T> qhT = transpose(to_frag<T>(q4 * eq * scale), ident), khT = transpose(to_frag<T>(k4 * ek), ident);
         const Frag<T> ahT[2] = {transpose(to_frag<T>(a4[0] * ea), ident), transpose(to_frag<T>(a4[1] * ea), ident)};
         const Frag<T> bhT[2] = {transpose(to_frag<T>(b4[0] * ek), ident), transpose(to_frag<T>(b4[1] * ek), ident)};
