@@ -45,7 +45,7 @@ def interface_bytes(kernel, pass_, K, V, es, gs):
     output written once (es = bytes per element of the inputs, gs = bytes per element of gk)."""
     W, UT, KGT, BGT, VTT, EGL = 32 * K * es, 32 * V * es, 16 * K * es, 32 * K * es, 16 * V * es, 4 * K
     QG, AQK, AQB = 16 * K * es, 256 * es, 512 * es
-    AQBT, BG, WT, QGT, TM = 512 * es, 32 * K * es, 32 * K * es, 16 * K * es, 4096
+    AQBT, BG, WT, QGT, TM = 512 * es, 32 * K * es, 32 * K * es, 16 * K * es, 1024 * es
     HC = DHC = K * V * es
     VN = DVN = 32 * V * es
     inputs = 2 * 16 * K * es + 16 * K * gs + 2 * 32 * K * es + 16 * V * es          # q,k,gk,a,b,v

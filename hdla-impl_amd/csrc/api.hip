@@ -60,7 +60,7 @@ int make_layout(const hdla_dims* d, int pass, WsLayout& L, int& nch) {
         const size_t sb = take(chw * (size_t)bb.SIZE);
         L.SB_STRIDE = bb.SIZE;
         L.BG = sb + bb.BG; L.WT = sb + bb.WT; L.QGT = sb + bb.QGT; L.AQBT = sb + bb.AQBT; L.EGLB = sb + bb.EGL;
-        L.TM = take(chw * 1024 * 4);
+        L.TM = take(chw * 1024 * es);
         L.HC = take(chw * K * V * es);
         L.DHC = take(chw * K * V * es);
         L.VN = take(chw * 2 * 16 * V * es);
@@ -84,7 +84,7 @@ void bind_ws(ChunkArgs<T>& a, const hdla_dims* d, const WsLayout& L, int nch, vo
     a.ws.HC = at(L.HC); a.ws.DHC = at(L.DHC); a.ws.VN = at(L.VN); a.ws.DVN = at(L.DVN);
     a.ws.EGL = reinterpret_cast<float*>(base + L.EGL);
     a.ws.EGLB = reinterpret_cast<float*>(base + L.EGLB);
-    a.ws.TM = reinterpret_cast<float*>(base + L.TM);
+    a.ws.TM = reinterpret_cast<T*>(base + L.TM);
     a.st.cu = d->cu_seqlens;
     a.st.chunk_off = d->cu_seqlens ? reinterpret_cast<const int32_t*>(base + L.CHUNK_OFF) : nullptr;
     a.st.chunk_seq = d->cu_seqlens ? reinterpret_cast<const int32_t*>(base + L.CHUNK_SEQ) : nullptr;

@@ -23,7 +23,7 @@ template <typename T, bool GKF32, int K, int V>
 __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     constexpr int KT = K / 16, VT = V / 16;
     constexpr int SFS = blk_fwd(K, sizeof(T), false).SIZE / (int)sizeof(T);   // elements between slots of the scan block
-    __shared__ __attribute__((aligned(16))) float sT[32 * LDG];   // (I - A_ab)^-1, rank-major
+    __shared__ __attribute__((aligned(16))) float sT[32 * LDG];   // 4608 bytes: stash of the transposed score-gradient tiles
     // do, v, v_new (2 ranks) and dv_new (2 ranks) of the chunk, [matrix][token][value], staged once: every one of
     // them is an operand of several products in every pass, and the working set of the resident waves is far
     // larger than the L2, so repeated global loads would mostly be repeated HBM reads
@@ -109,25 +109,11 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         }
     }
     auto tokf = [&](int m, int vt) __attribute__((always_inline)) { return ld_frag(&sTok[(m * CH + c) * VP + 16 * vt + 4 * g]); };
-    {
-        const float* tmw = p.ws.TM + chw * 1024;
-        const int row = l >> 1, c0 = (l & 1) * 16;
-#pragma unroll
-        for (int x = 0; x < 4; ++x)
-            *reinterpret_cast<f32x4*>(&sT[row * LDG + c0 + 4 * x]) = *reinterpret_cast<const f32x4*>(tmw + row * 32 + c0 + 4 * x);
-    }
-    __syncthreads();
-    // tmT[s][r] = F((Tm^{s r})^T): lane (g,c) reg i = Tm^{s r}[4g+i][c]
+    // tmT[s][r] = F((Tm^{s r})^T): lane (g,c) reg i = Tm^{s r}[4g+i][c], stored in this form by the prep kernel
     Frag<T> tmT[2][2];
 #pragma unroll
-    for (int s = 0; s < 2; ++s)
-#pragma unroll
-        for (int r = 0; r < 2; ++r) {
-            f32x4 t;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) t[i] = sT[(16 * s + 4 * g + i) * LDG + 16 * r + c];
-            tmT[s][r] = to_frag<T>(t);
-        }
+    for (int s = 0; s < 2; ++s) ld_pair(p.ws.TM + chw * 1024 + s * PAIR, tmT[s][0], tmT[s][1]);
+    __syncthreads();
 
     // ---- cumulative decays; A_qk^T and A_ak^T (rows j, inner i) -----------------------------------------------
     // (the decays are recomputed per channel tile wherever they are needed: a load and four DPP additions cost
@@ -255,8 +241,7 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         if (!(j < c)) { dAak[0][i] = 0.f; dAak[1][i] = 0.f; dAab[0][0][i] = 0.f; dAab[0][1][i] = 0.f; dAab[1][0][i] = 0.f; dAab[1][1][i] = 0.f; }
     }
     // The transposed tiles are needed once per channel tile of the second pass.  For 2-byte elements the nine of
-    // them fit exactly into the LDS that held (I - A_ab)^-1 (no longer needed) and are read back where used: 18
-    // registers less across the second pass, which is what lets two waves share a SIMD.
+    // them are kept in LDS (4608 bytes) and read back where used: 18 registers less across the second pass.
     constexpr bool STASH = sizeof(T) == 2;
     T* stash = reinterpret_cast<T*>(sT);
     const Frag<T> fAqk = to_frag<T>(dAqk);

@@ -71,7 +71,7 @@ struct WsLayout {
     size_t QGT;    // tiles  [K/16]      F(qg^T)       rows channel, inner token
     size_t EGLB;   // fp32   [K]         exp(g_last), copy inside the reverse-scan block
     size_t SA_STRIDE, SB_STRIDE;   // bytes between consecutive (chunk, head) slots of the two scan blocks
-    size_t TM;     // fp32   [32][32]    (I - A_ab)^-1 in rank-major order (row r*16+i, column s*16+j)
+    size_t TM;     // tiles  [2][2]      F((Tm^{s r})^T), Tm = (I - A_ab)^-1 in 16x16 blocks: rows j, inner i
     size_t HC;     // rows   [K][V]      state entering the chunk
     size_t DHC;    // rows   [K][V]      gradient of the state leaving the chunk
     size_t VN;     // rows   [2][16][V]  v_new, rank-major
@@ -85,7 +85,8 @@ struct WsLayout {
 template <typename T>
 struct Ws {
     T *W, *UT, *KGT, *BGT, *VTT, *QG, *AQK, *AQB, *AQBT, *BG, *WT, *QGT, *HC, *DHC, *VN, *DVN;
-    float *EGL, *EGLB, *TM;
+    float *EGL, *EGLB;
+    T* TM;
 };
 
 template <typename T>

@@ -134,15 +134,13 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2)
             tm[s][s2] = to_frag<T>(*reinterpret_cast<const f32x4*>(&sT[(16 * s + c) * LDP + 16 * s2 + 4 * g]));
-    if (BWD) {
-        float* tmw = p.ws.TM + chw * 1024;
-        const int row = l >> 1, c0 = (l & 1) * 16;
-#pragma unroll
-        for (int x = 0; x < 4; ++x)
-            *reinterpret_cast<f32x4*>(tmw + row * 32 + c0 + 4 * x) = *reinterpret_cast<const f32x4*>(&sT[row * LDP + c0 + 4 * x]);
-    }
-
     const Frag<T> ident = ident_frag<T>();
+    if (BWD) {
+        // for the chunk_grad kernel: the four blocks transposed, as fragments (two tile pairs), ready to load
+        T* tmw = p.ws.TM + chw * 1024;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) st_pair2(tmw + s * PAIR, transpose(tm[s][0], ident), transpose(tm[s][1], ident));
+    }
 
     // ---- phase C: w = Tm ag and the gated copies, two channel tiles (one stored pair) at a time -----------------
 #pragma unroll

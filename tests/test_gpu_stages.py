@@ -67,7 +67,7 @@ def test_workspace_buffers_backward_pass(B, T, H, K, V, dtype):
         "BG": (G.cat_tiles(G.pair_tiles(ws, L["BG"], dtype, H, nch, 2, KT, stride=SB), 3), bh(p["bg"])),
         "WT": (G.cat_tiles(G.pair_tiles(ws, L["WT"], dtype, H, nch, 2, KT, stride=SB), 3, transpose=True), bh(p["w"])),
         "QGT": (G.cat_tiles(G.pair_tiles(ws, L["QGT"], dtype, H, nch, KT, stride=SB), 2, transpose=True), bh(p["qg"])),
-        "TM": (G.rows(ws, L["TM"], torch.float32, H, nch, 2, 16, 2, 16), bh(p["Tm"]).permute(0, 1, 2, 4, 3, 5)),
+        "TM": (G.pair_tiles(ws, L["TM"], dtype, H, nch, 2, 2), bh(p["Tm"]).transpose(-1, -2)),   # tiles hold the blocks transposed
         "HC": (state(L["HC"]), bh(f["h"])),
         "VN": (vnew(L["VN"]), bh(f["vn"])),
         "DHC": (state(L["DHC"]), bh(r["dh"])),
