@@ -84,6 +84,18 @@ def test_forward_backward_parity(dtype, B, T, H, K, V, gk_div, scale):
     _compare(_gpu(inp, dtype, scale), _oracle(inp, dtype, scale), dtype, what=f"{dtype} B{B} T{T} H{H} K{K} V{V}")
 
 
+@pytest.mark.parametrize("B,H,K,V", [(1, 40, 64, 64), (3, 24, 64, 64), (1, 136, 64, 64), (2, 20, 128, 128), (1, 72, 64, 128),
+                                     (2, 68, 128, 64)])
+def test_every_split_of_the_scans(B, H, K, V):
+    """The scans spread a head's value columns over 4, 2 or 1 workgroups depending on how many (sequence, head)
+    pairs there are (so that the launch has about one workgroup per compute unit), separately for the forward
+    scan (one direction) and the backward pair (two): these head counts reach every variant for both."""
+    T, dtype = 120, torch.bfloat16                # seven full chunks and a ragged one: ring loop and remainder loop
+    inp = make_inputs(300 + H, B, T, H, K, V, gk_div=2.0)
+    heads = [0, 1, H // 2, H - 1]                 # the oracle on a few heads is enough: heads are independent
+    _compare(_gpu(inp, dtype, 0.9), _oracle(inp, dtype, 0.9, heads=heads), dtype, heads=heads, what=f"split B{B} H{H} K{K} V{V}")
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_no_initial_state_no_final_gradient(dtype):
     inp = make_inputs(7, 2, 48, 2, 64, 64)
