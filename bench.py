@@ -54,14 +54,14 @@ def interface_bytes(kernel, pass_, K, V, es, gs):
         return inputs + out
     if kernel == "scan_fwd":
         rd = W + UT + KGT + BGT + VTT + EGL
-        return rd + (QG + AQK + AQB + 16 * V * es if pass_ == 0 else HC + VN)
+        return rd + (QG + AQK + AQB + 16 * V * es if pass_ == 0 else HC)
     if kernel == "scan_bwd":
         return AQBT + BG + WT + QGT + EGL + 16 * V * es + DHC + DVN
     if kernel == "scan_pair":           # both scans of the backward pass in one launch
         return interface_bytes("scan_fwd", 1, K, V, es, gs) + interface_bytes("scan_bwd", 1, K, V, es, gs)
     if kernel == "chunk_grad":
         outs = 2 * 16 * K * es + 16 * K * gs + 2 * 32 * K * es + 16 * V * es
-        return inputs + 16 * V * es + TM + W + UT + HC + DHC + VN + DVN + outs
+        return inputs + 16 * V * es + TM + W + UT + HC + DHC + DVN + outs
     raise ValueError(kernel)
 
 

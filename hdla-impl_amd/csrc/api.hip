@@ -63,7 +63,6 @@ int make_layout(const hdla_dims* d, int pass, WsLayout& L, int& nch) {
         L.TM = take(chw * 1024 * es);
         L.HC = take(chw * K * V * es);
         L.DHC = take(chw * K * V * es);
-        L.VN = take(chw * 2 * 16 * V * es);
         L.DVN = take(chw * 2 * 16 * V * es);
     }
     if (d->cu_seqlens) {
@@ -81,7 +80,7 @@ void bind_ws(ChunkArgs<T>& a, const hdla_dims* d, const WsLayout& L, int nch, vo
     a.ws.W = at(L.W); a.ws.UT = at(L.UT); a.ws.KGT = at(L.KGT); a.ws.BGT = at(L.BGT); a.ws.VTT = at(L.VTT);
     a.ws.QG = at(L.QG); a.ws.AQK = at(L.AQK); a.ws.AQB = at(L.AQB);
     a.ws.AQBT = at(L.AQBT); a.ws.BG = at(L.BG); a.ws.WT = at(L.WT); a.ws.QGT = at(L.QGT);
-    a.ws.HC = at(L.HC); a.ws.DHC = at(L.DHC); a.ws.VN = at(L.VN); a.ws.DVN = at(L.DVN);
+    a.ws.HC = at(L.HC); a.ws.DHC = at(L.DHC); a.ws.DVN = at(L.DVN);
     a.ws.EGL = reinterpret_cast<float*>(base + L.EGL);
     a.ws.EGLB = reinterpret_cast<float*>(base + L.EGLB);
     a.ws.TM = reinterpret_cast<T*>(base + L.TM);
@@ -190,7 +189,7 @@ int hdla_workspace_layout(const hdla_dims* dims, int pass, hdla_ws_layout* out) 
     out->QG = L.QG; out->AQK = L.AQK; out->AQB = L.AQB;
     out->AQBT = L.AQBT; out->BG = L.BG; out->WT = L.WT; out->QGT = L.QGT; out->TM = L.TM;
     out->EGLB = L.EGLB; out->SA_STRIDE = L.SA_STRIDE; out->SB_STRIDE = L.SB_STRIDE;
-    out->HC = L.HC; out->DHC = L.DHC; out->VN = L.VN; out->DVN = L.DVN;
+    out->HC = L.HC; out->DHC = L.DHC; out->DVN = L.DVN;
     out->CHUNK_OFF = L.CHUNK_OFF; out->CHUNK_SEQ = L.CHUNK_SEQ;
     out->total = L.total;
     return HDLA_OK;

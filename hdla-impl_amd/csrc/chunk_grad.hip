@@ -56,7 +56,6 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     const float scale = p.scale;
     const T* HC = p.ws.HC + chw * (K * V);
     const T* DHC = p.ws.DHC + chw * (K * V);
-    const T* VN = p.ws.VN + chw * (2 * CH * V);
     const T* DVN = p.ws.DVN + chw * (2 * CH * V);
     const int blk = blockIdx.y * gridDim.x + blockIdx.x;
     PHASE_CLOCK(p, blk, 0);
@@ -66,6 +65,17 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     // loads are the first thing issued, so that they travel together with the staging loads below: a wave spends
     // most of its time waiting for memory, and every dependent round trip to HBM costs thousands of cycles.
     constexpr bool KEEP = sizeof(T) == 2;
+    // The smallest shape also keeps the whole checkpoint of S (all its tile pairs) from here to the end of the
+    // first pass over channel tiles; the other shapes read it tile by tile where it is used.
+    constexpr bool PF = sizeof(T) == 2 && K == 64 && V == 64;
+    constexpr int KT2 = KT / 2;
+    Frag<T> hcall[PF ? KT2 : 1][PF ? VT : 1][2];
+    if (PF) {
+#pragma unroll
+        for (int kp = 0; kp < KT2; ++kp)
+#pragma unroll
+            for (int vt = 0; vt < VT; ++vt) ld_pair(HC + (kp * VT + vt) * PAIR, hcall[PF ? kp : 0][PF ? vt : 0][0], hcall[PF ? kp : 0][PF ? vt : 0][1]);
+    }
     Frag<T> rq[KEEP ? KT : 1], rk[KEEP ? KT : 1], ra[2][KEEP ? KT : 1];
     f32x4 rg[KEEP ? KT : 1];
     if (KEEP) {
@@ -94,16 +104,38 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
                 if (r >= cp.len) x = (i32x4){0, 0, 0, 0};
                 *reinterpret_cast<i32x4*>(&sTok[(m * CH + r) * VP + e]) = x;
             }
-        // v_new and dv_new: the scans left them as fragments of the transposed tiles (rows value, inner token), the
-        // two ranks of a value tile paired; one transposing product each gives the rows
+        // dv_new: the reverse scan left it as fragments of the transposed tiles (rows value, inner token), the two
+        // ranks of a value tile paired; one transposing product each gives the rows.
+        // v_new is not checkpointed by the scan: v_new_s = w_s S + u_s is rebuilt here from the checkpoint of S, which
+        // is stored as exactly the operand this product needs (fragments of S^T), with the same bf16 operands and
+        // fp32 accumulation as in the scan.
+        Frag<T> wf[2][KT];
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int kp = 0; kp < KT / 2; ++kp)
+                ld_pair(p.ws.W + chw * SFS + (s * (KT / 2) + kp) * PAIR, wf[s][2 * kp], wf[s][2 * kp + 1]);
 #pragma unroll(sizeof(T) * V >= 512 ? 1 : VT)
         for (int vt = 0; vt < VT; ++vt) {
-            Frag<T> x0, x1, y0, y1;
-            ld_pair(VN + vt * PAIR, x0, x1);
+            Frag<T> u0, u1, y0, y1;
+            ld_pair(p.ws.UT + (chw * VT + vt) * PAIR, u0, u1);
             ld_pair(DVN + vt * PAIR, y0, y1);
+            f32x4 vn0 = zero4(), vn1 = zero4();
+#pragma unroll
+            for (int kp = 0; kp < KT / 2; ++kp) {
+                Frag<T> h0, h1;
+                if (PF) { h0 = hcall[PF ? kp : 0][PF ? vt : 0][0]; h1 = hcall[PF ? kp : 0][PF ? vt : 0][1]; }
+                else ld_pair(HC + (kp * VT + vt) * PAIR, h0, h1);
+                vn0 = mm(wf[0][2 * kp], h0, vn0);
+                vn1 = mm(wf[1][2 * kp], h0, vn1);
+                vn0 = mm(wf[0][2 * kp + 1], h1, vn0);
+                vn1 = mm(wf[1][2 * kp + 1], h1, vn1);
+            }
+            vn0 += to_f32(transpose(u0, ident));
+            vn1 += to_f32(transpose(u1, ident));
             T* dst = &sTok[c * VP + 16 * vt + 4 * g];
-            st_frag(dst + 2 * CH * VP, transpose(x0, ident));
-            st_frag(dst + 3 * CH * VP, transpose(x1, ident));
+            st_frag(dst + 2 * CH * VP, to_frag<T>(vn0));
+            st_frag(dst + 3 * CH * VP, to_frag<T>(vn1));
             st_frag(dst + 4 * CH * VP, transpose(y0, ident));
             st_frag(dst + 5 * CH * VP, transpose(y1, ident));
         }
@@ -144,17 +176,13 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     const Frag<T> aqkTf = to_frag<T>(aqkT);
     const Frag<T> aakTf[2] = {to_frag<T>(aakT[0]), to_frag<T>(aakT[1])};
 
-    // Checkpoints of the state (and, for the second pass, of its gradient) arrive a pair of channel tiles ahead of
-    // their use: [buffer][value tile][tile of the pair].  The first pair is requested here, before the loop over
-    // the value dimension, whose work covers the trip.  2-byte types only (registers).
-    constexpr bool PF = sizeof(T) == 2 && K == 64 && V == 64;
-    constexpr int KT2 = KT / 2;
+    // In the second pass the checkpoints of the state and of its gradient arrive a pair of channel tiles ahead of
+    // their use: [buffer][value tile][tile of the pair].
     Frag<T> hcp[PF ? 2 : 1][PF ? VT : 1][2], dhp[PF ? 2 : 1][PF ? VT : 1][2];
     auto fetch_pairs = [&](const T* src, Frag<T> (&dst)[PF ? VT : 1][2], int kp) __attribute__((always_inline)) {
 #pragma unroll
         for (int vt = 0; vt < VT; ++vt) ld_pair(src + (kp * VT + vt) * PAIR, dst[PF ? vt : 0][0], dst[PF ? vt : 0][1]);
     };
-    if (PF) fetch_pairs(HC, hcp[0], 0);
     PHASE_CLOCK(p, blk, 1);
     // ---- products over the value dimension -------------------------------------------------------------------
     f32x4 dAqk = zero4(), dAqb[2] = {zero4(), zero4()}, dAak[2] = {zero4(), zero4()};
@@ -199,11 +227,10 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     // ---- first pass over channel tiles: dw -> dag -> the w part of dA_ab (dag itself is rebuilt in pass two) ----
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
-        if (PF && !(kt & 1) && kt / 2 + 1 < KT2) fetch_pairs(HC, hcp[PF ? (kt / 2 + 1) & 1 : 0], kt / 2 + 1);
         f32x4 dwT[2] = {zero4(), zero4()};                // rows channel, inner token
 #pragma unroll
         for (int vt = 0; vt < VT; ++vt) {
-            const Frag<T> Sf = transpose(PF ? hcp[PF ? (kt / 2) & 1 : 0][PF ? vt : 0][kt & 1]
+            const Frag<T> Sf = transpose(PF ? hcall[PF ? kt / 2 : 0][PF ? vt : 0][kt & 1]
                                             : ld_pair_one(HC + ((kt / 2) * VT + vt) * PAIR, kt & 1), ident);
             dwT[0] = mm(Sf, tokf(4, vt), dwT[0]);
             dwT[1] = mm(Sf, tokf(5, vt), dwT[1]);

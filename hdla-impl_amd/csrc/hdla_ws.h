@@ -72,10 +72,9 @@ struct WsLayout {
     size_t EGLB;   // fp32   [K]         exp(g_last), copy inside the reverse-scan block
     size_t SA_STRIDE, SB_STRIDE;   // bytes between consecutive (chunk, head) slots of the two scan blocks
     size_t TM;     // tiles  [2][2]      F((Tm^{s r})^T), Tm = (I - A_ab)^-1 in 16x16 blocks: rows j, inner i
-    size_t HC;     // rows   [K][V]      state entering the chunk
-    size_t DHC;    // rows   [K][V]      gradient of the state leaving the chunk
-    size_t VN;     // rows   [2][16][V]  v_new, rank-major
-    size_t DVN;    // rows   [2][16][V]  gradient of v_new, rank-major
+    size_t HC;     // tiles  [K/32][V/16] pairs  F(S^T), state entering the chunk: rows value, inner channel
+    size_t DHC;    // tiles  [K/32][V/16] pairs  the same for the gradient of the state leaving the chunk
+    size_t DVN;    // tiles  [V/16] pairs        F(dv_new_s^T), the two ranks paired: rows value, inner token
     // chunk table (only with cu_seqlens)
     size_t CHUNK_OFF;  // int32 [N+1]
     size_t CHUNK_SEQ;  // int32 [nch]
@@ -84,7 +83,7 @@ struct WsLayout {
 
 template <typename T>
 struct Ws {
-    T *W, *UT, *KGT, *BGT, *VTT, *QG, *AQK, *AQB, *AQBT, *BG, *WT, *QGT, *HC, *DHC, *VN, *DVN;
+    T *W, *UT, *KGT, *BGT, *VTT, *QG, *AQK, *AQB, *AQBT, *BG, *WT, *QGT, *HC, *DHC, *DVN;
     float *EGL, *EGLB;
     T* TM;
 };

@@ -125,14 +125,19 @@ __device__ __forceinline__ void memory_wave(char* smem, int nsteps, int hw, BlkF
     out(nsteps - 1);
 }
 
-// LDS of a scan workgroup: the three operand slots, then (with memory waves) two outboxes.  An outbox of the
-// backward pass is the workgroup's part of the chunk's checkpoint record: [K/32][NWC] tile pairs of the state, then
-// [NWC] tile pairs of v_new (1 KiB a pair for 2-byte elements).  An outbox of the forward pass is the workgroup's
-// 16 x (16 NWC) piece of the output rows, padded by 16 bytes a row against bank conflicts.
-template <typename T, int K, int V, int NWC, int SLOT_, bool WRITE_O> struct ScanLds {
+// LDS of a scan workgroup: the three operand slots, then (with memory waves) two outboxes.  What an outbox holds:
+//   OUT_O      forward pass: the workgroup's 16 x (16 NWC) piece of the output rows, padded by 16 bytes a row
+//              against bank conflicts;
+//   OUT_STATE  forward scan of the backward pass: the workgroup's part of the chunk's state checkpoint,
+//              [K/32][NWC] tile pairs (1 KiB a pair for 2-byte elements).  v_new is not checkpointed: the
+//              chunk_grad kernel rebuilds it from this checkpoint, w and u;
+//   OUT_GRAD   reverse scan: the same for dS, followed by [NWC] tile pairs of dv_new.
+enum ScanOut { OUT_O, OUT_STATE, OUT_GRAD };
+template <typename T, int K, int V, int NWC, int SLOT_, ScanOut OUT> struct ScanLds {
     static constexpr int ES = sizeof(T), NM = ScanCfg<T, K, V, NWC>::NM, SLOT = SLOT_;
     static constexpr int OROW = 16 * NWC * ES + 16;
-    static constexpr int OB_HC = (K / 32) * NWC * PAIR * ES, OB = WRITE_O ? CH * OROW : OB_HC + NWC * PAIR * ES;
+    static constexpr int OB_HC = (K / 32) * NWC * PAIR * ES;
+    static constexpr int OB = OUT == OUT_O ? CH * OROW : OUT == OUT_STATE ? OB_HC : OB_HC + NWC * PAIR * ES;
     static constexpr int BYTES = NSLOT * SLOT + (NM ? 2 * OB : 0);
 };
 
@@ -145,7 +150,7 @@ __device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem,
     constexpr bool PIPE = C::pipelined(WRITE_O);
     constexpr bool PIPE_UPD = PIPE && C::early_update_reads();
     constexpr int NI = B.SIZE / 1024, SLOT = B.SIZE;
-    typedef ScanLds<T, K, V, NWC, SLOT, WRITE_O> L;
+    typedef ScanLds<T, K, V, NWC, SLOT, WRITE_O ? OUT_O : OUT_STATE> L;
     constexpr int OROW = L::OROW, OB_HC = L::OB_HC, OB = L::OB;
     char* const outbox = smem + NSLOT * SLOT;
 
@@ -187,15 +192,13 @@ __device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem,
                 }
             } else {
                 char* hc = reinterpret_cast<char*>(p.ws.HC + (chw0 + cid) * (K * V) + vt0 * PAIR);
-                char* vn = reinterpret_cast<char*>(p.ws.VN + (chw0 + cid) * (2 * CH * V) + vt0 * PAIR);
-                constexpr int NP = OB / 1024, NPH = OB_HC / 1024;
+                constexpr int NP = OB / 1024;
 #pragma unroll
                 for (int j = 0; j < (NP + (NM ? NM : 1) - 1) / (NM ? NM : 1); ++j) {
                     const int i = hw + j * (NM ? NM : 1);
-                    if (i < NP) {
-                        char* dst = i < NPH ? hc + ((i / NWC) * VT + i % NWC) * 1024 : vn + (i - NPH) * 1024;
-                        *reinterpret_cast<i32x4*>(dst + l * 16) = *reinterpret_cast<const i32x4*>(ob + i * 1024 + l * 16);
-                    }
+                    if (i < NP)
+                        *reinterpret_cast<i32x4*>(hc + ((i / NWC) * VT + i % NWC) * 1024 + l * 16) =
+                            *reinterpret_cast<const i32x4*>(ob + i * 1024 + l * 16);
                 }
             }
         });
@@ -300,14 +303,12 @@ __device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem,
         }
         const Frag<T> vnb[2] = {to_frag<T>(vn[0]), to_frag<T>(vn[1])};
         if (!WRITE_O) {
-            // checkpoint of the entering state and v_new, as the fragments held here (tile pairs, 16 bytes per
-            // lane, whole cache lines): the chunk_grad kernel turns them the way it needs them
+            // checkpoint of the entering state, as the fragments held here (tile pairs, 16 bytes per lane, whole
+            // cache lines): the chunk_grad kernel turns them the way it needs them
             T* hc = NM ? reinterpret_cast<T*>(ob) + wv * PAIR : p.ws.HC + chw * (K * V) + vt * PAIR;
-            T* vnp = NM ? reinterpret_cast<T*>(ob + OB_HC) + wv * PAIR : p.ws.VN + chw * (2 * CH * V) + vt * PAIR;
             constexpr int HSTR = (NM ? NWC : VT) * PAIR;  // elements between the pairs of consecutive channel tiles
 #pragma unroll
             for (int kp = 0; kp < KT2; ++kp) st_pair2(hc + kp * HSTR, sb[2 * kp], sb[2 * kp + 1]);
-            st_pair2(vnp, vnb[0], vnb[1]);
         }
         if (WRITE_O) {
             o = mm(aqb[0], vnb[0], o);
@@ -412,7 +413,7 @@ __device__ __forceinline__ void scan_bwd_body(const ChunkArgs<T>& p, char* smem,
     constexpr bool PIPE = C::pipelined(false);
     constexpr bool PIPE_UPD = PIPE && C::early_update_reads();
     constexpr int NI = B.SIZE / 1024, SLOT = B.SIZE;
-    typedef ScanLds<T, K, V, NWC, SLOT, false> L;
+    typedef ScanLds<T, K, V, NWC, SLOT, OUT_GRAD> L;
     constexpr int OB_HC = L::OB_HC, OB = L::OB;
     char* const outbox = smem + NSLOT * SLOT;
 
@@ -625,19 +626,19 @@ __device__ __forceinline__ void scan_bwd_body(const ChunkArgs<T>& p, char* smem,
 // grid = (H, N, directions * SPLIT); blockIdx.z = direction * SPLIT + split
 template <typename T, int K, int V, int NWC, bool WRITE_O>
 __global__ __launch_bounds__((ScanCfg<T, K, V, NWC>::THREADS)) void scan_fwd_kernel(ChunkArgs<T> p) {
-    __shared__ __attribute__((aligned(16))) char smem[ScanLds<T, K, V, NWC, blk_fwd(K, sizeof(T), WRITE_O).SIZE, WRITE_O>::BYTES];
+    __shared__ __attribute__((aligned(16))) char smem[ScanLds<T, K, V, NWC, blk_fwd(K, sizeof(T), WRITE_O).SIZE, WRITE_O ? OUT_O : OUT_STATE>::BYTES];
     scan_fwd_body<T, K, V, NWC, WRITE_O>(p, smem, blockIdx.z);
 }
 template <typename T, int K, int V, int NWC>
 __global__ __launch_bounds__((ScanCfg<T, K, V, NWC>::THREADS)) void scan_bwd_kernel(ChunkArgs<T> p) {
-    __shared__ __attribute__((aligned(16))) char smem[ScanLds<T, K, V, NWC, blk_bwd(K, sizeof(T)).SIZE, false>::BYTES];
+    __shared__ __attribute__((aligned(16))) char smem[ScanLds<T, K, V, NWC, blk_bwd(K, sizeof(T)).SIZE, OUT_GRAD>::BYTES];
     scan_bwd_body<T, K, V, NWC>(p, smem, blockIdx.z);
 }
 // Both scans of the backward pass in one launch: they depend on the prep kernel only, not on each other.
 template <typename T, int K, int V, int NWC>
 __global__ __launch_bounds__((ScanCfg<T, K, V, NWC>::THREADS)) void scan_pair_kernel(ChunkArgs<T> p) {
-    constexpr int NF = ScanLds<T, K, V, NWC, blk_fwd(K, sizeof(T), false).SIZE, false>::BYTES;
-    constexpr int NB = ScanLds<T, K, V, NWC, blk_bwd(K, sizeof(T)).SIZE, false>::BYTES;
+    constexpr int NF = ScanLds<T, K, V, NWC, blk_fwd(K, sizeof(T), false).SIZE, OUT_STATE>::BYTES;
+    constexpr int NB = ScanLds<T, K, V, NWC, blk_bwd(K, sizeof(T)).SIZE, OUT_GRAD>::BYTES;
     constexpr int SPLIT = ScanCfg<T, K, V, NWC>::SPLIT;
     __shared__ __attribute__((aligned(16))) char smem[NF > NB ? NF : NB];
     if (blockIdx.z < SPLIT) scan_fwd_body<T, K, V, NWC, false>(p, smem, blockIdx.z);

@@ -25,7 +25,7 @@ class HdlaDims(ctypes.Structure):
 
 class HdlaWsLayout(ctypes.Structure):
     _names = ["nch", "W", "UT", "KGT", "BGT", "VTT", "EGL", "QG", "AQK", "AQB", "AQBT", "BG", "WT", "QGT", "TM",
-              "HC", "DHC", "VN", "DVN", "EGLB", "SA_STRIDE", "SB_STRIDE", "CHUNK_OFF", "CHUNK_SEQ", "total"]
+              "HC", "DHC", "DVN", "EGLB", "SA_STRIDE", "SB_STRIDE", "CHUNK_OFF", "CHUNK_SEQ", "total"]
     _fields_ = [(n, ctypes.c_int64) for n in _names]
 
 

@@ -69,7 +69,7 @@ typedef struct hdla_dims {
  * with SB_STRIDE. */
 typedef struct hdla_ws_layout {
     int64_t nch;               /* chunk slots per head */
-    int64_t W, UT, KGT, BGT, VTT, EGL, QG, AQK, AQB, AQBT, BG, WT, QGT, TM, HC, DHC, VN, DVN;
+    int64_t W, UT, KGT, BGT, VTT, EGL, QG, AQK, AQB, AQBT, BG, WT, QGT, TM, HC, DHC, DVN;
     int64_t EGLB, SA_STRIDE, SB_STRIDE;
     int64_t CHUNK_OFF, CHUNK_SEQ;
     int64_t total;

@@ -50,7 +50,7 @@ def test_workspace_buffers_backward_pass(B, T, H, K, V, dtype):
         return t.permute(0, 1, 2, 4, 6, 3, 5).reshape(H, nch, K, V)
 
     def vnew(off):
-        """v_new / dv_new: tiles of the transposed matrices (rows value, inner token), the two ranks paired,
+        """dv_new: tiles of the transposed matrices (rows value, inner token), the two ranks paired,
         [V/16][pair] -> [H, nch, 2, 16, V]."""
         t = G.pair_tiles(ws, off, dtype, H, nch, VT, 2)                   # [.., vt, s, v, token]
         return t.permute(0, 1, 3, 5, 2, 4).reshape(H, nch, 2, 16, V)
@@ -69,7 +69,6 @@ def test_workspace_buffers_backward_pass(B, T, H, K, V, dtype):
         "QGT": (G.cat_tiles(G.pair_tiles(ws, L["QGT"], dtype, H, nch, KT, stride=SB), 2, transpose=True), bh(p["qg"])),
         "TM": (G.pair_tiles(ws, L["TM"], dtype, H, nch, 2, 2), bh(p["Tm"]).transpose(-1, -2)),   # tiles hold the blocks transposed
         "HC": (state(L["HC"]), bh(f["h"])),
-        "VN": (vnew(L["VN"]), bh(f["vn"])),
         "DHC": (state(L["DHC"]), bh(r["dh"])),
         "DVN": (vnew(L["DVN"]), bh(r["dvn"])),
     }
