@@ -65,8 +65,9 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     // loads are the first thing issued, so that they travel together with the staging loads below: a wave spends
     // most of its time waiting for memory, and every dependent round trip to HBM costs thousands of cycles.
     constexpr bool KEEP = sizeof(T) == 2;
-    // The smallest shape also keeps the whole checkpoint of S (all its tile pairs) from here to the end of the
-    // first pass over channel tiles; the other shapes read it tile by tile where it is used.
+    // The smallest shape also keeps the whole checkpoint of S (all its tile pairs) in registers from here to the
+    // end: it is used three times (v_new, first and second pass over channel tiles) and a later read would mostly
+    // come from HBM again; the other shapes read it tile by tile where it is used.
     constexpr bool PF = sizeof(T) == 2 && K == 64 && V == 64;
     constexpr int KT2 = KT / 2;
     Frag<T> hcall[PF ? KT2 : 1][PF ? VT : 1][2];
@@ -176,9 +177,9 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     const Frag<T> aqkTf = to_frag<T>(aqkT);
     const Frag<T> aakTf[2] = {to_frag<T>(aakT[0]), to_frag<T>(aakT[1])};
 
-    // In the second pass the checkpoints of the state and of its gradient arrive a pair of channel tiles ahead of
-    // their use: [buffer][value tile][tile of the pair].
-    Frag<T> hcp[PF ? 2 : 1][PF ? VT : 1][2], dhp[PF ? 2 : 1][PF ? VT : 1][2];
+    // In the second pass the checkpoint of the state gradient arrives a pair of channel tiles ahead of its use:
+    // [buffer][value tile][tile of the pair].
+    Frag<T> dhp[PF ? 2 : 1][PF ? VT : 1][2];
     auto fetch_pairs = [&](const T* src, Frag<T> (&dst)[PF ? VT : 1][2], int kp) __attribute__((always_inline)) {
 #pragma unroll
         for (int vt = 0; vt < VT; ++vt) ld_pair(src + (kp * VT + vt) * PAIR, dst[PF ? vt : 0][0], dst[PF ? vt : 0][1]);
@@ -248,10 +249,7 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
 
     // for the second pass: the first pair of S and dS tiles, and all of b (used there only), requested now
     Frag<T> rb[2][KEEP ? KT : 1];
-    if (PF) {
-        fetch_pairs(HC, hcp[0], 0);
-        fetch_pairs(DHC, dhp[0], 0);
-    }
+    if (PF) fetch_pairs(DHC, dhp[0], 0);
     if (KEEP) {
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt) {
@@ -304,10 +302,7 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     // ---- second pass over channel tiles: state products, score backward, final gradients ----------------------
 #pragma unroll(KEEP ? KT : 1)
     for (int kt = 0; kt < KT; ++kt) {
-        if (PF && !(kt & 1) && kt / 2 + 1 < KT2) {
-            fetch_pairs(HC, hcp[PF ? (kt / 2 + 1) & 1 : 0], kt / 2 + 1);
-            fetch_pairs(DHC, dhp[PF ? (kt / 2 + 1) & 1 : 0], kt / 2 + 1);
-        }
+        if (PF && !(kt & 1) && kt / 2 + 1 < KT2) fetch_pairs(DHC, dhp[PF ? (kt / 2 + 1) & 1 : 0], kt / 2 + 1);
         // (a) what the loop over value tiles needs: only kg of this channel tile
         const f32x4 g4 = KEEP ? rg[KEEP ? kt : 0] : ld_gk4<GKF32>(gkp + go + 16 * kt * GS, 0, rowok);
         const f32x4 gi = scan16_incl(g4);
@@ -324,7 +319,7 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         for (int vt = 0; vt < VT; ++vt) {
             // the scans checkpoint S and dS as fragments of the transposed tiles (rows value, inner channel)
             const Frag<T> dST = PF ? dhp[PF ? (kt / 2) & 1 : 0][PF ? vt : 0][kt & 1] : ld_pair_one(DHC + ((kt / 2) * VT + vt) * PAIR, kt & 1);
-            const Frag<T> Sf = transpose(PF ? hcp[PF ? (kt / 2) & 1 : 0][PF ? vt : 0][kt & 1]
+            const Frag<T> Sf = transpose(PF ? hcall[PF ? kt / 2 : 0][PF ? vt : 0][kt & 1]
                                             : ld_pair_one(HC + ((kt / 2) * VT + vt) * PAIR, kt & 1), ident);
             const Frag<T> dSf = transpose(dST, ident);
             const Frag<T> doN = tokf(0, vt);
