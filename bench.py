@@ -45,20 +45,20 @@ def interface_bytes(kernel, pass_, K, V, es, gs):
     output written once (es = bytes per element of the inputs, gs = bytes per element of gk)."""
     W, UT, KGT, BGT, VTT, EGL = 32 * K * es, 32 * V * es, 16 * K * es, 32 * K * es, 16 * V * es, 4 * K
     QG, AQK, AQB = 16 * K * es, 256 * es, 512 * es
-    AQBT, BG, WT, QGT, TM = 512 * es, 32 * K * es, 32 * K * es, 16 * K * es, 1024 * es
+    AQBT, QGT, TM = 512 * es, 16 * K * es, 1024 * es
     HC = DHC = K * V * es
     VN = DVN = 32 * V * es
     inputs = 2 * 16 * K * es + 16 * K * gs + 2 * 32 * K * es + 16 * V * es          # q,k,gk,a,b,v
     if kernel == "prep":
-        out = W + UT + KGT + BGT + VTT + EGL + ((QG + AQK + AQB) if pass_ == 0 else (AQBT + BG + WT + QGT + TM))
+        out = W + UT + KGT + BGT + VTT + EGL + ((QG + AQK + AQB) if pass_ == 0 else (AQBT + QGT + TM))
         return inputs + out
     if kernel == "scan_fwd":
         rd = W + UT + KGT + BGT + VTT + EGL
         return rd + (QG + AQK + AQB + 16 * V * es if pass_ == 0 else HC)
     if kernel == "scan_bwd":
-        return AQBT + BG + WT + QGT + EGL + 16 * V * es + DHC + DVN
-    if kernel == "scan_pair":           # both scans of the backward pass in one launch
-        return interface_bytes("scan_fwd", 1, K, V, es, gs) + interface_bytes("scan_bwd", 1, K, V, es, gs)
+        return AQBT + W + BGT + QGT + EGL + 16 * V * es + DHC + DVN
+    if kernel == "scan_pair":           # both scans of the backward pass in one launch; w, bg and the decay feed both
+        return interface_bytes("scan_fwd", 1, K, V, es, gs) + interface_bytes("scan_bwd", 1, K, V, es, gs) - (W + BGT + EGL)
     if kernel == "chunk_grad":
         outs = 2 * 16 * K * es + 16 * K * gs + 2 * 32 * K * es + 16 * V * es
         return inputs + 16 * V * es + TM + W + UT + HC + DHC + DVN + outs

@@ -59,7 +59,7 @@ int make_layout(const hdla_dims* d, int pass, WsLayout& L, int& nch) {
         const BlkB bb = blk_bwd(d->K, (int)es);
         const size_t sb = take(chw * (size_t)bb.SIZE);
         L.SB_STRIDE = bb.SIZE;
-        L.BG = sb + bb.BG; L.WT = sb + bb.WT; L.QGT = sb + bb.QGT; L.AQBT = sb + bb.AQBT; L.EGLB = sb + bb.EGL;
+        L.QGT = sb + bb.QGT; L.AQBT = sb + bb.AQBT;
         L.TM = take(chw * 1024 * es);
         L.HC = take(chw * K * V * es);
         L.DHC = take(chw * K * V * es);
@@ -79,10 +79,9 @@ void bind_ws(ChunkArgs<T>& a, const hdla_dims* d, const WsLayout& L, int nch, vo
     auto at = [&](size_t o) { return reinterpret_cast<T*>(base + o); };
     a.ws.W = at(L.W); a.ws.UT = at(L.UT); a.ws.KGT = at(L.KGT); a.ws.BGT = at(L.BGT); a.ws.VTT = at(L.VTT);
     a.ws.QG = at(L.QG); a.ws.AQK = at(L.AQK); a.ws.AQB = at(L.AQB);
-    a.ws.AQBT = at(L.AQBT); a.ws.BG = at(L.BG); a.ws.WT = at(L.WT); a.ws.QGT = at(L.QGT);
+    a.ws.AQBT = at(L.AQBT); a.ws.QGT = at(L.QGT);
     a.ws.HC = at(L.HC); a.ws.DHC = at(L.DHC); a.ws.DVN = at(L.DVN);
     a.ws.EGL = reinterpret_cast<float*>(base + L.EGL);
-    a.ws.EGLB = reinterpret_cast<float*>(base + L.EGLB);
     a.ws.TM = reinterpret_cast<T*>(base + L.TM);
     a.st.cu = d->cu_seqlens;
     a.st.chunk_off = d->cu_seqlens ? reinterpret_cast<const int32_t*>(base + L.CHUNK_OFF) : nullptr;
@@ -187,8 +186,8 @@ int hdla_workspace_layout(const hdla_dims* dims, int pass, hdla_ws_layout* out) 
     out->nch = nch;
     out->W = L.W; out->UT = L.UT; out->KGT = L.KGT; out->BGT = L.BGT; out->VTT = L.VTT; out->EGL = L.EGL;
     out->QG = L.QG; out->AQK = L.AQK; out->AQB = L.AQB;
-    out->AQBT = L.AQBT; out->BG = L.BG; out->WT = L.WT; out->QGT = L.QGT; out->TM = L.TM;
-    out->EGLB = L.EGLB; out->SA_STRIDE = L.SA_STRIDE; out->SB_STRIDE = L.SB_STRIDE;
+    out->AQBT = L.AQBT; out->QGT = L.QGT; out->TM = L.TM;
+    out->SA_STRIDE = L.SA_STRIDE; out->SB_STRIDE = L.SB_STRIDE;
     out->HC = L.HC; out->DHC = L.DHC; out->DVN = L.DVN;
     out->CHUNK_OFF = L.CHUNK_OFF; out->CHUNK_SEQ = L.CHUNK_SEQ;
     out->total = L.total;

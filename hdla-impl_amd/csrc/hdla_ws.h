@@ -27,11 +27,12 @@ struct SeqTab {
 // block per (chunk, head), so that a workgroup can copy a block into LDS with a few whole-kilobyte loads.
 // Byte offsets inside a block, by head size K, element size es and pass:
 //   forward-scan block:  W [2][K/16] | BGT [2][K/16] | KGT [K/16] | (QG [K/16] | AQB [2] | AQK [1]) | EGL fp32[K]
-//   reverse-scan block:  BG [2][K/16] | WT [2][K/16] | QGT [K/16] | AQBT [2] | EGL fp32[K]
+//   reverse-scan block:  QGT [K/16] | AQBT [2]       (the reverse scan also reads W, BGT and EGL of the forward-scan
+//                        block and turns the tiles of W and BGT itself)
 // (tiles of 256 elements in fragment order, consecutive tile pairs interleaved; the part in parentheses only in
 // the forward pass, where the scan also produces the output)
 struct BlkF { int W, BGT, KGT, QG, AQB, AQK, EGL, SIZE; };
-struct BlkB { int BG, WT, QGT, AQBT, EGL, SIZE; };
+struct BlkB { int QGT, AQBT, SIZE; };
 constexpr BlkF blk_fwd(int K, int es, bool with_o) {
     const int tb = 256 * es, KT = K / 16;
     BlkF b{};
@@ -44,13 +45,26 @@ constexpr BlkF blk_fwd(int K, int es, bool with_o) {
 constexpr BlkB blk_bwd(int K, int es) {
     const int tb = 256 * es, KT = K / 16;
     BlkB b{};
-    b.BG = 0; b.WT = 2 * KT * tb; b.QGT = 4 * KT * tb; b.AQBT = 5 * KT * tb; b.EGL = (5 * KT + 2) * tb;
-    b.SIZE = (b.EGL + 4 * K + 1023) & ~1023;
+    b.QGT = 0; b.AQBT = KT * tb;
+    b.SIZE = ((KT + 2) * tb + 1023) & ~1023;
     return b;
 }
 
+// LDS slot of the reverse scan, assembled from 1-KiB pieces of both blocks of a (chunk, head): W and BGT (the first
+// NIF pieces of the forward-scan block), the piece holding EGL, then the reverse-scan block.
+struct SlotB { int W, BGT, EGL, QGT, AQBT, SIZE, NIF, EGL_SRC; };
+constexpr SlotB slot_bwd(int K, int es) {
+    const int tb = 256 * es, KT = K / 16;
+    SlotB s{};
+    s.W = 0; s.BGT = 2 * KT * tb; s.NIF = 4 * KT * tb / 1024;
+    s.EGL = s.NIF * 1024; s.EGL_SRC = blk_fwd(K, es, false).EGL;      // EGL is 1 KiB aligned in the forward block
+    s.QGT = s.EGL + 1024; s.AQBT = s.QGT + KT * tb;
+    s.SIZE = s.QGT + blk_bwd(K, es).SIZE;
+    return s;
+}
+
 // Byte offsets into the caller's workspace; 0-sized entries are unused in the given pass.  The entries of the
-// two scan blocks (W .. EGL and BG .. EGLB) are the offsets of that part for (chunk, head) slot 0; consecutive
+// two scan blocks (W .. EGL and QGT, AQBT) are the offsets of that part for (chunk, head) slot 0; consecutive
 // slots are SA_STRIDE / SB_STRIDE bytes apart.
 struct WsLayout {
     // written by prep, read by the scans
@@ -66,10 +80,7 @@ struct WsLayout {
     size_t AQB;    // tiles  [2]         F(A_qb^s)     rows i, inner j
     // backward pass only
     size_t AQBT;   // tiles  [2]         F(A_qb^s^T)   rows j, inner i
-    size_t BG;     // tiles  [2][K/16]   F(bg_s)       rows token, inner channel
-    size_t WT;     // tiles  [2][K/16]   F(w_s^T)      rows channel, inner token
     size_t QGT;    // tiles  [K/16]      F(qg^T)       rows channel, inner token
-    size_t EGLB;   // fp32   [K]         exp(g_last), copy inside the reverse-scan block
     size_t SA_STRIDE, SB_STRIDE;   // bytes between consecutive (chunk, head) slots of the two scan blocks
     size_t TM;     // tiles  [2][2]      F((Tm^{s r})^T), Tm = (I - A_ab)^-1 in 16x16 blocks: rows j, inner i
     size_t HC;     // tiles  [K/32][V/16] pairs  F(S^T), state entering the chunk: rows value, inner channel
@@ -83,8 +94,8 @@ struct WsLayout {
 
 template <typename T>
 struct Ws {
-    T *W, *UT, *KGT, *BGT, *VTT, *QG, *AQK, *AQB, *AQBT, *BG, *WT, *QGT, *HC, *DHC, *DVN;
-    float *EGL, *EGLB;
+    T *W, *UT, *KGT, *BGT, *VTT, *QG, *AQK, *AQB, *AQBT, *QGT, *HC, *DHC, *DVN;
+    float *EGL;
     T* TM;
 };
 

@@ -145,7 +145,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 
     // ---- phase C: w = Tm ag and the gated copies, two channel tiles (one stored pair) at a time -----------------
 #pragma unroll
     for (int kp = 0; kp < KT2; ++kp) {
-        Frag<T> fw[2][2], fwT[2][2], fkgT[2], fbgT[2][2], fqg[2], fqgT[2], fbg[2][2];   // [..][tile of the pair]
+        Frag<T> fw[2][2], fkgT[2], fbgT[2][2], fqg[2], fqgT[2];   // [..][tile of the pair]
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const int kt = 2 * kp + e;
@@ -158,34 +158,22 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 
                 f32x4 w = mm(tm[s][0], agT[0], zero4());
                 w = mm(tm[s][1], agT[1], w);
                 fw[s][e] = to_frag<T>(w);
-                if (BWD) {
-                    f32x4 wT = mm(agT[0], tm[s][0], zero4());
-                    wT = mm(agT[1], tm[s][1], wT);
-                    fwT[s][e] = to_frag<T>(wT);
-                }
             }
             fqg[e] = to_frag<T>(to_f32(rq[kt]) * egi * scale);
             const Frag<T> kg = to_frag<T>(to_f32(rk[kt]) * edn);
-            fbg[0][e] = to_frag<T>(to_f32(rb[0][kt]) * edn);
-            fbg[1][e] = to_frag<T>(to_f32(rb[1][kt]) * edn);
             fkgT[e] = transpose(kg, ident);
-            fbgT[0][e] = transpose(fbg[0][e], ident);
-            fbgT[1][e] = transpose(fbg[1][e], ident);
+            fbgT[0][e] = transpose(to_frag<T>(to_f32(rb[0][kt]) * edn), ident);
+            fbgT[1][e] = transpose(to_frag<T>(to_f32(rb[1][kt]) * edn), ident);
             if (BWD) fqgT[e] = transpose(fqg[e], ident);
             if (c == 0) {
                 const f32x4 egl = exp4<T>(gl);
                 *reinterpret_cast<f32x4*>(p.ws.EGL + chw * (SAS * (int)sizeof(T) / 4) + 16 * kt + 4 * g) = egl;
-                if (BWD) *reinterpret_cast<f32x4*>(p.ws.EGLB + chw * (SBS * (int)sizeof(T) / 4) + 16 * kt + 4 * g) = egl;
             }
         }
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
             st_pair2(p.ws.W + chw * SAS + (s * KT2 + kp) * PAIR, fw[s][0], fw[s][1]);
             st_pair2(p.ws.BGT + chw * SAS + (s * KT2 + kp) * PAIR, fbgT[s][0], fbgT[s][1]);
-            if (BWD) {
-                st_pair2(p.ws.WT + chw * SBS + (s * KT2 + kp) * PAIR, fwT[s][0], fwT[s][1]);
-                st_pair2(p.ws.BG + chw * SBS + (s * KT2 + kp) * PAIR, fbg[s][0], fbg[s][1]);
-            }
         }
         st_pair2(p.ws.KGT + chw * SAS + kp * PAIR, fkgT[0], fkgT[1]);
         if (!BWD) st_pair2(p.ws.QG + chw * SAS + kp * PAIR, fqg[0], fqg[1]);

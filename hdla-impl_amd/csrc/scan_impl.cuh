@@ -65,16 +65,61 @@ template <typename T, int K, int V, int NWC> struct ScanCfg {
     static constexpr bool early_update_reads() { return KB <= 128 || (KB <= 256 && NWC <= 4 && NM == 0); }
 };
 
-// one wave's share of a shared operand block: the 1-KiB pieces w, w+NLD, ... of its NI pieces
-template <int NI, int NLD> struct Share {
+// A shared operand block as the loading waves see it: NI pieces of 1 KiB, lane l taking 16 bytes of each.  The
+// first NT pieces hold tiles that are handed to LDS transposed, so a lane must hold whole fragments of them: for
+// 2-byte elements a piece is a tile pair in its stored order; for 4-byte elements a piece is one tile of a pair,
+// 16 of every 32 bytes.
+template <int ES> __device__ __forceinline__ int piece_off(int i, int l, bool tiles) {
+    if (ES == 4 && tiles) return (i >> 1) * 2048 + l * 32 + (i & 1) * 16;
+    return i * 1024 + l * 16;
+}
+// the whole block is contiguous in global memory (forward scans)
+struct BlockOne {
+    const char* p;
+    __device__ __forceinline__ const char* piece(int i, int l, bool) const { return p + i * 1024 + l * 16; }
+};
+// reverse scan: W and BGT (NIF pieces) and the piece holding EGL come from the forward-scan block of the (chunk,
+// head), the rest is the reverse-scan block
+template <typename T, int K> struct BlockTwo {
+    const char *f, *r;
+    __device__ __forceinline__ const char* piece(int i, int l, bool tiles) const {
+        constexpr SlotB S = slot_bwd(K, sizeof(T));
+        static_assert(S.EGL_SRC % 1024 == 0, "EGL starts a piece");
+        if (i < S.NIF) return f + piece_off<sizeof(T)>(i, l, tiles);
+        if (i == S.NIF) return f + S.EGL_SRC + l * 16;
+        return r + (i - S.NIF - 1) * 1024 + l * 16;
+    }
+};
+
+// 16 bytes of fragments of type T, each tile transposed (a product with the identity: exact)
+template <typename T> __device__ __forceinline__ i32x4 transpose_piece(i32x4 x) {
+    const Frag<T> ident = ident_frag<T>();
+    if constexpr (sizeof(T) == 2) {
+        const s16x8 y = __builtin_bit_cast(s16x8, x);
+        Frag<T> f0, f1;
+        f0.v = __builtin_shufflevector(y, y, 0, 1, 2, 3);
+        f1.v = __builtin_shufflevector(y, y, 4, 5, 6, 7);
+        f0 = transpose(f0, ident);
+        f1 = transpose(f1, ident);
+        return __builtin_bit_cast(i32x4, __builtin_shufflevector(f0.v, f1.v, 0, 1, 2, 3, 4, 5, 6, 7));
+    } else {
+        Frag<T> f;
+        f.v = __builtin_bit_cast(f32x4, x);
+        return __builtin_bit_cast(i32x4, transpose(f, ident).v);
+    }
+}
+
+// one wave's share of a shared operand block: the pieces w, w+NLD, ... of its NI pieces
+template <typename T, int NI, int NLD, int NT = 0> struct Share {
     static constexpr int CNT = (NI + NLD - 1) / NLD;
+    static_assert(NT % NLD == 0 && NT < NI, "whether a piece is transposed must not depend on the wave");
     i32x4 a[CNT];
-    __device__ __forceinline__ void load(const char* blk, int w) {
+    template <typename Blk> __device__ __forceinline__ void load(const Blk& blk, int w) {
         const int l = lane_id();
 #pragma unroll
         for (int j = 0; j < CNT; ++j) {
             const int i = min(w + j * NLD, NI - 1);       // the last pieces may be fetched twice; never out of range
-            a[j] = *reinterpret_cast<const i32x4*>(blk + i * 1024 + l * 16);
+            a[j] = *reinterpret_cast<const i32x4*>(blk.piece(i, l, j * NLD < NT));
         }
     }
     __device__ __forceinline__ void to_lds(char* slot, int w) const {
@@ -82,7 +127,8 @@ template <int NI, int NLD> struct Share {
 #pragma unroll
         for (int j = 0; j < CNT; ++j) {
             const int i = min(w + j * NLD, NI - 1);
-            *reinterpret_cast<i32x4*>(slot + i * 1024 + l * 16) = a[j];
+            const bool tiles = j * NLD < NT;
+            *reinterpret_cast<i32x4*>(slot + piece_off<sizeof(T)>(i, l, tiles)) = tiles ? transpose_piece<T>(a[j]) : a[j];
         }
     }
 };
@@ -90,10 +136,10 @@ template <int NI, int NLD> struct Share {
 // A memory wave.  blk(t): block of step t (clamped to the last step by the caller); out(t): copy the outbox of
 // step t to global memory.  Barriers: one closing the prologue, one per step, one handing over the last outbox;
 // the computing waves execute exactly the same sequence.
-template <int NI, int NM, int DR, int SLOT, typename BlkFn, typename OutFn>
+template <typename T, int NI, int NM, int DR, int SLOT, int NT, typename BlkFn, typename OutFn>
 __device__ __forceinline__ void memory_wave(char* smem, int nsteps, int hw, BlkFn blk, OutFn out) {
     static_assert(DR % NSLOT == 0 && DR >= NSLOT, "ring depth must be a multiple of the slot count");
-    Share<NI, NM> sh[DR];
+    Share<T, NI, NM, NT> sh[DR];
 #pragma unroll
     for (int d = 0; d < DR; ++d) sh[d].load(blk(d), hw);
     sh[0].to_lds(smem, hw);
@@ -116,7 +162,7 @@ __device__ __forceinline__ void memory_wave(char* smem, int nsteps, int hw, BlkF
 #pragma unroll 1
     for (int t = nfull * DR; t < nsteps; ++t) {           // fewer than DR steps left: one block at a time
         lds_barrier();
-        Share<NI, NM> tmp;
+        Share<T, NI, NM, NT> tmp;
         tmp.load(blk(t + 2), hw);
         if (t > 0) out(t - 1);
         tmp.to_lds(smem + ((t + 2) % NSLOT) * SLOT, hw);
@@ -168,13 +214,13 @@ __device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem,
     // block of step t; steps past the end of the sequence are clamped, so every load is unconditional (a load
     // that may or may not have been issued would make the compiler wait for all outstanding loads)
     auto blk = [&](int t) __attribute__((always_inline)) {
-        return reinterpret_cast<const char*>(p.ws.W) + (chw0 + min(c0 + t, last)) * SLOT;
+        return BlockOne{reinterpret_cast<const char*>(p.ws.W) + (chw0 + min(c0 + t, last)) * SLOT};
     };
 
     if (NM && wv >= NWC) {
         if (nchunks <= 0) return;
         const int hw = wv - NWC;
-        memory_wave<NI, NM ? NM : 1, NM ? C::DR_SHARE : NSLOT, SLOT>(smem, nchunks, hw, blk, [&](int t) __attribute__((always_inline)) {
+        memory_wave<T, NI, NM ? NM : 1, NM ? C::DR_SHARE : NSLOT, SLOT, 0>(smem, nchunks, hw, blk, [&](int t) __attribute__((always_inline)) {
             const int cid = c0 + t;
             const char* ob = outbox + (t & 1) * OB;
             if (WRITE_O) {
@@ -335,7 +381,7 @@ __device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem,
         constexpr int DRO = C::DR_OWN, DRS = NM ? 0 : C::DR_SHARE;   // without memory waves both rings are one
         int done = 0;
         if constexpr (DRO > 0) {
-            Share<NI, NWC> sh[DRS ? DRS : 1];
+            Share<T, NI, NWC> sh[DRS ? DRS : 1];
             Own own[DRO];
 #pragma unroll
             for (int d = 0; d < DRO; ++d) {
@@ -369,7 +415,7 @@ __device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem,
             }
             done = nfull * DRO;
         } else {
-            Share<NI, NWC> tmp;
+            Share<T, NI, NWC> tmp;
             tmp.load(blk(0), wv);
             tmp.to_lds(smem, wv);
             tmp.load(blk(1), wv);
@@ -384,7 +430,7 @@ __device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem,
 #pragma unroll 1
             for (int t = done; t < nchunks; ++t) {
                 lds_barrier();
-                Share<NI, NWC> tmp;
+                Share<T, NI, NWC> tmp;
                 if (!NM) tmp.load(blk(t + 2), wv);
                 Own nxt;
                 load_own(nxt, t + 1);
@@ -409,7 +455,9 @@ template <typename T, int K, int V, int NWC>
 __device__ __forceinline__ void scan_bwd_body(const ChunkArgs<T>& p, char* smem, int split) {
     typedef ScanCfg<T, K, V, NWC> C;
     constexpr int KT = K / 16, KT2 = KT / 2, VT = V / 16, NM = C::NM, ES = sizeof(T);
-    constexpr BlkB B = blk_bwd(K, sizeof(T));
+    // LDS slot: [BG | WT] (BGT and W of the forward-scan block, transposed on their way in) | EGL | QGT | AQBT
+    constexpr SlotB B = slot_bwd(K, sizeof(T));
+    constexpr int SFWD = blk_fwd(K, sizeof(T), false).SIZE, SBWD = blk_bwd(K, sizeof(T)).SIZE, NT = B.NIF;
     constexpr bool PIPE = C::pipelined(false);
     constexpr bool PIPE_UPD = PIPE && C::early_update_reads();
     constexpr int NI = B.SIZE / 1024, SLOT = B.SIZE;
@@ -429,13 +477,14 @@ __device__ __forceinline__ void scan_bwd_body(const ChunkArgs<T>& p, char* smem,
     const int64_t chw0 = (int64_t)h * p.st.nch;
     const int nchunks = c1 - c0, first = c1 - 1;
     auto blk = [&](int t) __attribute__((always_inline)) {
-        return reinterpret_cast<const char*>(p.ws.BG) + (chw0 + max(first - t, c0)) * SLOT;
+        const int64_t slot = chw0 + max(first - t, c0);
+        return BlockTwo<T, K>{reinterpret_cast<const char*>(p.ws.W) + slot * SFWD, reinterpret_cast<const char*>(p.ws.QGT) + slot * SBWD};
     };
 
     if (NM && wv >= NWC) {
         if (nchunks <= 0) return;
         const int hw = wv - NWC;
-        memory_wave<NI, NM ? NM : 1, NM ? C::DR_SHARE : NSLOT, SLOT>(smem, nchunks, hw, blk, [&](int t) __attribute__((always_inline)) {
+        memory_wave<T, NI, NM ? NM : 1, NM ? C::DR_SHARE : NSLOT, SLOT, NT>(smem, nchunks, hw, blk, [&](int t) __attribute__((always_inline)) {
             const int cid = first - t;
             const char* ob = outbox + (t & 1) * OB;
             char* hc = reinterpret_cast<char*>(p.ws.DHC + (chw0 + cid) * (K * V) + vt0 * PAIR);
@@ -475,7 +524,7 @@ __device__ __forceinline__ void scan_bwd_body(const ChunkArgs<T>& p, char* smem,
 
     Frag<T> aq[2], bg[2][KT];                             // phase-1 operands; when pipelined, read a step ahead
     auto read_bg = [&](const char* slot, int kp) __attribute__((always_inline)) {
-        const T* sBG = reinterpret_cast<const T*>(slot + B.BG);
+        const T* sBG = reinterpret_cast<const T*>(slot + B.BGT);
         ld_pair(sBG + (0 * KT2 + kp) * PAIR, bg[0][2 * kp], bg[0][2 * kp + 1]);
         ld_pair(sBG + (1 * KT2 + kp) * PAIR, bg[1][2 * kp], bg[1][2 * kp + 1]);
     };
@@ -488,7 +537,7 @@ __device__ __forceinline__ void scan_bwd_body(const ChunkArgs<T>& p, char* smem,
     auto step = [&](const char* slot, const char* slot_next, char* ob, Frag<T> don, int t) __attribute__((always_inline)) {
         const int cid = first - t;
         const int64_t chw = chw0 + cid;
-        const T* sWT = reinterpret_cast<const T*>(slot + B.WT);
+        const T* sWT = reinterpret_cast<const T*>(slot + B.W);
         const T* sQGT = reinterpret_cast<const T*>(slot + B.QGT);
         const float* sEGL = reinterpret_cast<const float*>(slot + B.EGL);
         Frag<T> qgt[KT], wt[2][KT];
@@ -557,7 +606,7 @@ __device__ __forceinline__ void scan_bwd_body(const ChunkArgs<T>& p, char* smem,
         constexpr int DRO = C::DR_OWN, DRS = NM ? 0 : C::DR_SHARE;
         int done = 0;
         if constexpr (DRO > 0) {
-            Share<NI, NWC> sh[DRS ? DRS : 1];
+            Share<T, NI, NWC, NT> sh[DRS ? DRS : 1];
             Frag<T> own[DRO];
 #pragma unroll
             for (int d = 0; d < DRO; ++d) {
@@ -589,7 +638,7 @@ __device__ __forceinline__ void scan_bwd_body(const ChunkArgs<T>& p, char* smem,
             }
             done = nfull * DRO;
         } else {
-            Share<NI, NWC> tmp;
+            Share<T, NI, NWC, NT> tmp;
             tmp.load(blk(0), wv);
             tmp.to_lds(smem, wv);
             tmp.load(blk(1), wv);
@@ -603,7 +652,7 @@ __device__ __forceinline__ void scan_bwd_body(const ChunkArgs<T>& p, char* smem,
 #pragma unroll 1
             for (int t = done; t < nchunks; ++t) {
                 lds_barrier();
-                Share<NI, NWC> tmp;
+                Share<T, NI, NWC, NT> tmp;
                 if (!NM) tmp.load(blk(t + 2), wv);
                 Frag<T> nxt;
                 load_own(nxt, t + 1);
@@ -631,14 +680,14 @@ __global__ __launch_bounds__((ScanCfg<T, K, V, NWC>::THREADS)) void scan_fwd_ker
 }
 template <typename T, int K, int V, int NWC>
 __global__ __launch_bounds__((ScanCfg<T, K, V, NWC>::THREADS)) void scan_bwd_kernel(ChunkArgs<T> p) {
-    __shared__ __attribute__((aligned(16))) char smem[ScanLds<T, K, V, NWC, blk_bwd(K, sizeof(T)).SIZE, OUT_GRAD>::BYTES];
+    __shared__ __attribute__((aligned(16))) char smem[ScanLds<T, K, V, NWC, slot_bwd(K, sizeof(T)).SIZE, OUT_GRAD>::BYTES];
     scan_bwd_body<T, K, V, NWC>(p, smem, blockIdx.z);
 }
 // Both scans of the backward pass in one launch: they depend on the prep kernel only, not on each other.
 template <typename T, int K, int V, int NWC>
 __global__ __launch_bounds__((ScanCfg<T, K, V, NWC>::THREADS)) void scan_pair_kernel(ChunkArgs<T> p) {
     constexpr int NF = ScanLds<T, K, V, NWC, blk_fwd(K, sizeof(T), false).SIZE, OUT_STATE>::BYTES;
-    constexpr int NB = ScanLds<T, K, V, NWC, blk_bwd(K, sizeof(T)).SIZE, OUT_GRAD>::BYTES;
+    constexpr int NB = ScanLds<T, K, V, NWC, slot_bwd(K, sizeof(T)).SIZE, OUT_GRAD>::BYTES;
     constexpr int SPLIT = ScanCfg<T, K, V, NWC>::SPLIT;
     __shared__ __attribute__((aligned(16))) char smem[NF > NB ? NF : NB];
     if (blockIdx.z < SPLIT) scan_fwd_body<T, K, V, NWC, false>(p, smem, blockIdx.z);

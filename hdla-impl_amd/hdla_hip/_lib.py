@@ -24,8 +24,8 @@ class HdlaDims(ctypes.Structure):
 
 
 class HdlaWsLayout(ctypes.Structure):
-    _names = ["nch", "W", "UT", "KGT", "BGT", "VTT", "EGL", "QG", "AQK", "AQB", "AQBT", "BG", "WT", "QGT", "TM",
-              "HC", "DHC", "DVN", "EGLB", "SA_STRIDE", "SB_STRIDE", "CHUNK_OFF", "CHUNK_SEQ", "total"]
+    _names = ["nch", "W", "UT", "KGT", "BGT", "VTT", "EGL", "QG", "AQK", "AQB", "AQBT", "QGT", "TM",
+              "HC", "DHC", "DVN", "SA_STRIDE", "SB_STRIDE", "CHUNK_OFF", "CHUNK_SEQ", "total"]
     _fields_ = [(n, ctypes.c_int64) for n in _names]
 
 

@@ -65,12 +65,12 @@ typedef struct hdla_dims {
  * fragment order (element 4*lane + i of a block is row lane%16, inner index 4*(lane/16) + i; consecutive
  * tile pairs are stored interleaved, element 8*lane + 4*which + i), "rows" are row-major, all laid out
  * [H][nch][...].  W, BGT, KGT, QG, AQB, AQK, EGL are parts of one block per (head, chunk) slot: the value given
- * is the offset for slot 0 and consecutive slots are SA_STRIDE bytes apart; likewise BG, WT, QGT, AQBT, EGLB
+ * is the offset for slot 0 and consecutive slots are SA_STRIDE bytes apart; likewise QGT, AQBT
  * with SB_STRIDE. */
 typedef struct hdla_ws_layout {
     int64_t nch;               /* chunk slots per head */
-    int64_t W, UT, KGT, BGT, VTT, EGL, QG, AQK, AQB, AQBT, BG, WT, QGT, TM, HC, DHC, DVN;
-    int64_t EGLB, SA_STRIDE, SB_STRIDE;
+    int64_t W, UT, KGT, BGT, VTT, EGL, QG, AQK, AQB, AQBT, QGT, TM, HC, DHC, DVN;
+    int64_t SA_STRIDE, SB_STRIDE;
     int64_t CHUNK_OFF, CHUNK_SEQ;
     int64_t total;
 } hdla_ws_layout;

@@ -62,10 +62,7 @@ def test_workspace_buffers_backward_pass(B, T, H, K, V, dtype):
         "BGT": (G.cat_tiles(G.pair_tiles(ws, L["BGT"], dtype, H, nch, 2, KT, stride=SA), 3, transpose=True), bh(p["bg"])),
         "VTT": (G.cat_tiles(G.tiles(ws, L["VTT"], dtype, H, nch, VT), 2, transpose=True), bh(p["v"])),
         "EGL": (G.rows(ws, L["EGL"], torch.float32, H, nch, K, stride=SA), bh(torch.exp(p["gl"]))[..., 0, :]),
-        "EGLB": (G.rows(ws, L["EGLB"], torch.float32, H, nch, K, stride=SB), bh(torch.exp(p["gl"]))[..., 0, :]),
         "AQBT": (G.pair_tiles(ws, L["AQBT"], dtype, H, nch, 2, stride=SB), bh(p["Aqb"]).transpose(-1, -2)),
-        "BG": (G.cat_tiles(G.pair_tiles(ws, L["BG"], dtype, H, nch, 2, KT, stride=SB), 3), bh(p["bg"])),
-        "WT": (G.cat_tiles(G.pair_tiles(ws, L["WT"], dtype, H, nch, 2, KT, stride=SB), 3, transpose=True), bh(p["w"])),
         "QGT": (G.cat_tiles(G.pair_tiles(ws, L["QGT"], dtype, H, nch, KT, stride=SB), 2, transpose=True), bh(p["qg"])),
         "TM": (G.pair_tiles(ws, L["TM"], dtype, H, nch, 2, 2), bh(p["Tm"]).transpose(-1, -2)),   # tiles hold the blocks transposed
         "HC": (state(L["HC"]), bh(f["h"])),

@@ -45,12 +45,12 @@ def test_workspace_size_and_layout():
     L = _lib.workspace_layout(d, 1)
     assert L["nch"] == 2 * 4 and L["total"] == bwd
     # the two scan operand blocks come first in each slot order; every buffer starts on a 256-byte boundary
-    offs = [L[k] for k in ("W", "BGT", "KGT", "EGL", "UT", "VTT", "BG", "WT", "QGT", "AQBT", "EGLB", "TM", "HC", "DHC", "DVN")]
+    offs = [L[k] for k in ("W", "BGT", "KGT", "EGL", "UT", "VTT", "QGT", "AQBT", "TM", "HC", "DHC", "DVN")]
     assert offs == sorted(offs) and len(set(offs)) == len(offs) and all(o % 256 == 0 for o in offs)
     K = d.K
     assert L["SA_STRIDE"] % 1024 == 0 and L["SA_STRIDE"] >= 5 * (K // 16) * 512 + 4 * K       # bf16 tiles + fp32 decay
-    assert L["SB_STRIDE"] % 1024 == 0 and L["SB_STRIDE"] >= (5 * (K // 16) + 2) * 512 + 4 * K
-    assert L["UT"] - L["W"] >= d.H * L["nch"] * L["SA_STRIDE"] and L["TM"] - L["BG"] >= d.H * L["nch"] * L["SB_STRIDE"]
+    assert L["SB_STRIDE"] % 1024 == 0 and L["SB_STRIDE"] >= (K // 16 + 2) * 512
+    assert L["UT"] - L["W"] >= d.H * L["nch"] * L["SA_STRIDE"] and L["TM"] - L["QGT"] >= d.H * L["nch"] * L["SB_STRIDE"]
     Lf = _lib.workspace_layout(d, 0)
     assert Lf["W"] < Lf["QG"] < Lf["AQB"] < Lf["AQK"] < Lf["EGL"] < Lf["W"] + Lf["SA_STRIDE"] and Lf["SB_STRIDE"] == 0
     # ragged T and packed sequences reserve one extra chunk per sequence
