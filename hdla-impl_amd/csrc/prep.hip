@@ -44,6 +44,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 
     // the inputs of the chunk stay in registers (as loaded) for the second use in phase C: the working set of the
     // resident waves is larger than the L2, so a second load would come from HBM again
     Frag<T> rq[KT], rk[KT], ra[2][KT], rb[2][KT];
+    // v is used last (phase D) but requested first: the barriers in between would otherwise keep its loads, and a
+    // full round trip to HBM, behind everything else
+    Frag<T> rv[VT];
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt) rv[vt] = ld_frag_sel(p.v + voff + 16 * vt, rowok);
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
         const f32x4 g4 = ld_gk4<GKF32>(p.gk, qoff + 16 * kt, rowok);
@@ -185,7 +190,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 
     const Frag<T> aakf[2] = {to_frag<T>(aak[0]), to_frag<T>(aak[1])};
 #pragma unroll
     for (int vt = 0; vt < VT; ++vt) {
-        const Frag<T> vT = transpose(ld_frag_sel(p.v + voff + 16 * vt, rowok), ident);
+        const Frag<T> vT = transpose(rv[vt], ident);
         st_tile(p.ws.VTT + (chw * VT + vt) * TILE, vT);
         const Frag<T> mT[2] = {to_frag<T>(mm(vT, aakf[0], zero4())), to_frag<T>(mm(vT, aakf[1], zero4()))};
         Frag<T> fu[2];
