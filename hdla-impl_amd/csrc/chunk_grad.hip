@@ -1,44 +1,74 @@
 // chunk_grad kernel: everything of the backward pass that is local to one 16-token chunk.
 //
-// One wavefront per (chunk, head) fuses what the reference runs as five launches: the dA part of
+// One workgroup of four wavefronts per (chunk, head) fuses what the reference runs as five launches: the dA part of
 // HRDPLR/bwd_triton.py:30-105, the dv kernel :239-290, the dqg/dkg/dbg/dw/dgk_last kernel :309-487, the WY
 // backward :503-612, the score backward :627-883 and the log-decay gradient :899-948.  Its inputs are the
-// original tensors, do, and per chunk the state entering it (h), the gradient of the state leaving it (dh),
-// v_new and its gradient, all left in the workspace by the two scans.  Nothing but the seven gradients is
-// written back.
+// original tensors, do, and per chunk the state entering it (h), the gradient of the state leaving it (dh) and
+// the gradient of v_new, left in the workspace by the two scans.  Nothing but the seven gradients is written back.
 //
 // Two differences from the reference's algebra, both exact:
 //  * the WY backward never forms d(Tm): with X = [w | u] = Tm R, R = [ag | A_ak v] one has dR = Tm^T dX and
 //    dA_ab = mask(dR X^T), which replaces the Tm^T dTm Tm^T chain of bwd_triton.py:577-612;
 //  * the score backward covers the whole 16 x 16 (x2 ranks) tile with MFMA products against the same
 //    factorised operands as the forward pass instead of a serial per-column loop.
+//
+// Division of the work: every product here contracts over channels or over value columns, so wave w owns the
+// channel tiles kt = w*KT/4 .. and the value tiles vt = w*VT/4 ..; what is summed over the other dimension (the
+// score tiles, their gradients, dv) is exchanged through LDS, with four workgroup barriers in all.  One wave per
+// chunk would hold the whole chunk in registers, at one wave per SIMD, and nothing would overlap its arithmetic
+// with the memory round trips of its neighbours; four waves on a quarter each leave room for two workgroups per
+// compute unit.
 #include "hdla_common.cuh"
 #include "hdla_launch.h"
 
 namespace hdla {
 
-constexpr int LDG = 36;
+constexpr int NW = 4;     // wavefronts per (chunk, head)
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+// LDS of a workgroup (byte offsets)
+template <typename T, int K, int V> struct CgLds {
+    static constexpr int ES = sizeof(T);
+    // do, v, v_new (2 ranks), dv_new (2 ranks) of the chunk, [matrix][token][value], rows padded by 16 bytes
+    static constexpr int VP = V + 16 / ES;
+    static constexpr int TOK = 0, TOK_B = 6 * CH * VP * ES;
+    // per wave: its part of A_qk^T, A_ak^T (2 ranks), fp32 tiles in fragment order
+    static constexpr int SCORE = TOK + TOK_B, SCORE_B = NW * 3 * 1024;
+    // kg of every channel tile (fragments), for dv
+    static constexpr int KG = SCORE + SCORE_B, KG_B = (K / 16) * TILE * ES;
+    // the nine score-gradient tiles, as fragments and as fragments of their transposes
+    static constexpr int FIN = KG + KG_B, FIN_B = 18 * TILE * ES;
+    // first: per wave its part of the nine tiles (fp32); later, for 2-byte elements: the rows of the seven
+    // gradients, so that they leave as whole rows (a lane holds 8 bytes of a row; 8-byte stores of four lanes
+    // would write 32-byte pieces, half of what HBM writes at once)
+    static constexpr bool STAGE_OUT = ES == 2;
+    static constexpr int OPK = K * ES + 16, OPV = V * ES + 16;       // padded rows
+    static constexpr int PART_B = NW * 9 * 1024, OUT_B = STAGE_OUT ? (7 * OPK + OPV) * CH : 0;
+    static constexpr int R1 = FIN + FIN_B, R1_B = PART_B > OUT_B ? PART_B : OUT_B;
+    static constexpr int BYTES = R1 + R1_B;
+};
 
 template <typename T, bool GKF32, int K, int V>
-__global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
-    constexpr int KT = K / 16, VT = V / 16;
+__global__ __launch_bounds__(64 * NW) void chunk_grad_kernel(ChunkArgs<T> p) {
+    constexpr int KT = K / 16, VT = V / 16, KT2 = KT / 2, KTW = KT / NW, VTW = VT / NW;
+    static_assert(KT % NW == 0 && VT % NW == 0 && (KTW == 1 || KTW == 2), "a wave owns one channel tile or one stored pair");
+    typedef CgLds<T, K, V> L;
+    constexpr int VP = L::VP;
+    constexpr bool STAGE_OUT = L::STAGE_OUT;
     constexpr int SFS = blk_fwd(K, sizeof(T), false).SIZE / (int)sizeof(T);   // elements between slots of the scan block
-    __shared__ __attribute__((aligned(16))) float sT[32 * LDG];   // 4608 bytes: stash of the transposed score-gradient tiles
-    // do, v, v_new (2 ranks) and dv_new (2 ranks) of the chunk, [matrix][token][value], staged once: every one of
-    // them is an operand of several products in every pass, and the working set of the resident waves is far
-    // larger than the L2, so repeated global loads would mostly be repeated HBM reads
-    constexpr int VP = V + 16 / (int)sizeof(T);                    // padded row, keeps 16-byte alignment
-    __shared__ __attribute__((aligned(16))) T sTok[6 * CH * VP];
-    // Results of 2-byte elements leave through LDS: a lane holds 8 bytes of a row, and 8-byte stores of four lanes
-    // would write 32-byte pieces of rows, half of what HBM writes at once.  Two adjacent 16-column tiles are put
-    // side by side in LDS and stored 16 bytes a lane, 64 contiguous bytes a row.
-    constexpr bool STAGE_OUT = sizeof(T) == 2;
-    constexpr int OPITCH = 80;                                     // bytes; 64 of data, padded against bank conflicts
-    __shared__ __attribute__((aligned(16))) char sOut[STAGE_OUT ? 7 * CH * OPITCH : 16];
+    __shared__ __attribute__((aligned(16))) char smem[L::BYTES];
+    T* const sTok = reinterpret_cast<T*>(smem + L::TOK);
+    float* const sScore = reinterpret_cast<float*>(smem + L::SCORE);
+    T* const sKg = reinterpret_cast<T*>(smem + L::KG);
+    T* const sFin = reinterpret_cast<T*>(smem + L::FIN);
+    float* const sPart = reinterpret_cast<float*>(smem + L::R1);
+    char* const sOut = smem + L::R1;
 
     const int cid = blockIdx.x, h = blockIdx.y;
     ChunkPos cp;
-    if (!locate_chunk(p.st, cid, cp)) return;
+    if (!locate_chunk(p.st, cid, cp)) return;                 // uniform over the workgroup
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int l = lane_id(), g = l >> 4, c = l & 15;
     const int H = p.H;
     const bool rowok = c < cp.len;
@@ -57,140 +87,152 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
     const T* HC = p.ws.HC + chw * (K * V);
     const T* DHC = p.ws.DHC + chw * (K * V);
     const T* DVN = p.ws.DVN + chw * (2 * CH * V);
-    const int blk = blockIdx.y * gridDim.x + blockIdx.x;
-    PHASE_CLOCK(p, blk, 0);
+    const T* Wb = p.ws.W + chw * SFS;
+    const int kt0 = w * KTW, vt0 = w * VTW;                   // first own channel tile / value tile
 
-    // q, k, a and gk of the chunk stay in registers for their second use in the last pass (a second load would
-    // mostly be a second HBM read); bf16 operands only, fp32 ones would not fit next to the accumulators.  Their
-    // loads are the first thing issued, so that they travel together with the staging loads below: a wave spends
-    // most of its time waiting for memory, and every dependent round trip to HBM costs thousands of cycles.
-    constexpr bool KEEP = sizeof(T) == 2;
-    // The smallest shape also keeps the whole checkpoint of S (all its tile pairs) in registers from here to the
-    // end: it is used three times (v_new, first and second pass over channel tiles) and a later read would mostly
-    // come from HBM again; the other shapes read it tile by tile where it is used.
-    constexpr bool PF = sizeof(T) == 2 && K == 64 && V == 64;
-    constexpr int KT2 = KT / 2;
-    Frag<T> hcall[PF ? KT2 : 1][PF ? VT : 1][2];
-    if (PF) {
+    // ---- everything the wave reads from global memory is requested here, before any arithmetic -----------------
+    // (only the checkpoint of dS waits for the large shapes: it is used last and would not fit next to the rest)
+    Frag<T> rq[KTW], rk[KTW], ra[2][KTW], rb[2][KTW];          // own channel tiles of the inputs
+    f32x4 rg[KTW];
 #pragma unroll
-        for (int kp = 0; kp < KT2; ++kp)
-#pragma unroll
-            for (int vt = 0; vt < VT; ++vt) ld_pair(HC + (kp * VT + vt) * PAIR, hcall[PF ? kp : 0][PF ? vt : 0][0], hcall[PF ? kp : 0][PF ? vt : 0][1]);
+    for (int j = 0; j < KTW; ++j) {
+        const uint32_t ko = 16 * (kt0 + j);
+        rg[j] = ld_gk4<GKF32>(gkp + go + ko * GS, 0, rowok);
+        rq[j] = ld_frag_sel(at(p.q + qb, qo + ko * ES), rowok);
+        rk[j] = ld_frag_sel(at(p.k + qb, qo + ko * ES), rowok);
+        ra[0][j] = ld_frag_sel(at(p.a + ab, ao0 + ko * ES), rowok);
+        ra[1][j] = ld_frag_sel(at(p.a + ab, ao1 + ko * ES), rowok);
+        rb[0][j] = ld_frag_sel(at(p.b + ab, ao0 + ko * ES), rowok);
+        rb[1][j] = ld_frag_sel(at(p.b + ab, ao1 + ko * ES), rowok);
     }
-    Frag<T> rq[KEEP ? KT : 1], rk[KEEP ? KT : 1], ra[2][KEEP ? KT : 1];
-    f32x4 rg[KEEP ? KT : 1];
-    if (KEEP) {
+    // rows of do and v: 16 bytes a lane, the waves take turns
+    constexpr int EPL = 16 / (int)sizeof(T), LPR = V / EPL, RPI = 64 / LPR, NRI = 2 * CH / RPI;   // elements/lane, lanes/row, rows/instr
+    static_assert(NRI % NW == 0, "");
+    i32x4 rows[NRI / NW];
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) {
-            rg[KEEP ? kt : 0] = ld_gk4<GKF32>(gkp + go + 16 * kt * GS, 0, rowok);
-            rq[KEEP ? kt : 0] = ld_frag_sel(at(p.q + qb, qo + 16 * kt * ES), rowok);
-            rk[KEEP ? kt : 0] = ld_frag_sel(at(p.k + qb, qo + 16 * kt * ES), rowok);
-            ra[0][KEEP ? kt : 0] = ld_frag_sel(at(p.a + ab, ao0 + 16 * kt * ES), rowok);
-            ra[1][KEEP ? kt : 0] = ld_frag_sel(at(p.a + ab, ao1 + 16 * kt * ES), rowok);
-        }
+    for (int j = 0; j < NRI / NW; ++j) {
+        const int i = w + j * NW, m = i / (CH / RPI), r = (i % (CH / RPI)) * RPI + l / LPR;
+        rows[j] = *reinterpret_cast<const i32x4*>(at((m == 0 ? p.dout : p.v) + vb, (uint32_t)(min(r, cp.len - 1) * H * V + (l % LPR) * EPL) * ES));
     }
-    const Frag<T> ident = ident_frag<T>();
-    {
-        // do and v: rows of the original tensors, 16 bytes per lane
-        constexpr int EPL = 16 / (int)sizeof(T), LPR = V / EPL, RPI = 64 / LPR;    // elements/lane, lanes/row, rows/instr
-        const int rr = l / LPR, e = (l % LPR) * EPL;
-        typedef int i32x4 __attribute__((ext_vector_type(4)));
+    // the scans checkpoint S and dS as fragments of the transposed tiles (rows value, inner channel), tile pairs
+    // [channel pair][value tile]: pair_of(X, kp, vt)
+    auto own_kt_tiles = [&](const T* X, Frag<T> (&dst)[KTW][VT]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int m = 0; m < 2; ++m)
-#pragma unroll
-            for (int r0 = 0; r0 < CH; r0 += RPI) {
-                const int r = r0 + rr;
-                const T* src = at((m == 0 ? p.dout : p.v) + vb, (uint32_t)(min(r, cp.len - 1) * H * V + e) * ES);
-                i32x4 x = *reinterpret_cast<const i32x4*>(src);
-                if (r >= cp.len) x = (i32x4){0, 0, 0, 0};
-                *reinterpret_cast<i32x4*>(&sTok[(m * CH + r) * VP + e]) = x;
-            }
-        // dv_new: the reverse scan left it as fragments of the transposed tiles (rows value, inner token), the two
-        // ranks of a value tile paired; one transposing product each gives the rows.
-        // v_new is not checkpointed by the scan: v_new_s = w_s S + u_s is rebuilt here from the checkpoint of S, which
-        // is stored as exactly the operand this product needs (fragments of S^T), with the same bf16 operands and
-        // fp32 accumulation as in the scan.
-        Frag<T> wf[2][KT];
-#pragma unroll
-        for (int s = 0; s < 2; ++s)
-#pragma unroll
-            for (int kp = 0; kp < KT / 2; ++kp)
-                ld_pair(p.ws.W + chw * SFS + (s * (KT / 2) + kp) * PAIR, wf[s][2 * kp], wf[s][2 * kp + 1]);
-#pragma unroll(sizeof(T) * V >= 512 ? 1 : VT)
         for (int vt = 0; vt < VT; ++vt) {
-            Frag<T> u0, u1, y0, y1;
-            ld_pair(p.ws.UT + (chw * VT + vt) * PAIR, u0, u1);
-            ld_pair(DVN + vt * PAIR, y0, y1);
-            f32x4 vn0 = zero4(), vn1 = zero4();
-#pragma unroll
-            for (int kp = 0; kp < KT / 2; ++kp) {
-                Frag<T> h0, h1;
-                if (PF) { h0 = hcall[PF ? kp : 0][PF ? vt : 0][0]; h1 = hcall[PF ? kp : 0][PF ? vt : 0][1]; }
-                else ld_pair(HC + (kp * VT + vt) * PAIR, h0, h1);
-                vn0 = mm(wf[0][2 * kp], h0, vn0);
-                vn1 = mm(wf[1][2 * kp], h0, vn1);
-                vn0 = mm(wf[0][2 * kp + 1], h1, vn0);
-                vn1 = mm(wf[1][2 * kp + 1], h1, vn1);
-            }
-            vn0 += to_f32(transpose(u0, ident));
-            vn1 += to_f32(transpose(u1, ident));
-            T* dst = &sTok[c * VP + 16 * vt + 4 * g];
-            st_frag(dst + 2 * CH * VP, to_frag<T>(vn0));
-            st_frag(dst + 3 * CH * VP, to_frag<T>(vn1));
-            st_frag(dst + 4 * CH * VP, transpose(y0, ident));
-            st_frag(dst + 5 * CH * VP, transpose(y1, ident));
+            if (KTW == 2) ld_pair(X + (w * VT + vt) * PAIR, dst[0][vt], dst[KTW - 1][vt]);
+            else dst[0][vt] = ld_pair_one(X + ((w >> 1) * VT + vt) * PAIR, w & 1);
         }
+    };
+    auto own_vt_tiles = [&](const T* X, Frag<T> (&dst)[VTW][KT]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < VTW; ++j)
+#pragma unroll
+            for (int kp = 0; kp < KT2; ++kp) ld_pair(X + (kp * VT + vt0 + j) * PAIR, dst[j][2 * kp], dst[j][2 * kp + 1]);
+    };
+    Frag<T> wf[2][KT], wk[2][KTW];                             // w: all of it (v_new), and the own channel tiles
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+#pragma unroll
+        for (int kp = 0; kp < KT2; ++kp) ld_pair(Wb + (s * KT2 + kp) * PAIR, wf[s][2 * kp], wf[s][2 * kp + 1]);
+        if (KTW == 2) ld_pair(Wb + (s * KT2 + w) * PAIR, wk[s][0], wk[s][KTW - 1]);
+        else wk[s][0] = ld_pair_one(Wb + (s * KT2 + (w >> 1)) * PAIR, w & 1);
     }
-    auto tokf = [&](int m, int vt) __attribute__((always_inline)) { return ld_frag(&sTok[(m * CH + c) * VP + 16 * vt + 4 * g]); };
+    Frag<T> hv[VTW][KT], hk[KTW][VT], dhv[VTW][KT], dhk[KTW][VT];
+    own_vt_tiles(HC, hv);
+    own_kt_tiles(HC, hk);
+    Frag<T> ut[VTW][2], yt[VTW][2];                            // u^T and dv_new^T of the own value tiles, both ranks
+#pragma unroll
+    for (int j = 0; j < VTW; ++j) {
+        ld_pair(p.ws.UT + (chw * VT + vt0 + j) * PAIR, ut[j][0], ut[j][1]);
+        ld_pair(DVN + (vt0 + j) * PAIR, yt[j][0], yt[j][1]);
+    }
     // tmT[s][r] = F((Tm^{s r})^T): lane (g,c) reg i = Tm^{s r}[4g+i][c], stored in this form by the prep kernel
     Frag<T> tmT[2][2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) ld_pair(p.ws.TM + chw * 1024 + s * PAIR, tmT[s][0], tmT[s][1]);
-    __syncthreads();
+    constexpr bool EARLY_DH = sizeof(T) * K * V <= 2 * 64 * 64;
+    if (EARLY_DH) { own_kt_tiles(DHC, dhk); own_vt_tiles(DHC, dhv); }
 
-    // ---- cumulative decays; A_qk^T and A_ak^T (rows j, inner i) -----------------------------------------------
-    // (the decays are recomputed per channel tile wherever they are needed: a load and four DPP additions cost
-    // less than keeping 2*K/16 vector registers alive across the kernel)
-    f32x4 aqkT = zero4(), aakT[2] = {zero4(), zero4()};
-#pragma unroll
-    for (int kt = 0; kt < KT; ++kt) {
-        const f32x4 g4 = KEEP ? rg[KEEP ? kt : 0] : ld_gk4<GKF32>(gkp + go + 16 * kt * GS, 0, rowok);
-        const f32x4 gi = scan16_incl(g4), ge = gi - g4;
-        const f32x4 m = bcast16(gi, MID);
-        const f32x4 eq = exp4<T>(gi - m), ek = exp4<T>(m - gi), ea = exp4<T>(ge - m);
-        const Frag<T> fq = KEEP ? rq[KEEP ? kt : 0] : ld_frag_sel(at(p.q + qb, qo + 16 * kt * ES), rowok);
-        const Frag<T> fk = KEEP ? rk[KEEP ? kt : 0] : ld_frag_sel(at(p.k + qb, qo + 16 * kt * ES), rowok);
-        const Frag<T> fa0 = KEEP ? ra[0][KEEP ? kt : 0] : ld_frag_sel(at(p.a + ab, ao0 + 16 * kt * ES), rowok);
-        const Frag<T> fa1 = KEEP ? ra[1][KEEP ? kt : 0] : ld_frag_sel(at(p.a + ab, ao1 + 16 * kt * ES), rowok);
-        const f32x4 q4 = to_f32(fq), k4 = to_f32(fk), a0 = to_f32(fa0), a1 = to_f32(fa1);
-        const Frag<T> qh = to_frag<T>(q4 * eq * scale), kh = to_frag<T>(k4 * ek);
-        aqkT = mm(kh, qh, aqkT);
-        aakT[0] = mm(kh, to_frag<T>(a0 * ea), aakT[0]);
-        aakT[1] = mm(kh, to_frag<T>(a1 * ea), aakT[1]);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {          // row j = c, inner i = 4g+i
-        const int ii = 4 * g + i;
-        if (!(c <= ii)) aqkT[i] = 0.f;
-        if (!(c < ii)) { aakT[0][i] = 0.f; aakT[1][i] = 0.f; }
-    }
-    const Frag<T> aqkTf = to_frag<T>(aqkT);
-    const Frag<T> aakTf[2] = {to_frag<T>(aakT[0]), to_frag<T>(aakT[1])};
+    const Frag<T> ident = ident_frag<T>();
 
-    // In the second pass the checkpoint of the state gradient arrives a pair of channel tiles ahead of its use:
-    // [buffer][value tile][tile of the pair].
-    Frag<T> dhp[PF ? 2 : 1][PF ? VT : 1][2];
-    auto fetch_pairs = [&](const T* src, Frag<T> (&dst)[PF ? VT : 1][2], int kp) __attribute__((always_inline)) {
+    // ---- own channel tiles: part of A_qk^T and A_ak^T (rows j, inner i); kg for everybody ------------------------
+    {
+        f32x4 aqkT = zero4(), aakT[2] = {zero4(), zero4()};
 #pragma unroll
-        for (int vt = 0; vt < VT; ++vt) ld_pair(src + (kp * VT + vt) * PAIR, dst[PF ? vt : 0][0], dst[PF ? vt : 0][1]);
-    };
-    PHASE_CLOCK(p, blk, 1);
-    // ---- products over the value dimension -------------------------------------------------------------------
+        for (int j = 0; j < KTW; ++j) {
+            const f32x4 g4 = rg[j];
+            const f32x4 gi = scan16_incl(g4), ge = gi - g4;
+            const f32x4 m = bcast16(gi, MID);
+            const f32x4 eq = exp4<T>(gi - m), ek = exp4<T>(m - gi), ea = exp4<T>(ge - m);
+            const f32x4 q4 = to_f32(rq[j]), k4 = to_f32(rk[j]), a0 = to_f32(ra[0][j]), a1 = to_f32(ra[1][j]);
+            const Frag<T> qh = to_frag<T>(q4 * eq * scale), kh = to_frag<T>(k4 * ek);
+            aqkT = mm(kh, qh, aqkT);
+            aakT[0] = mm(kh, to_frag<T>(a0 * ea), aakT[0]);
+            aakT[1] = mm(kh, to_frag<T>(a1 * ea), aakT[1]);
+            const f32x4 edn = exp4<T>(bcast16(gi, CH - 1) - gi);
+            st_tile(sKg + (kt0 + j) * TILE, to_frag<T>(k4 * edn));
+        }
+        *reinterpret_cast<f32x4*>(sScore + ((w * 3 + 0) * 64 + l) * 4) = aqkT;
+        *reinterpret_cast<f32x4*>(sScore + ((w * 3 + 1) * 64 + l) * 4) = aakT[0];
+        *reinterpret_cast<f32x4*>(sScore + ((w * 3 + 2) * 64 + l) * 4) = aakT[1];
+    }
+    // ---- staging: rows of do and v; own value tiles of v_new and dv_new ------------------------------------------
+#pragma unroll
+    for (int j = 0; j < NRI / NW; ++j) {
+        const int i = w + j * NW, m = i / (CH / RPI), r = (i % (CH / RPI)) * RPI + l / LPR;
+        *reinterpret_cast<i32x4*>(&sTok[(m * CH + r) * VP + (l % LPR) * EPL]) = r < cp.len ? rows[j] : (i32x4){0, 0, 0, 0};
+    }
+    // v_new is not checkpointed by the scan: v_new_s = w_s S + u_s is rebuilt here from the checkpoint of S, which
+    // is stored as exactly the operand this product needs (fragments of S^T), with the same bf16 operands and
+    // fp32 accumulation as in the scan.  dv_new arrives as fragments of the transposed tiles (rows value, inner
+    // token); one transposing product each gives the rows.
+    Frag<T> uN[VTW][2];                                       // u of the own value tiles: rows token, inner value
+#pragma unroll
+    for (int j = 0; j < VTW; ++j) {
+        f32x4 vn0 = zero4(), vn1 = zero4();
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            vn0 = mm(wf[0][kt], hv[j][kt], vn0);
+            vn1 = mm(wf[1][kt], hv[j][kt], vn1);
+        }
+        uN[j][0] = transpose(ut[j][0], ident);
+        uN[j][1] = transpose(ut[j][1], ident);
+        vn0 += to_f32(uN[j][0]);
+        vn1 += to_f32(uN[j][1]);
+        T* dst = &sTok[c * VP + 16 * (vt0 + j) + 4 * g];
+        st_frag(dst + 2 * CH * VP, to_frag<T>(vn0));
+        st_frag(dst + 3 * CH * VP, to_frag<T>(vn1));
+        st_frag(dst + 4 * CH * VP, transpose(yt[j][0], ident));
+        st_frag(dst + 5 * CH * VP, transpose(yt[j][1], ident));
+    }
+    __syncthreads();                                           // (1) sTok, sScore, sKg complete
+    auto tokf = [&](int m, int vt) __attribute__((always_inline)) { return ld_frag(&sTok[(m * CH + c) * VP + 16 * vt + 4 * g]); };
+
+    Frag<T> aqkTf, aakTf[2];
+    {
+        f32x4 t[3] = {zero4(), zero4(), zero4()};
+#pragma unroll
+        for (int ww = 0; ww < NW; ++ww)
+#pragma unroll
+            for (int i = 0; i < 3; ++i) t[i] += *reinterpret_cast<const f32x4*>(sScore + ((ww * 3 + i) * 64 + l) * 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {          // row j = c, inner i = 4g+i
+            const int ii = 4 * g + i;
+            if (!(c <= ii)) t[0][i] = 0.f;
+            if (!(c < ii)) { t[1][i] = 0.f; t[2][i] = 0.f; }
+        }
+        aqkTf = to_frag<T>(t[0]);
+        aakTf[0] = to_frag<T>(t[1]);
+        aakTf[1] = to_frag<T>(t[2]);
+    }
+
+    // ---- own value tiles: products over the value dimension ------------------------------------------------------
     f32x4 dAqk = zero4(), dAqb[2] = {zero4(), zero4()}, dAak[2] = {zero4(), zero4()};
     f32x4 dAab[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
-    f32x4 dv[VT];
+    f32x4 dv[VTW];
 #pragma unroll
-    for (int vt = 0; vt < VT; ++vt) {
+    for (int j = 0; j < VTW; ++j) {
+        const int vt = vt0 + j;
         const Frag<T> doN = tokf(0, vt);
         const Frag<T> vN = tokf(1, vt);
         const Frag<T> vnN[2] = {tokf(2, vt), tokf(3, vt)};
@@ -198,141 +240,112 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
         dAqb[0] = mm(doN, vnN[0], dAqb[0]);
         dAqb[1] = mm(doN, vnN[1], dAqb[1]);
         const Frag<T> doT = transpose(doN, ident);
-        Frag<T> dvnT[2];                                  // as the reverse scan left them: rows value, inner token
-        ld_pair(DVN + vt * PAIR, dvnT[0], dvnT[1]);
         Frag<T> dMf[2], dMTf[2];
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
-            f32x4 x = mm(tmT[0][r], dvnT[0], zero4());
-            x = mm(tmT[1][r], dvnT[1], x);
+            f32x4 x = mm(tmT[0][r], yt[j][0], zero4());
+            x = mm(tmT[1][r], yt[j][1], x);
             dMf[r] = to_frag<T>(x);                       // dM_r   rows i, inner value
-            f32x4 y = mm(dvnT[0], tmT[0][r], zero4());
-            y = mm(dvnT[1], tmT[1][r], y);
+            f32x4 y = mm(yt[j][0], tmT[0][r], zero4());
+            y = mm(yt[j][1], tmT[1][r], y);
             dMTf[r] = to_frag<T>(y);                      // dM_r^T rows value, inner i
         }
-        const Frag<T> uN[2] = {transpose(ld_pair_one(p.ws.UT + (chw * VT + vt) * PAIR, 0), ident),
-                               transpose(ld_pair_one(p.ws.UT + (chw * VT + vt) * PAIR, 1), ident)};
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
             dAak[r] = mm(dMf[r], vN, dAak[r]);
-            dAab[r][0] = mm(dMf[r], uN[0], dAab[r][0]);
-            dAab[r][1] = mm(dMf[r], uN[1], dAab[r][1]);
+            dAab[r][0] = mm(dMf[r], uN[j][0], dAab[r][0]);
+            dAab[r][1] = mm(dMf[r], uN[j][1], dAab[r][1]);
         }
         f32x4 x = mm(aqkTf, doT, zero4());
         x = mm(aakTf[0], dMTf[0], x);
         x = mm(aakTf[1], dMTf[1], x);
-        dv[vt] = x;                                       // rows token, inner value; kg dS is added below
+        dv[j] = x;                                        // rows token, inner value; kg dS is added at the end
     }
 
-    PHASE_CLOCK(p, blk, 2);
-    // ---- first pass over channel tiles: dw -> dag -> the w part of dA_ab (dag itself is rebuilt in pass two) ----
+    // ---- own channel tiles, first pass: dw -> dag -> the w part of dA_ab -------------------------------------------
+    Frag<T> Sf[KTW][VT];                                      // S of the own channel tiles: rows channel, inner value
+    f32x4 dag[KTW][2];                                        // dag_r = sum_s (Tm^{s r})^T dw_s, rows token, inner channel
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt) {
+    for (int j = 0; j < KTW; ++j) {
         f32x4 dwT[2] = {zero4(), zero4()};                // rows channel, inner token
 #pragma unroll
         for (int vt = 0; vt < VT; ++vt) {
-            const Frag<T> Sf = transpose(PF ? hcall[PF ? kt / 2 : 0][PF ? vt : 0][kt & 1]
-                                            : ld_pair_one(HC + ((kt / 2) * VT + vt) * PAIR, kt & 1), ident);
-            dwT[0] = mm(Sf, tokf(4, vt), dwT[0]);
-            dwT[1] = mm(Sf, tokf(5, vt), dwT[1]);
+            Sf[j][vt] = transpose(hk[j][vt], ident);
+            dwT[0] = mm(Sf[j][vt], tokf(4, vt), dwT[0]);
+            dwT[1] = mm(Sf[j][vt], tokf(5, vt), dwT[1]);
         }
         const Frag<T> dwTf[2] = {to_frag<T>(dwT[0]), to_frag<T>(dwT[1])};
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
-            f32x4 x = mm(tmT[0][r], dwTf[0], zero4());
-            x = mm(tmT[1][r], dwTf[1], x);                // dag_r: rows token, inner channel
-            const Frag<T> dagf = to_frag<T>(x);
-            dAab[r][0] = mm(dagf, ld_pair_one(p.ws.W + chw * SFS + (0 * (KT / 2) + kt / 2) * PAIR, kt & 1), dAab[r][0]);
-            dAab[r][1] = mm(dagf, ld_pair_one(p.ws.W + chw * SFS + (1 * (KT / 2) + kt / 2) * PAIR, kt & 1), dAab[r][1]);
+            dag[j][r] = mm(tmT[0][r], dwTf[0], zero4());
+            dag[j][r] = mm(tmT[1][r], dwTf[1], dag[j][r]);
+            const Frag<T> dagf = to_frag<T>(dag[j][r]);
+            dAab[r][0] = mm(dagf, wk[0][j], dAab[r][0]);
+            dAab[r][1] = mm(dagf, wk[1][j], dAab[r][1]);
         }
     }
-
-    // for the second pass: the first pair of S and dS tiles, and all of b (used there only), requested now
-    Frag<T> rb[2][KEEP ? KT : 1];
-    if (PF) fetch_pairs(DHC, dhp[0], 0);
-    if (KEEP) {
+    // tile indices: 0 A_qk, 1+s A_qb^s, 3+s A_ak^s, 5+2r+s A_ab^{r s}
+    {
+        auto part = [&](int idx, f32x4 x) __attribute__((always_inline)) { *reinterpret_cast<f32x4*>(sPart + ((w * 9 + idx) * 64 + l) * 4) = x; };
+        part(0, dAqk);
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) {
-            rb[0][KEEP ? kt : 0] = ld_frag_sel(at(p.b + ab, ao0 + 16 * kt * ES), rowok);
-            rb[1][KEEP ? kt : 0] = ld_frag_sel(at(p.b + ab, ao1 + 16 * kt * ES), rowok);
+        for (int s = 0; s < 2; ++s) {
+            part(1 + s, dAqb[s]);
+            part(3 + s, dAak[s]);
+            part(5 + s, dAab[0][s]);
+            part(7 + s, dAab[1][s]);
         }
     }
-    PHASE_CLOCK(p, blk, 3);
-    // ---- masks; both orientations of the nine score-gradient tiles --------------------------------------------
+    if (!EARLY_DH) { own_kt_tiles(DHC, dhk); own_vt_tiles(DHC, dhv); }
+    __syncthreads();                                           // (2) the parts of the nine tiles are complete
+    // the waves share out the nine tiles: sum of the parts, causal mask, both orientations as fragments
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {          // row i = c, inner j = 4g+i
-        const int j = 4 * g + i;
-        if (!(j <= c)) { dAqk[i] = 0.f; dAqb[0][i] = 0.f; dAqb[1][i] = 0.f; }
-        if (!(j < c)) { dAak[0][i] = 0.f; dAak[1][i] = 0.f; dAab[0][0][i] = 0.f; dAab[0][1][i] = 0.f; dAab[1][0][i] = 0.f; dAab[1][1][i] = 0.f; }
+    for (int t = 0; t < (9 + NW - 1) / NW; ++t) {
+        const int idx = w + t * NW;
+        if (idx < 9) {
+            f32x4 x = zero4();
+#pragma unroll
+            for (int ww = 0; ww < NW; ++ww) x += *reinterpret_cast<const f32x4*>(sPart + ((ww * 9 + idx) * 64 + l) * 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {      // row i = c, inner j = 4g+i; A_qk and A_qb keep the diagonal
+                const int jj = 4 * g + i;
+                if (idx < 3 ? !(jj <= c) : !(jj < c)) x[i] = 0.f;
+            }
+            const Frag<T> f = to_frag<T>(x);
+            st_tile(sFin + idx * TILE, f);
+            st_tile(sFin + (9 + idx) * TILE, transpose(f, ident));
+        }
     }
-    // The transposed tiles are needed once per channel tile of the second pass.  For 2-byte elements the nine of
-    // them are kept in LDS (4608 bytes) and read back where used: 18 registers less across the second pass.
-    constexpr bool STASH = sizeof(T) == 2;
-    T* stash = reinterpret_cast<T*>(sT);
-    const Frag<T> fAqk = to_frag<T>(dAqk);
-    Frag<T> fAqb[2], fAak[2], fAab[2][2];
-    Frag<T> rT[STASH ? 1 : 9];                             // transposes kept in registers otherwise
-    auto putT = [&](int idx, Frag<T> f) __attribute__((always_inline)) {
-        const Frag<T> t = transpose(f, ident);
-        if (STASH) st_tile(stash + idx * TILE, t);
-        else rT[STASH ? 0 : idx] = t;
+    __syncthreads();                                           // (3) sFin complete; sPart may be overwritten (sOut)
+    auto fin = [&](int idx) __attribute__((always_inline)) { return ld_tile(sFin + idx * TILE); };
+    auto finT = [&](int idx) __attribute__((always_inline)) { return ld_tile(sFin + (9 + idx) * TILE); };
+    // put(m, kt, f): tile f of gradient m (0 dq, 1 dk, 2/3 da, 4/5 db, 6 dgk) at channel tile kt of the staged rows
+    auto put = [&](int m, int kt, Frag<T> f) __attribute__((always_inline)) {
+        st_frag(reinterpret_cast<T*>(sOut + (m * CH + c) * L::OPK) + 16 * kt + 4 * g, f);
     };
-    auto getT = [&](int idx) __attribute__((always_inline)) { return STASH ? ld_tile(stash + idx * TILE) : rT[STASH ? 0 : idx]; };
-    // indices: 0 A_qk, 1+s A_qb^s, 3+s A_ak^s, 5+2r+s A_ab^{r s}
-    putT(0, fAqk);
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-        fAqb[s] = to_frag<T>(dAqb[s]); putT(1 + s, fAqb[s]);
-        fAak[s] = to_frag<T>(dAak[s]); putT(3 + s, fAak[s]);
-#pragma unroll
-        for (int r = 0; r < 2; ++r) { fAab[r][s] = to_frag<T>(dAab[r][s]); putT(5 + 2 * r + s, fAab[r][s]); }
-    }
 
-    // put(m, half, f): tile f of output m into column half `half`; flush(m, base, byte0): the 16 x 32 block out
-    auto put = [&](int m, int half, Frag<T> f) __attribute__((always_inline)) {
-        st_frag(reinterpret_cast<T*>(sOut + (m * CH + c) * OPITCH + half * 32) + 4 * g, f);
-    };
-    auto flush = [&](int m, T* ubase, uint32_t row_pitch_bytes, uint32_t byte0) __attribute__((always_inline)) {
-        typedef int i32x4 __attribute__((ext_vector_type(4)));
-        const int r = l >> 2, piece = l & 3;
-        const i32x4 x = *reinterpret_cast<const i32x4*>(sOut + (m * CH + r) * OPITCH + piece * 16);
-        if (r < cp.len) *reinterpret_cast<i32x4*>(reinterpret_cast<char*>(ubase) + (uint32_t)r * row_pitch_bytes + byte0 + piece * 16) = x;
-    };
-    PHASE_CLOCK(p, blk, 4);
-    // ---- second pass over channel tiles: state products, score backward, final gradients ----------------------
-#pragma unroll(KEEP ? KT : 1)
-    for (int kt = 0; kt < KT; ++kt) {
-        if (PF && !(kt & 1) && kt / 2 + 1 < KT2) fetch_pairs(DHC, dhp[PF ? (kt / 2 + 1) & 1 : 0], kt / 2 + 1);
-        // (a) what the loop over value tiles needs: only kg of this channel tile
-        const f32x4 g4 = KEEP ? rg[KEEP ? kt : 0] : ld_gk4<GKF32>(gkp + go + 16 * kt * GS, 0, rowok);
+    // ---- own channel tiles, second pass: state products, score backward, final gradients ---------------------------
+#pragma unroll
+    for (int j = 0; j < KTW; ++j) {
+        const int kt = kt0 + j;
+        const f32x4 g4 = rg[j];
         const f32x4 gi = scan16_incl(g4);
         const f32x4 gl = bcast16(gi, CH - 1);
         const f32x4 edn = exp4<T>(gl - gi);
-        const f32x4 k4 = to_f32(KEEP ? rk[KEEP ? kt : 0] : ld_frag_sel(at(p.k + qb, qo + 16 * kt * ES), rowok));
+        const f32x4 k4 = to_f32(rk[j]);
         const f32x4 kg4 = k4 * edn;
-        const Frag<T> kgf = to_frag<T>(kg4);
 
         f32x4 dqg = zero4(), dkg = zero4(), dbg[2] = {zero4(), zero4()};
-        f32x4 dwT[2] = {zero4(), zero4()};                 // dw_s^T for this channel tile (rows channel, inner token)
         float hh = 0.f;                                    // partial of sum_v S * dS for channel 16kt + c
-#pragma unroll(sizeof(T) == 2 ? VT : 2)
+#pragma unroll
         for (int vt = 0; vt < VT; ++vt) {
-            // the scans checkpoint S and dS as fragments of the transposed tiles (rows value, inner channel)
-            const Frag<T> dST = PF ? dhp[PF ? (kt / 2) & 1 : 0][PF ? vt : 0][kt & 1] : ld_pair_one(DHC + ((kt / 2) * VT + vt) * PAIR, kt & 1);
-            const Frag<T> Sf = transpose(PF ? hcall[PF ? kt / 2 : 0][PF ? vt : 0][kt & 1]
-                                            : ld_pair_one(HC + ((kt / 2) * VT + vt) * PAIR, kt & 1), ident);
-            const Frag<T> dSf = transpose(dST, ident);
-            const Frag<T> doN = tokf(0, vt);
-            const Frag<T> vN = tokf(1, vt);
-            dqg = mm(doN, Sf, dqg);
-            dwT[0] = mm(Sf, tokf(4, vt), dwT[0]);
-            dwT[1] = mm(Sf, tokf(5, vt), dwT[1]);
-            dkg = mm(vN, dSf, dkg);
+            const Frag<T> dSf = transpose(dhk[j][vt], ident);
+            dqg = mm(tokf(0, vt), Sf[j][vt], dqg);
+            dkg = mm(tokf(1, vt), dSf, dkg);
             dbg[0] = mm(tokf(2, vt), dSf, dbg[0]);
             dbg[1] = mm(tokf(3, vt), dSf, dbg[1]);
-            const f32x4 s4 = to_f32(Sf), d4 = to_f32(dSf);
+            const f32x4 s4 = to_f32(Sf[j][vt]), d4 = to_f32(dSf);
             hh += s4[0] * d4[0] + s4[1] * d4[1] + s4[2] * d4[2] + s4[3] * d4[3];
-            dv[vt] = mm(kgf, dST, dv[vt]);
         }
         hh += __shfl_xor(hh, 16);
         hh += __shfl_xor(hh, 32);
@@ -340,73 +353,53 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) hh4[i] = __shfl(hh, 4 * g + i);
 
-        const Frag<T> dwTf[2] = {to_frag<T>(dwT[0]), to_frag<T>(dwT[1])};
-        f32x4 dag[2];                                      // dag_r = sum_s (Tm^{s r})^T dw_s, rows token, inner channel
-#pragma unroll
-        for (int r = 0; r < 2; ++r) {
-            dag[r] = mm(tmT[0][r], dwTf[0], zero4());
-            dag[r] = mm(tmT[1][r], dwTf[1], dag[r]);
-        }
-        // (b) the factorised operands and decay factors of this channel tile, for the score backward
+        // the factorised operands and decay factors of this channel tile, for the score backward
         const f32x4 ge = gi - g4;
         const f32x4 m = bcast16(gi, MID);
         const f32x4 eq = exp4<T>(gi - m), ek = exp4<T>(m - gi), ea = exp4<T>(ge - m);
         const f32x4 egi = exp4<T>(gi), ege = exp4<T>(ge);
-        const f32x4 q4 = to_f32(KEEP ? rq[KEEP ? kt : 0] : ld_frag_sel(at(p.q + qb, qo + 16 * kt * ES), rowok));
-        const f32x4 a4[2] = {to_f32(KEEP ? ra[0][KEEP ? kt : 0] : ld_frag_sel(at(p.a + ab, ao0 + 16 * kt * ES), rowok)),
-                             to_f32(KEEP ? ra[1][KEEP ? kt : 0] : ld_frag_sel(at(p.a + ab, ao1 + 16 * kt * ES), rowok))};
-        const f32x4 b4[2] = {to_f32(KEEP ? rb[0][KEEP ? kt : 0] : ld_frag_sel(at(p.b + ab, ao0 + 16 * kt * ES), rowok)),
-                             to_f32(KEEP ? rb[1][KEEP ? kt : 0] : ld_frag_sel(at(p.b + ab, ao1 + 16 * kt * ES), rowok))};
+        const f32x4 q4 = to_f32(rq[j]);
+        const f32x4 a4[2] = {to_f32(ra[0][j]), to_f32(ra[1][j])};
+        const f32x4 b4[2] = {to_f32(rb[0][j]), to_f32(rb[1][j])};
         const Frag<T> qhT = transpose(to_frag<T>(q4 * eq * scale), ident), khT = transpose(to_frag<T>(k4 * ek), ident);
         const Frag<T> ahT[2] = {transpose(to_frag<T>(a4[0] * ea), ident), transpose(to_frag<T>(a4[1] * ea), ident)};
         const Frag<T> bhT[2] = {transpose(to_frag<T>(b4[0] * ek), ident), transpose(to_frag<T>(b4[1] * ek), ident)};
         const f32x4 bg4[2] = {b4[0] * edn, b4[1] * edn};
-        f32x4 dqh = mm(fAqk, khT, zero4());
-        dqh = mm(fAqb[0], bhT[0], dqh);
-        dqh = mm(fAqb[1], bhT[1], dqh);
-        f32x4 dkh = mm(getT(0), qhT, zero4());
-        dkh = mm(getT(3), ahT[0], dkh);
-        dkh = mm(getT(4), ahT[1], dkh);
+        f32x4 dqh = mm(fin(0), khT, zero4());
+        dqh = mm(fin(1), bhT[0], dqh);
+        dqh = mm(fin(2), bhT[1], dqh);
+        f32x4 dkh = mm(finT(0), qhT, zero4());
+        dkh = mm(finT(3), ahT[0], dkh);
+        dkh = mm(finT(4), ahT[1], dkh);
         f32x4 dah[2], dbh[2];
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
-            f32x4 x = mm(fAak[r], khT, zero4());
-            x = mm(fAab[r][0], bhT[0], x);
-            x = mm(fAab[r][1], bhT[1], x);
+            f32x4 x = mm(fin(3 + r), khT, zero4());
+            x = mm(fin(5 + 2 * r), bhT[0], x);
+            x = mm(fin(6 + 2 * r), bhT[1], x);
             dah[r] = x;
-            f32x4 y = mm(getT(1 + r), qhT, zero4());          // here r plays the role of the b rank s
-            y = mm(getT(5 + r), ahT[0], y);
-            y = mm(getT(7 + r), ahT[1], y);
+            f32x4 y = mm(finT(1 + r), qhT, zero4());          // here r plays the role of the b rank s
+            y = mm(finT(5 + r), ahT[0], y);
+            y = mm(finT(7 + r), ahT[1], y);
             dbh[r] = y;
         }
         const f32x4 dq = (dqh * eq + dqg * egi) * scale;
         const f32x4 dk = dkh * ek + dkg * edn;
-        const f32x4 da[2] = {dah[0] * ea + dag[0] * ege, dah[1] * ea + dag[1] * ege};
+        const f32x4 da[2] = {dah[0] * ea + dag[j][0] * ege, dah[1] * ea + dag[j][1] * ege};
         const f32x4 db[2] = {dbh[0] * ek + dbg[0] * edn, dbh[1] * ek + dbg[1] * edn};
         const f32x4 Dge = da[0] * a4[0] + da[1] * a4[1];
         const f32x4 Dgi = dq * q4 - dk * k4 - db[0] * b4[0] - db[1] * b4[1];
         const f32x4 dgl = exp4<T>(gl) * hh4 + sum16(dkg * kg4 + dbg[0] * bg4[0] + dbg[1] * bg4[1]);
         const f32x4 dg = rscan16_incl(Dgi + Dge) - Dge + dgl;
         if (STAGE_OUT) {
-            const int half = kt & 1;
-            put(0, half, to_frag<T>(dq));
-            put(1, half, to_frag<T>(dk));
-            put(2, half, to_frag<T>(da[0]));
-            put(3, half, to_frag<T>(da[1]));
-            put(4, half, to_frag<T>(db[0]));
-            put(5, half, to_frag<T>(db[1]));
-            if (!GKF32) put(6, half, to_frag<T>(dg));
+            put(0, kt, to_frag<T>(dq));
+            put(1, kt, to_frag<T>(dk));
+            put(2, kt, to_frag<T>(da[0]));
+            put(3, kt, to_frag<T>(da[1]));
+            put(4, kt, to_frag<T>(db[0]));
+            put(5, kt, to_frag<T>(db[1]));
+            if (!GKF32) put(6, kt, to_frag<T>(dg));
             else if (rowok) st_gk4<GKF32>(dgkp + go + 16 * kt * GS, 0, dg);
-            if (half) {
-                const uint32_t qpitch = (uint32_t)(H * K) * ES, apitch = qpitch * RANK, b0 = (uint32_t)(16 * (kt - 1)) * ES;
-                flush(0, p.dq + qb, qpitch, b0);
-                flush(1, p.dk + qb, qpitch, b0);
-                flush(2, p.da + ab, apitch, b0);
-                flush(3, p.da + ab, apitch, b0 + qpitch);
-                flush(4, p.db + ab, apitch, b0);
-                flush(5, p.db + ab, apitch, b0 + qpitch);
-                if (!GKF32) flush(6, reinterpret_cast<T*>(dgkp), qpitch, b0);
-            }
         } else if (rowok) {
             st_frag(at(p.dq + qb, qo + 16 * kt * ES), to_frag<T>(dq));
             st_frag(at(p.dk + qb, qo + 16 * kt * ES), to_frag<T>(dk));
@@ -417,23 +410,43 @@ __global__ __launch_bounds__(64) void chunk_grad_kernel(ChunkArgs<T> p) {
             st_gk4<GKF32>(dgkp + go + 16 * kt * GS, 0, dg);
         }
     }
-    if (STAGE_OUT) {
+    // ---- own value tiles: dv += kg dS over all channel tiles ------------------------------------------------------
 #pragma unroll
-        for (int vt = 0; vt < VT; vt += 2) {
-            put(0, 0, to_frag<T>(dv[vt]));
-            put(0, 1, to_frag<T>(dv[vt + 1]));
-            flush(0, p.dv + vb, (uint32_t)(H * V) * ES, (uint32_t)(16 * vt) * ES);
-        }
-    } else if (rowok) {
+    for (int j = 0; j < VTW; ++j) {
+        f32x4 x = dv[j];
 #pragma unroll
-        for (int vt = 0; vt < VT; ++vt) st_frag(at(p.dv + vb, vo + 16 * vt * ES), to_frag<T>(dv[vt]));
+        for (int kt = 0; kt < KT; ++kt) x = mm(ld_tile(sKg + kt * TILE), dhv[j][kt], x);
+        if (STAGE_OUT) st_frag(reinterpret_cast<T*>(sOut + 7 * CH * L::OPK + c * L::OPV) + 16 * (vt0 + j) + 4 * g, to_frag<T>(x));
+        else if (rowok) st_frag(at(p.dv + vb, vo + 16 * (vt0 + j) * ES), to_frag<T>(x));
     }
-    PHASE_CLOCK(p, blk, 5);
+    if (STAGE_OUT) {
+        __syncthreads();                                       // (4) the staged rows are complete
+        // whole rows, 16 bytes a lane; the waves take turns over the instructions
+        constexpr int LRK = K * (int)ES / 16, RPK = 64 / LRK, NUK = CH / RPK;   // lanes per row, rows per instruction, instructions per tensor
+        constexpr int LRV = V * (int)ES / 16, RPV = 64 / LRV, NUV = CH / RPV;
+        constexpr int NKT = GKF32 ? 6 : 7, NU = NKT * NUK + NUV;
+        const uint32_t qpitch = (uint32_t)(H * K) * ES, apitch = qpitch * RANK;
+#pragma unroll
+        for (int t = 0; t < (NU + NW - 1) / NW; ++t) {
+            const int u = w + t * NW;
+            if (u < NKT * NUK) {
+                const int m = u / NUK, r = (u % NUK) * RPK + l / LRK, e = (l % LRK) * 16;
+                char* base = reinterpret_cast<char*>(m == 0 ? p.dq + qb : m == 1 ? p.dk + qb : m < 4 ? p.da + ab : m < 6 ? p.db + ab : reinterpret_cast<T*>(dgkp));
+                const uint32_t pitch = (m < 2 || m == 6) ? qpitch : apitch, off = (m == 3 || m == 5) ? qpitch : 0;
+                const i32x4 x = *reinterpret_cast<const i32x4*>(sOut + (m * CH + r) * L::OPK + e);
+                if (r < cp.len) *reinterpret_cast<i32x4*>(base + (uint32_t)r * pitch + off + e) = x;
+            } else if (u < NU) {
+                const int r = (u - NKT * NUK) * RPV + l / LRV, e = (l % LRV) * 16;
+                const i32x4 x = *reinterpret_cast<const i32x4*>(sOut + 7 * CH * L::OPK + r * L::OPV + e);
+                if (r < cp.len) *reinterpret_cast<i32x4*>(reinterpret_cast<char*>(p.dv + vb) + (uint32_t)r * (uint32_t)(H * V) * ES + e) = x;
+            }
+        }
+    }
 }
 
 template <typename T, int K, int V>
 static hipError_t launch_chunk_grad_kv(const ChunkArgs<T>& a, hipStream_t stream) {
-    dim3 grid(a.st.nch, a.H), block(64);
+    dim3 grid(a.st.nch, a.H), block(64 * NW);
     constexpr bool kAlwaysF32 = sizeof(T) == 4;
     if (kAlwaysF32 || a.gk_f32) hipLaunchKernelGGL((chunk_grad_kernel<T, true, K, V>), grid, block, 0, stream, a);
     else hipLaunchKernelGGL((chunk_grad_kernel<T, kAlwaysF32, K, V>), grid, block, 0, stream, a);
