@@ -33,24 +33,24 @@ template <typename T, int K, int V> struct CgLds {
     // do, v, v_new (2 ranks), dv_new (2 ranks) of the chunk, [matrix][token][value], rows padded by 16 bytes
     static constexpr int VP = V + 16 / ES;
     static constexpr int TOK = 0, TOK_B = 6 * CH * VP * ES;
-    // per wave: its part of A_qk^T, A_ak^T (2 ranks), fp32 tiles in fragment order
-    static constexpr int SCORE = TOK + TOK_B, SCORE_B = NW * 3 * 1024;
+    // first, per wave: its part of A_qk^T, A_ak^T (2 ranks), fp32 tiles in fragment order (read between barriers 1
+    // and 2); later the nine score-gradient tiles, as fragments and as fragments of their transposes (written
+    // between barriers 2 and 3)
+    static constexpr int SCORE = TOK + TOK_B, SCORE_B = NW * 3 * 1024, FIN = SCORE, FIN_B = 18 * TILE * ES;
     // kg of every channel tile (fragments), for dv
-    static constexpr int KG = SCORE + SCORE_B, KG_B = (K / 16) * TILE * ES;
-    // the nine score-gradient tiles, as fragments and as fragments of their transposes
-    static constexpr int FIN = KG + KG_B, FIN_B = 18 * TILE * ES;
+    static constexpr int KG = SCORE + (SCORE_B > FIN_B ? SCORE_B : FIN_B), KG_B = (K / 16) * TILE * ES;
     // first: per wave its part of the nine tiles (fp32); later, for 2-byte elements: the rows of the seven
     // gradients, so that they leave as whole rows (a lane holds 8 bytes of a row; 8-byte stores of four lanes
     // would write 32-byte pieces, half of what HBM writes at once)
     static constexpr bool STAGE_OUT = ES == 2;
     static constexpr int OPK = K * ES + 16, OPV = V * ES + 16;       // padded rows
     static constexpr int PART_B = NW * 9 * 1024, OUT_B = STAGE_OUT ? (7 * OPK + OPV) * CH : 0;
-    static constexpr int R1 = FIN + FIN_B, R1_B = PART_B > OUT_B ? PART_B : OUT_B;
+    static constexpr int R1 = KG + KG_B, R1_B = PART_B > OUT_B ? PART_B : OUT_B;
     static constexpr int BYTES = R1 + R1_B;
 };
 
 template <typename T, bool GKF32, int K, int V>
-__global__ __launch_bounds__(64 * NW) void chunk_grad_kernel(ChunkArgs<T> p) {
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2))) void chunk_grad_kernel(ChunkArgs<T> p) {
     constexpr int KT = K / 16, VT = V / 16, KT2 = KT / 2, KTW = KT / NW, VTW = VT / NW;
     static_assert(KT % NW == 0 && VT % NW == 0 && (KTW == 1 || KTW == 2), "a wave owns one channel tile or one stored pair");
     typedef CgLds<T, K, V> L;
@@ -91,7 +91,8 @@ __global__ __launch_bounds__(64 * NW) void chunk_grad_kernel(ChunkArgs<T> p) {
     const int kt0 = w * KTW, vt0 = w * VTW;                   // first own channel tile / value tile
 
     // ---- everything the wave reads from global memory is requested here, before any arithmetic -----------------
-    // (only the checkpoint of dS waits for the large shapes: it is used last and would not fit next to the rest)
+    // (the large shapes cannot hold all of it at once at two waves per SIMD: there the tiles of S and dS that are
+    // used later are requested later, each a phase of arithmetic ahead of its first use)
     Frag<T> rq[KTW], rk[KTW], ra[2][KTW], rb[2][KTW];          // own channel tiles of the inputs
     f32x4 rg[KTW];
 #pragma unroll
@@ -130,16 +131,21 @@ __global__ __launch_bounds__(64 * NW) void chunk_grad_kernel(ChunkArgs<T> p) {
             for (int kp = 0; kp < KT2; ++kp) ld_pair(X + (kp * VT + vt0 + j) * PAIR, dst[j][2 * kp], dst[j][2 * kp + 1]);
     };
     Frag<T> wf[2][KT], wk[2][KTW];                             // w: all of it (v_new), and the own channel tiles
+    auto own_w_tiles = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
+        for (int s = 0; s < 2; ++s) {
+            if (KTW == 2) ld_pair(Wb + (s * KT2 + w) * PAIR, wk[s][0], wk[s][KTW - 1]);
+            else wk[s][0] = ld_pair_one(Wb + (s * KT2 + (w >> 1)) * PAIR, w & 1);
+        }
+    };
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
 #pragma unroll
         for (int kp = 0; kp < KT2; ++kp) ld_pair(Wb + (s * KT2 + kp) * PAIR, wf[s][2 * kp], wf[s][2 * kp + 1]);
-        if (KTW == 2) ld_pair(Wb + (s * KT2 + w) * PAIR, wk[s][0], wk[s][KTW - 1]);
-        else wk[s][0] = ld_pair_one(Wb + (s * KT2 + (w >> 1)) * PAIR, w & 1);
-    }
     Frag<T> hv[VTW][KT], hk[KTW][VT], dhv[VTW][KT], dhk[KTW][VT];
+    constexpr bool EARLY = sizeof(T) * K * V <= 2 * 64 * 64;
     own_vt_tiles(HC, hv);
-    own_kt_tiles(HC, hk);
+    if (EARLY) { own_kt_tiles(HC, hk); own_w_tiles(); }
     Frag<T> ut[VTW][2], yt[VTW][2];                            // u^T and dv_new^T of the own value tiles, both ranks
 #pragma unroll
     for (int j = 0; j < VTW; ++j) {
@@ -150,8 +156,7 @@ __global__ __launch_bounds__(64 * NW) void chunk_grad_kernel(ChunkArgs<T> p) {
     Frag<T> tmT[2][2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) ld_pair(p.ws.TM + chw * 1024 + s * PAIR, tmT[s][0], tmT[s][1]);
-    constexpr bool EARLY_DH = sizeof(T) * K * V <= 2 * 64 * 64;
-    if (EARLY_DH) { own_kt_tiles(DHC, dhk); own_vt_tiles(DHC, dhv); }
+    if (EARLY) { own_kt_tiles(DHC, dhk); own_vt_tiles(DHC, dhv); }
 
     const Frag<T> ident = ident_frag<T>();
 
@@ -205,6 +210,7 @@ __global__ __launch_bounds__(64 * NW) void chunk_grad_kernel(ChunkArgs<T> p) {
         st_frag(dst + 4 * CH * VP, transpose(yt[j][0], ident));
         st_frag(dst + 5 * CH * VP, transpose(yt[j][1], ident));
     }
+    if (!EARLY) { own_kt_tiles(HC, hk); own_w_tiles(); }
     __syncthreads();                                           // (1) sTok, sScore, sKg complete
     auto tokf = [&](int m, int vt) __attribute__((always_inline)) { return ld_frag(&sTok[(m * CH + c) * VP + 16 * vt + 4 * g]); };
 
@@ -296,7 +302,7 @@ __global__ __launch_bounds__(64 * NW) void chunk_grad_kernel(ChunkArgs<T> p) {
             part(7 + s, dAab[1][s]);
         }
     }
-    if (!EARLY_DH) { own_kt_tiles(DHC, dhk); own_vt_tiles(DHC, dhv); }
+    if (!EARLY) { own_kt_tiles(DHC, dhk); own_vt_tiles(DHC, dhv); }
     __syncthreads();                                           // (2) the parts of the nine tiles are complete
     // the waves share out the nine tiles: sum of the parts, causal mask, both orientations as fragments
 #pragma unroll
@@ -324,6 +330,15 @@ __global__ __launch_bounds__(64 * NW) void chunk_grad_kernel(ChunkArgs<T> p) {
         st_frag(reinterpret_cast<T*>(sOut + (m * CH + c) * L::OPK) + 16 * kt + 4 * g, f);
     };
 
+    // ---- own value tiles: dv += kg dS over all channel tiles ------------------------------------------------------
+#pragma unroll
+    for (int j = 0; j < VTW; ++j) {
+        f32x4 x = dv[j];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) x = mm(ld_tile(sKg + kt * TILE), dhv[j][kt], x);
+        if (STAGE_OUT) st_frag(reinterpret_cast<T*>(sOut + 7 * CH * L::OPK + c * L::OPV) + 16 * (vt0 + j) + 4 * g, to_frag<T>(x));
+        else if (rowok) st_frag(at(p.dv + vb, vo + 16 * (vt0 + j) * ES), to_frag<T>(x));
+    }
     // ---- own channel tiles, second pass: state products, score backward, final gradients ---------------------------
 #pragma unroll
     for (int j = 0; j < KTW; ++j) {
@@ -409,15 +424,6 @@ __global__ __launch_bounds__(64 * NW) void chunk_grad_kernel(ChunkArgs<T> p) {
             st_frag(at(p.db + ab, ao1 + 16 * kt * ES), to_frag<T>(db[1]));
             st_gk4<GKF32>(dgkp + go + 16 * kt * GS, 0, dg);
         }
-    }
-    // ---- own value tiles: dv += kg dS over all channel tiles ------------------------------------------------------
-#pragma unroll
-    for (int j = 0; j < VTW; ++j) {
-        f32x4 x = dv[j];
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt) x = mm(ld_tile(sKg + kt * TILE), dhv[j][kt], x);
-        if (STAGE_OUT) st_frag(reinterpret_cast<T*>(sOut + 7 * CH * L::OPK + c * L::OPV) + 16 * (vt0 + j) + 4 * g, to_frag<T>(x));
-        else if (rowok) st_frag(at(p.dv + vb, vo + 16 * (vt0 + j) * ES), to_frag<T>(x));
     }
     if (STAGE_OUT) {
         __syncthreads();                                       // (4) the staged rows are complete
