@@ -67,7 +67,7 @@ def interface_bytes(kernel, pass_, K, V, es, gs):
 
 def measured_traffic(workload, kernel_key, K, V):
     """HBM bytes per launch of one kernel from the committed rocprofv3 counter summary (profiles/hbm_traffic.json:
-    FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the same counter reads for a plain 1 GiB copy), or
+    FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the same counter reads for the streaming kernel of known traffic), or
     None when that summary does not cover the kernel.  The counters cannot be collected from inside this script."""
     try:
         table = json.load(open(os.path.join(ROOT, "profiles", "hbm_traffic.json"))).get(workload, {})
@@ -183,14 +183,31 @@ def main():
     torch.cuda.set_device(dev)
     wl = args.workload
     if wl == "copy":
-        # calibration workload for the HBM traffic counters: a plain device-to-device copy of known size
-        # (reads n bytes, writes n bytes per launch); not a benchmark of this library
-        n = 1 << 30
-        x = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
-        y = torch.empty_like(x)
-        sec = time_steps(lambda: y.copy_(x), args.steps, args.warmup)
+        # calibration workload, not a benchmark of the operator: the library's streaming kernel, whose traffic per
+        # launch is known exactly (the HBM traffic counters are scaled by what they read for the 1:1 launches,
+        # which come last and are the ones timed for "GB/s"), and the rate HBM sustains for several read:write mixes
+        import ctypes
+        from hdla_hip import _lib
+        lib = _lib.load()
+        n = 256 << 20
+        bufs = [torch.empty(n, dtype=torch.uint8, device=dev).fill_(i + 1) for i in range(6)]
+        stream = _lib.current_stream(dev)
+        turn = [0]
+
+        def launch(nr, nw):
+            # successive launches take different buffers, so that none is served from the 256 MB last-level cache
+            turn[0] += 1
+            rot = bufs[turn[0] % 6:] + bufs[:turn[0] % 6]
+            rd = (ctypes.c_void_p * 3)(*[b.data_ptr() for b in rot[:nr]], *([None] * (3 - nr)))
+            wr = (ctypes.c_void_p * 2)(*[b.data_ptr() for b in rot[3:3 + nw]], *([None] * (2 - nw)))
+            _lib.check(lib.hdla_calib_stream(rd, nr, wr, nw, n, stream), "hdla_calib_stream")
+
+        mixes = {}
+        for nr, nw in ((1, 0), (0, 1), (3, 1), (2, 1), (1, 2), (1, 1)):
+            sec = time_steps(lambda: launch(nr, nw), args.steps, args.warmup)
+            mixes[f"{nr}:{nw}"] = round((nr + nw) * n / sec / 1e9)
         print(json.dumps({"metric": "copy calibration", "bytes_read_per_launch": n, "bytes_written_per_launch": n,
-                          "ms_per_step": sec * 1e3, "GB/s": 2 * n / sec / 1e9}))
+                          "ms_per_step": sec * 1e3, "GB/s": 2 * n / sec / 1e9, "GB/s_by_read_write_mix": mixes}))
         return
     cfg = {"train": 2, "fwd": 1, "varlen": 3, "decode": 4}[wl]
     B, T, H, K, V = CONFIG_SHAPES[cfg]

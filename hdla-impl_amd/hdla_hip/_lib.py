@@ -63,6 +63,8 @@ def load():
     lib.hdla_chunk_bwd.argtypes = [F] + [P] * 16 + [P, ctypes.c_size_t, P]
     lib.hdla_chunk_stages.restype = ctypes.c_int
     lib.hdla_chunk_stages.argtypes = [F, ctypes.c_int, ctypes.c_int] + [P] * 18 + [P, ctypes.c_size_t, P]
+    lib.hdla_calib_stream.restype = ctypes.c_int
+    lib.hdla_calib_stream.argtypes = [ctypes.POINTER(P), ctypes.c_int, ctypes.POINTER(P), ctypes.c_int, ctypes.c_size_t, P]
     lib.hdla_recurrent_fwd.restype = ctypes.c_int
     lib.hdla_recurrent_fwd.argtypes = [F] + [P] * 6 + [ctypes.c_int] + [P] * 4
     _lib = lib

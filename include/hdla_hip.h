@@ -117,6 +117,14 @@ int hdla_recurrent_fwd(const hdla_dims* dims, const void* q, const void* k, cons
                        const void* b, const void* gk, int reverse, const float* h0, void* o, float* ht,
                        void* stream);
 
+/* Measurement aid; it has no counterpart in the reference.  One launch of a kernel that reads `n_read` (0..3)
+ * buffers and writes `n_write` (0..2) buffers of `bytes` bytes each (a multiple of 16; every pointer 16-byte
+ * aligned) and does nothing else.  Supported mixes (reads:writes): 1:0, 0:1, 1:1, 2:1, 3:1, 1:2; others return
+ * HDLA_ERR_SHAPE.  Its traffic is known exactly, which is what hardware traffic counters are scaled by, and the
+ * rate it reaches is the rate HBM sustains for that mix. */
+int hdla_calib_stream(const void* const* reads, int n_read, void* const* writes, int n_write, size_t bytes,
+                      void* stream);
+
 #ifdef __cplusplus
 }
 #endif
