@@ -40,7 +40,9 @@ int make_layout(const hdla_dims* d, int pass, WsLayout& L, int& nch) {
     if (rc) return rc;
     if (d->N > 65535) return HDLA_ERR_SHAPE;
     const int NT = (d->T + CHUNK - 1) / CHUNK;
-    nch = d->cu_seqlens ? NT + d->N : d->B * NT;
+    const long long nch64 = d->cu_seqlens ? (long long)NT + d->N : (long long)d->B * NT;
+    if (nch64 * d->H > 0x7fffffffLL) return HDLA_ERR_SHAPE;        // one workgroup per (chunk, head), one grid dimension
+    nch = (int)nch64;
     const size_t es = d->in_dtype == HDLA_BF16 ? 2 : 4;
     const size_t chw = (size_t)d->H * (size_t)nch;
     const size_t K = d->K, V = d->V;
@@ -158,7 +160,7 @@ const char* hdla_strerror(int code) {
     switch (code) {
         case HDLA_OK: return "success";
         case HDLA_ERR_NULL: return "a required pointer is NULL";
-        case HDLA_ERR_SHAPE: return "unsupported shape (need K,V in {64,128}, B,H,N >= 1, T >= 0, H,N <= 65535)";
+        case HDLA_ERR_SHAPE: return "unsupported shape (need K,V in {64,128}, B,H,N >= 1, T >= 0, H,N <= 65535, chunks x heads < 2^31)";
         case HDLA_ERR_RANK: return "only rank R = 2 is supported";
         case HDLA_ERR_DTYPE: return "unsupported dtype (in_dtype bf16|fp32; gk fp32, or bf16 with bf16 inputs)";
         case HDLA_ERR_WORKSPACE: return "workspace is NULL, not 256-byte aligned, or smaller than hdla_workspace_bytes()";

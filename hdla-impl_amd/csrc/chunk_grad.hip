@@ -65,7 +65,14 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
     float* const sPart = reinterpret_cast<float*>(smem + L::R1);
     char* const sOut = smem + L::R1;
 
-    const int cid = blockIdx.x, h = blockIdx.y;
+    // Which of the two indices runs fastest over the workgroups decides which rows of the [token][head][channel]
+    // tensors the workgroups resident at one time touch.  Measured: with rows of 4 KiB and more, neighbouring
+    // workgroups should be the heads of one chunk (together they read whole rows; chunk-fastest, all of them would
+    // touch the same few hundred bytes of every row, a fraction of the HBM channels); with shorter rows the chunks
+    // of one head, whose workspace records are contiguous.
+    const bool head_fastest = (uint32_t)(p.H * K) * sizeof(T) >= 4096;
+    const int cid = head_fastest ? blockIdx.x / p.H : blockIdx.x % p.st.nch;
+    const int h = head_fastest ? blockIdx.x % p.H : blockIdx.x / p.st.nch;
     ChunkPos cp;
     if (!locate_chunk(p.st, cid, cp)) return;                 // uniform over the workgroup
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -452,7 +459,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 
 template <typename T, int K, int V>
 static hipError_t launch_chunk_grad_kv(const ChunkArgs<T>& a, hipStream_t stream) {
-    dim3 grid(a.st.nch, a.H), block(64 * NW);
+    dim3 grid(a.st.nch * a.H), block(64 * NW);
     constexpr bool kAlwaysF32 = sizeof(T) == 4;
     if (kAlwaysF32 || a.gk_f32) hipLaunchKernelGGL((chunk_grad_kernel<T, true, K, V>), grid, block, 0, stream, a);
     else hipLaunchKernelGGL((chunk_grad_kernel<T, kAlwaysF32, K, V>), grid, block, 0, stream, a);

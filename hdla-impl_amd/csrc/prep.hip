@@ -20,7 +20,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 
     __shared__ __attribute__((aligned(16))) float sN[32 * LDP];   // A_ab, rank-major
     __shared__ __attribute__((aligned(16))) float sT[32 * LDP];   // (I - A_ab)^-1
 
-    const int cid = blockIdx.x, h = blockIdx.y;
+    // Which of the two indices runs fastest over the workgroups decides which rows of the [token][head][channel]
+    // tensors the workgroups resident at one time touch.  Measured: with rows of 4 KiB and more, neighbouring
+    // workgroups should be the heads of one chunk (together they read whole rows; chunk-fastest, all of them would
+    // touch the same few hundred bytes of every row, a fraction of the HBM channels); with shorter rows the chunks
+    // of one head, whose workspace records are contiguous.
+    const bool head_fastest = (uint32_t)(p.H * K) * sizeof(T) >= 4096;
+    const int cid = head_fastest ? blockIdx.x / p.H : blockIdx.x % p.st.nch;
+    const int h = head_fastest ? blockIdx.x % p.H : blockIdx.x / p.st.nch;
     ChunkPos cp;
     if (!locate_chunk(p.st, cid, cp)) return;
     const int l = lane_id(), g = l >> 4, c = l & 15;
@@ -33,7 +40,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 
     const int64_t voff = (tok * H + h) * V + 4 * g;
     const int64_t chw = (int64_t)h * p.st.nch + cid;                // chunk-head slot in the workspace
     const float scale = p.scale;
-    const int blk = blockIdx.y * gridDim.x + blockIdx.x;
+    const int blk = blockIdx.x;
     PHASE_CLOCK(p, blk, 0);
 
     // ---- phase A: cumulative decays and the score tiles (rows i, inner j) -----------------------------------
@@ -233,7 +240,7 @@ __global__ void build_chunk_table_kernel(const int64_t* cu, int N, int nch, int3
 
 template <typename T, int K, int V>
 static hipError_t launch_prep_kv(const ChunkArgs<T>& a, bool bwd, hipStream_t stream) {
-    dim3 grid(a.st.nch, a.H), block(64);
+    dim3 grid(a.st.nch * a.H), block(64);
     constexpr bool kAlwaysF32 = sizeof(T) == 4;
     if (kAlwaysF32 || a.gk_f32) {
         if (bwd) hipLaunchKernelGGL((prep_kernel<T, true, K, V, true>), grid, block, 0, stream, a);
