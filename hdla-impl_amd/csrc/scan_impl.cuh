@@ -62,7 +62,7 @@ template <typename T, int K, int V, int NWC> struct ScanCfg {
     // puts them (the shapes whose operands would not fit the register file twice over) ...
     static constexpr bool pipelined(bool with_o) { return KB <= 128 || (KB <= 256 && !(NWC == 8 && with_o)); }
     // ... and whether that includes the operands of the state update
-    static constexpr bool early_update_reads() { return KB <= 128 || (KB <= 256 && NWC <= 4 && NM == 0); }
+    static constexpr bool early_update_reads(bool with_o) { return KB <= 128 || (KB <= 256 && NWC <= 4 && (NM == 0 || with_o)); }
 };
 
 // A shared operand block as the loading waves see it: NI pieces of 1 KiB, lane l taking 16 bytes of each.  The
@@ -194,7 +194,7 @@ __device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem,
     constexpr int KT = K / 16, KT2 = KT / 2, VT = V / 16, NM = C::NM, ES = sizeof(T);
     constexpr BlkF B = blk_fwd(K, sizeof(T), WRITE_O);
     constexpr bool PIPE = C::pipelined(WRITE_O);
-    constexpr bool PIPE_UPD = PIPE && C::early_update_reads();
+    constexpr bool PIPE_UPD = PIPE && C::early_update_reads(WRITE_O);
     constexpr int NI = B.SIZE / 1024, SLOT = B.SIZE;
     typedef ScanLds<T, K, V, NWC, SLOT, WRITE_O ? OUT_O : OUT_STATE> L;
     constexpr int OROW = L::OROW, OB_HC = L::OB_HC, OB = L::OB;
@@ -459,7 +459,7 @@ __device__ __forceinline__ void scan_bwd_body(const ChunkArgs<T>& p, char* smem,
     constexpr SlotB B = slot_bwd(K, sizeof(T));
     constexpr int SFWD = blk_fwd(K, sizeof(T), false).SIZE, SBWD = blk_bwd(K, sizeof(T)).SIZE, NT = B.NIF;
     constexpr bool PIPE = C::pipelined(false);
-    constexpr bool PIPE_UPD = PIPE && C::early_update_reads();
+    constexpr bool PIPE_UPD = PIPE && C::early_update_reads(false);
     constexpr int NI = B.SIZE / 1024, SLOT = B.SIZE;
     typedef ScanLds<T, K, V, NWC, SLOT, OUT_GRAD> L;
     constexpr int OB_HC = L::OB_HC, OB = L::OB;
