@@ -1,10 +1,15 @@
 // prep kernel: everything of a 16-token chunk that does not depend on the recurrent state.
 //
-// Replaces, for one (chunk, head) per wavefront, the reference's chunk-local cumsum (fla chunk_rwkv6_fwd_cumsum,
+// Replaces, for one (chunk, head) per workgroup, the reference's chunk-local cumsum (fla chunk_rwkv6_fwd_cumsum,
 // called at HRDPLR/hrdplr.py:44), the two score kernels (HRDPLR/fwd_triton.py:22-290 and :305-514), the
 // triangular inverse (HRDPLR/fwd_triton.py:601-667) and the WY kernel (HRDPLR/fwd_triton.py:685-790).
 // The four score matrices never reach HBM: they are MFMA accumulators, (I - A_ab)^-1 is solved in LDS, and
 // w, u and the gated copies are written once, in the fragment order the state scans read them in.
+//
+// A wave handles 64 channels: K = 64 is one wave per (chunk, head); K = 128 is a workgroup of two, each with its
+// half of the channel tiles and of the value tiles.  The score tiles are sums over channels: the two exchange
+// their parts through LDS and each then solves the (small) triangular system for itself.  One wave with all 128
+// channels needs the whole register file, and at one wave per SIMD nothing hides its memory round trips.
 #include "hdla_common.cuh"
 #include "hdla_launch.h"
 
@@ -13,12 +18,19 @@ namespace hdla {
 constexpr int LDP = 36;   // padded row length of the 32x32 LDS matrices (keeps 16-byte row alignment)
 
 template <typename T, bool GKF32, int K, int V, bool BWD>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 : 1, K == 64 ? 2 : 1))) void prep_kernel(ChunkArgs<T> p) {
-    constexpr int KT = K / 16, VT = V / 16, KT2 = KT / 2;
+__global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void prep_kernel(ChunkArgs<T> p) {
+    constexpr int NWP = K / 64;                       // waves per (chunk, head)
+    constexpr int KTW = 4, VT = V / 16, VTW = VT / NWP, KT2 = K / 32;
     constexpr int SAS = blk_fwd(K, sizeof(T), !BWD).SIZE / (int)sizeof(T);   // elements between (chunk, head) slots
     constexpr int SBS = blk_bwd(K, sizeof(T)).SIZE / (int)sizeof(T);
-    __shared__ __attribute__((aligned(16))) float sN[32 * LDP];   // A_ab, rank-major
-    __shared__ __attribute__((aligned(16))) float sT[32 * LDP];   // (I - A_ab)^-1
+    __shared__ __attribute__((aligned(16))) float sNw[NWP][32 * LDP];   // A_ab, rank-major (one copy per wave)
+    __shared__ __attribute__((aligned(16))) float sTw[NWP][32 * LDP];   // (I - A_ab)^-1
+    constexpr int NPART = BWD ? 8 : 9;                                    // score tiles that are summed over the waves
+    __shared__ __attribute__((aligned(16))) float sPart[NWP > 1 ? NWP * NPART * 256 : 4];
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    float* const sN = sNw[w];
+    float* const sT = sTw[w];
+    const int kt0 = w * KTW, vt0 = w * VTW;                              // first own channel tile / value tile
 
     // Which of the two indices runs fastest over the workgroups decides which rows of the [token][head][channel]
     // tensors the workgroups resident at one time touch.  Measured: with rows of 4 KiB and more, neighbouring
@@ -44,27 +56,28 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 
     PHASE_CLOCK(p, blk, 0);
 
     // ---- phase A: cumulative decays and the score tiles (rows i, inner j) -----------------------------------
-    f32x4 gi[KT], ge[KT];
+    f32x4 gi[KTW], ge[KTW];
     f32x4 aqk = zero4(), aqb[2] = {zero4(), zero4()}, aak[2] = {zero4(), zero4()};
     f32x4 aab[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
     f32x4 aqbT[2] = {zero4(), zero4()};
     // the inputs of the chunk stay in registers (as loaded) for the second use in phase C: the working set of the
     // resident waves is larger than the L2, so a second load would come from HBM again
-    Frag<T> rq[KT], rk[KT], ra[2][KT], rb[2][KT];
+    Frag<T> rq[KTW], rk[KTW], ra[2][KTW], rb[2][KTW];       // own channel tiles; index kt below is local, kt0 + kt global
     // v is used last (phase D) but requested first: the barriers in between would otherwise keep its loads, and a
     // full round trip to HBM, behind everything else
-    Frag<T> rv[VT];
+    Frag<T> rv[VTW];
 #pragma unroll
-    for (int vt = 0; vt < VT; ++vt) rv[vt] = ld_frag_sel(p.v + voff + 16 * vt, rowok);
+    for (int vt = 0; vt < VTW; ++vt) rv[vt] = ld_frag_sel(p.v + voff + 16 * (vt0 + vt), rowok);
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt) {
-        const f32x4 g4 = ld_gk4<GKF32>(p.gk, qoff + 16 * kt, rowok);
-        rq[kt] = ld_frag_sel(p.q + qoff + 16 * kt, rowok);
-        rk[kt] = ld_frag_sel(p.k + qoff + 16 * kt, rowok);
-        ra[0][kt] = ld_frag_sel(p.a + aoff0 + 16 * kt, rowok);
-        ra[1][kt] = ld_frag_sel(p.a + aoff1 + 16 * kt, rowok);
-        rb[0][kt] = ld_frag_sel(p.b + aoff0 + 16 * kt, rowok);
-        rb[1][kt] = ld_frag_sel(p.b + aoff1 + 16 * kt, rowok);
+    for (int kt = 0; kt < KTW; ++kt) {
+        const int ko = 16 * (kt0 + kt);
+        const f32x4 g4 = ld_gk4<GKF32>(p.gk, qoff + ko, rowok);
+        rq[kt] = ld_frag_sel(p.q + qoff + ko, rowok);
+        rk[kt] = ld_frag_sel(p.k + qoff + ko, rowok);
+        ra[0][kt] = ld_frag_sel(p.a + aoff0 + ko, rowok);
+        ra[1][kt] = ld_frag_sel(p.a + aoff1 + ko, rowok);
+        rb[0][kt] = ld_frag_sel(p.b + aoff0 + ko, rowok);
+        rb[1][kt] = ld_frag_sel(p.b + aoff1 + ko, rowok);
         gi[kt] = scan16_incl(g4);
         ge[kt] = gi[kt] - g4;
         const f32x4 m = bcast16(gi[kt], MID);
@@ -88,6 +101,19 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 
             for (int r = 0; r < 2; ++r) aab[r][s] = mm3(ah[r], bh[s], aab[r][s]);
         }
     }
+    if (NWP > 1) {
+        // sums over all channels: every wave leaves its parts in LDS and adds the others'
+        f32x4* const tiles[9] = {&aak[0], &aak[1], &aab[0][0], &aab[0][1], &aab[1][0], &aab[1][1],
+                                 BWD ? &aqbT[0] : &aqb[0], BWD ? &aqbT[1] : &aqb[1], &aqk};
+#pragma unroll
+        for (int i = 0; i < NPART; ++i) *reinterpret_cast<f32x4*>(&sPart[((w * NPART + i) * 64 + l) * 4]) = *tiles[i];
+        __syncthreads();
+#pragma unroll
+        for (int ww = 1; ww < NWP; ++ww)
+#pragma unroll
+            for (int i = 0; i < NPART; ++i)
+                *tiles[i] += *reinterpret_cast<const f32x4*>(&sPart[((((w + ww) % NWP) * NPART + i) * 64 + l) * 4]);
+    }
     // causal masks: lane (g,c) reg i is entry (row c, inner 4g+i)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -97,11 +123,13 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 
         if (!lt) { aak[0][i] = 0.f; aak[1][i] = 0.f; aab[0][0][i] = 0.f; aab[0][1][i] = 0.f; aab[1][0][i] = 0.f; aab[1][1][i] = 0.f; }
         if (!tle) { aqbT[0][i] = 0.f; aqbT[1][i] = 0.f; }
     }
-    if (!BWD) {
-        st_tile(p.ws.AQK + chw * SAS, to_frag<T>(aqk));
-        st_pair2(p.ws.AQB + chw * SAS, to_frag<T>(aqb[0]), to_frag<T>(aqb[1]));
-    } else {
-        st_pair2(p.ws.AQBT + chw * SBS, to_frag<T>(aqbT[0]), to_frag<T>(aqbT[1]));
+    if (w == 0) {
+        if (!BWD) {
+            st_tile(p.ws.AQK + chw * SAS, to_frag<T>(aqk));
+            st_pair2(p.ws.AQB + chw * SAS, to_frag<T>(aqb[0]), to_frag<T>(aqb[1]));
+        } else {
+            st_pair2(p.ws.AQBT + chw * SBS, to_frag<T>(aqbT[0]), to_frag<T>(aqbT[1]));
+        }
     }
 #pragma unroll
     for (int r = 0; r < 2; ++r)
@@ -147,7 +175,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 
         for (int s2 = 0; s2 < 2; ++s2)
             tm[s][s2] = to_frag<T>(*reinterpret_cast<const f32x4*>(&sT[(16 * s + c) * LDP + 16 * s2 + 4 * g]));
     const Frag<T> ident = ident_frag<T>();
-    if (BWD) {
+    if (BWD && w == NWP - 1) {
         // for the chunk_grad kernel: the four blocks transposed, as fragments (two tile pairs), ready to load
         T* tmw = p.ws.TM + chw * 1024;
 #pragma unroll
@@ -156,11 +184,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 
 
     // ---- phase C: w = Tm ag and the gated copies, two channel tiles (one stored pair) at a time -----------------
 #pragma unroll
-    for (int kp = 0; kp < KT2; ++kp) {
+    for (int kpl = 0; kpl < KTW / 2; ++kpl) {
+        const int kp = kt0 / 2 + kpl;                         // stored pair
         Frag<T> fw[2][2], fkgT[2], fbgT[2][2], fqg[2], fqgT[2];   // [..][tile of the pair]
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-            const int kt = 2 * kp + e;
+            const int kt = 2 * kpl + e;
             const f32x4 gl = bcast16(gi[kt], CH - 1);
             const f32x4 egi = exp4<T>(gi[kt]), ege = exp4<T>(ge[kt]), edn = exp4<T>(gl - gi[kt]);
             const Frag<T> agT[2] = {transpose(to_frag<T>(to_f32(ra[0][kt]) * ege), ident),
@@ -179,7 +208,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 
             if (BWD) fqgT[e] = transpose(fqg[e], ident);
             if (c == 0) {
                 const f32x4 egl = exp4<T>(gl);
-                *reinterpret_cast<f32x4*>(p.ws.EGL + chw * (SAS * (int)sizeof(T) / 4) + 16 * kt + 4 * g) = egl;
+                *reinterpret_cast<f32x4*>(p.ws.EGL + chw * (SAS * (int)sizeof(T) / 4) + 16 * (kt0 + kt) + 4 * g) = egl;
             }
         }
 #pragma unroll
@@ -196,8 +225,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(K == 64 ? 2 
     // ---- phase D: u = Tm (A_ak v), kept transposed (rows value, inner token) ---------------------------------
     const Frag<T> aakf[2] = {to_frag<T>(aak[0]), to_frag<T>(aak[1])};
 #pragma unroll
-    for (int vt = 0; vt < VT; ++vt) {
-        const Frag<T> vT = transpose(rv[vt], ident);
+    for (int vl = 0; vl < VTW; ++vl) {
+        const int vt = vt0 + vl;
+        const Frag<T> vT = transpose(rv[vl], ident);
         st_tile(p.ws.VTT + (chw * VT + vt) * TILE, vT);
         const Frag<T> mT[2] = {to_frag<T>(mm(vT, aakf[0], zero4())), to_frag<T>(mm(vT, aakf[1], zero4()))};
         Frag<T> fu[2];
@@ -240,7 +270,7 @@ __global__ void build_chunk_table_kernel(const int64_t* cu, int N, int nch, int3
 
 template <typename T, int K, int V>
 static hipError_t launch_prep_kv(const ChunkArgs<T>& a, bool bwd, hipStream_t stream) {
-    dim3 grid(a.st.nch * a.H), block(64);
+    dim3 grid(a.st.nch * a.H), block(K);
     constexpr bool kAlwaysF32 = sizeof(T) == 4;
     if (kAlwaysF32 || a.gk_f32) {
         if (bwd) hipLaunchKernelGGL((prep_kernel<T, true, K, V, true>), grid, block, 0, stream, a);
