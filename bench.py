@@ -47,7 +47,7 @@ def interface_bytes(kernel, pass_, K, V, es, gs):
     QG, AQK, AQB = 16 * K * es, 256 * es, 512 * es
     AQBT, QGT, TM = 512 * es, 16 * K * es, 1024 * es
     HC = DHC = K * V * es
-    VN = DVN = 32 * V * es
+    DVN = 32 * V * es
     inputs = 2 * 16 * K * es + 16 * K * gs + 2 * 32 * K * es + 16 * V * es          # q,k,gk,a,b,v
     if kernel == "prep":
         out = W + UT + KGT + BGT + VTT + EGL + ((QG + AQK + AQB) if pass_ == 0 else (AQBT + QGT + TM))
