@@ -39,18 +39,18 @@ template <typename T, int K, int V> struct CgLds {
     static constexpr int SCORE = TOK + TOK_B, SCORE_B = NW * 3 * 1024, FIN = SCORE, FIN_B = 18 * TILE * ES;
     // kg of every channel tile (fragments), for dv
     static constexpr int KG = SCORE + (SCORE_B > FIN_B ? SCORE_B : FIN_B), KG_B = (K / 16) * TILE * ES;
-    // first: per wave its part of the nine tiles (fp32); later, for 2-byte elements: the rows of the seven
+    // first: the parts of the nine tiles (fp32), summed in two rounds through NW/2 slots; later, for 2-byte elements: the rows of the seven
     // gradients, so that they leave as whole rows (a lane holds 8 bytes of a row; 8-byte stores of four lanes
     // would write 32-byte pieces, half of what HBM writes at once)
     static constexpr bool STAGE_OUT = ES == 2;
     static constexpr int OPK = K * ES + 16, OPV = V * ES + 16;       // padded rows
-    static constexpr int PART_B = NW * 9 * 1024, OUT_B = STAGE_OUT ? (7 * OPK + OPV) * CH : 0;
+    static constexpr int PART_B = (NW / 2) * 9 * 1024, OUT_B = STAGE_OUT ? (7 * OPK + OPV) * CH : 0;
     static constexpr int R1 = KG + KG_B, R1_B = PART_B > OUT_B ? PART_B : OUT_B;
     static constexpr int BYTES = R1 + R1_B;
 };
 
 template <typename T, bool GKF32, int K, int V>
-__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2))) void chunk_grad_kernel(ChunkArgs<T> p) {
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((sizeof(T) * K * V <= 2 * 64 * 64) ? 3 : sizeof(T) == 2 ? 2 : 1, (sizeof(T) * K * V <= 2 * 64 * 64) ? 3 : 2))) void chunk_grad_kernel(ChunkArgs<T> p) {
     constexpr int KT = K / 16, VT = V / 16, KT2 = KT / 2, KTW = KT / NW, VTW = VT / NW;
     static_assert(KT % NW == 0 && VT % NW == 0 && (KTW == 1 || KTW == 2), "a wave owns one channel tile or one stored pair");
     typedef CgLds<T, K, V> L;
@@ -298,19 +298,26 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
         }
     }
     // tile indices: 0 A_qk, 1+s A_qb^s, 3+s A_ak^s, 5+2r+s A_ab^{r s}
+    // Sum over the waves in two rounds (half the LDS of one round): the upper half of the waves leave their parts,
+    // the lower half add them to their own and leave the sums.
+    if (!EARLY) { own_kt_tiles(DHC, dhk); own_vt_tiles(DHC, dhv); }
     {
-        auto part = [&](int idx, f32x4 x) __attribute__((always_inline)) { *reinterpret_cast<f32x4*>(sPart + ((w * 9 + idx) * 64 + l) * 4) = x; };
-        part(0, dAqk);
+        f32x4* const tiles[9] = {&dAqk, &dAqb[0], &dAqb[1], &dAak[0], &dAak[1], &dAab[0][0], &dAab[0][1], &dAab[1][0], &dAab[1][1]};
+        float* const slot = sPart + (w % (NW / 2)) * 9 * 256;
+        if (w >= NW / 2) {
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            part(1 + s, dAqb[s]);
-            part(3 + s, dAak[s]);
-            part(5 + s, dAab[0][s]);
-            part(7 + s, dAab[1][s]);
+            for (int i = 0; i < 9; ++i) *reinterpret_cast<f32x4*>(slot + (i * 64 + l) * 4) = *tiles[i];
+        }
+        __syncthreads();                                       // (2a)
+        if (w < NW / 2) {
+#pragma unroll
+            for (int i = 0; i < 9; ++i) {
+                f32x4* const q = reinterpret_cast<f32x4*>(slot + (i * 64 + l) * 4);
+                *q = *q + *tiles[i];
+            }
         }
     }
-    if (!EARLY) { own_kt_tiles(DHC, dhk); own_vt_tiles(DHC, dhv); }
-    __syncthreads();                                           // (2) the parts of the nine tiles are complete
+    __syncthreads();                                           // (2b) the parts of the nine tiles are complete
     // the waves share out the nine tiles: sum of the parts, causal mask, both orientations as fragments
 #pragma unroll
     for (int t = 0; t < (9 + NW - 1) / NW; ++t) {
@@ -318,7 +325,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
         if (idx < 9) {
             f32x4 x = zero4();
 #pragma unroll
-            for (int ww = 0; ww < NW; ++ww) x += *reinterpret_cast<const f32x4*>(sPart + ((ww * 9 + idx) * 64 + l) * 4);
+            for (int ww = 0; ww < NW / 2; ++ww) x += *reinterpret_cast<const f32x4*>(sPart + ((ww * 9 + idx) * 64 + l) * 4);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {      // row i = c, inner j = 4g+i; A_qk and A_qb keep the diagonal
                 const int jj = 4 * g + i;
