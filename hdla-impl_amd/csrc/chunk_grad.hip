@@ -14,10 +14,10 @@
 //
 // Division of the work: every product here contracts over channels or over value columns, so wave w owns the
 // channel tiles kt = w*KT/4 .. and the value tiles vt = w*VT/4 ..; what is summed over the other dimension (the
-// score tiles, their gradients, dv) is exchanged through LDS, with four workgroup barriers in all.  One wave per
+// score tiles, their gradients, dv) is exchanged through LDS, with five workgroup barriers in all.  One wave per
 // chunk would hold the whole chunk in registers, at one wave per SIMD, and nothing would overlap its arithmetic
-// with the memory round trips of its neighbours; four waves on a quarter each leave room for two workgroups per
-// compute unit.
+// with the memory round trips of its neighbours; four waves on a quarter each leave room for two or three
+// workgroups per compute unit.
 #include "hdla_common.cuh"
 #include "hdla_launch.h"
 
