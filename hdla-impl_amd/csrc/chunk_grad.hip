@@ -110,9 +110,15 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((sizeof
         rk[j] = ld_frag_sel(at(p.k + qb, qo + ko * ES), rowok);
         ra[0][j] = ld_frag_sel(at(p.a + ab, ao0 + ko * ES), rowok);
         ra[1][j] = ld_frag_sel(at(p.a + ab, ao1 + ko * ES), rowok);
-        rb[0][j] = ld_frag_sel(at(p.b + ab, ao0 + ko * ES), rowok);
-        rb[1][j] = ld_frag_sel(at(p.b + ab, ao1 + ko * ES), rowok);
     }
+    auto load_b = [&]() __attribute__((always_inline)) {       // b is used in the second pass only
+#pragma unroll
+        for (int j = 0; j < KTW; ++j) {
+            const uint32_t ko = 16 * (kt0 + j);
+            rb[0][j] = ld_frag_sel(at(p.b + ab, ao0 + ko * ES), rowok);
+            rb[1][j] = ld_frag_sel(at(p.b + ab, ao1 + ko * ES), rowok);
+        }
+    };
     // rows of do and v: 16 bytes a lane, the waves take turns
     constexpr int EPL = 16 / (int)sizeof(T), LPR = V / EPL, RPI = 64 / LPR, NRI = 2 * CH / RPI;   // elements/lane, lanes/row, rows/instr
     static_assert(NRI % NW == 0, "");
@@ -130,6 +136,12 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((sizeof
             if (KTW == 2) ld_pair(X + (w * VT + vt) * PAIR, dst[0][vt], dst[KTW - 1][vt]);
             else dst[0][vt] = ld_pair_one(X + ((w >> 1) * VT + vt) * PAIR, w & 1);
         }
+    };
+    // one of the own channel tiles only (the large shapes request the second one when the first has been used)
+    auto own_kt_tile = [&](const T* X, Frag<T> (&dst)[VT], int j) __attribute__((always_inline)) {
+#pragma unroll
+        for (int vt = 0; vt < VT; ++vt)
+            dst[vt] = KTW == 2 ? ld_pair_one(X + (w * VT + vt) * PAIR, j) : ld_pair_one(X + ((w >> 1) * VT + vt) * PAIR, w & 1);
     };
     auto own_vt_tiles = [&](const T* X, Frag<T> (&dst)[VTW][KT]) __attribute__((always_inline)) {
 #pragma unroll
@@ -163,7 +175,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((sizeof
     Frag<T> tmT[2][2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) ld_pair(p.ws.TM + chw * 1024 + s * PAIR, tmT[s][0], tmT[s][1]);
-    if (EARLY) { own_kt_tiles(DHC, dhk); own_vt_tiles(DHC, dhv); }
+    if (EARLY) { own_kt_tiles(DHC, dhk); own_vt_tiles(DHC, dhv); load_b(); }
 
     const Frag<T> ident = ident_frag<T>();
 
@@ -300,7 +312,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((sizeof
     // tile indices: 0 A_qk, 1+s A_qb^s, 3+s A_ak^s, 5+2r+s A_ab^{r s}
     // Sum over the waves in two rounds (half the LDS of one round): the upper half of the waves leave their parts,
     // the lower half add them to their own and leave the sums.
-    if (!EARLY) { own_kt_tiles(DHC, dhk); own_vt_tiles(DHC, dhv); }
+    if (!EARLY) { own_kt_tile(DHC, dhk[0], 0); own_vt_tiles(DHC, dhv); load_b(); }
     {
         f32x4* const tiles[9] = {&dAqk, &dAqb[0], &dAqb[1], &dAak[0], &dAak[1], &dAab[0][0], &dAab[0][1], &dAab[1][0], &dAab[1][1]};
         float* const slot = sPart + (w % (NW / 2)) * 9 * 256;
@@ -376,6 +388,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((sizeof
             const f32x4 s4 = to_f32(Sf[j][vt]), d4 = to_f32(dSf);
             hh += s4[0] * d4[0] + s4[1] * d4[1] + s4[2] * d4[2] + s4[3] * d4[3];
         }
+        if (!EARLY && KTW == 2 && j == 0) own_kt_tile(DHC, dhk[KTW - 1], 1);
         hh += __shfl_xor(hh, 16);
         hh += __shfl_xor(hh, 32);
         f32x4 hh4;
@@ -390,9 +403,12 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((sizeof
         const f32x4 q4 = to_f32(rq[j]);
         const f32x4 a4[2] = {to_f32(ra[0][j]), to_f32(ra[1][j])};
         const f32x4 b4[2] = {to_f32(rb[0][j]), to_f32(rb[1][j])};
-        const Frag<T> qhT = transpose(to_frag<T>(q4 * eq * scale), ident), khT = transpose(to_frag<T>(k4 * ek), ident);
-        const Frag<T> ahT[2] = {transpose(to_frag<T>(a4[0] * ea), ident), transpose(to_frag<T>(a4[1] * ea), ident)};
-        const Frag<T> bhT[2] = {transpose(to_frag<T>(b4[0] * ek), ident), transpose(to_frag<T>(b4[1] * ek), ident)};
+        const Frag<T> qh = to_frag<T>(q4 * eq * scale), kh = to_frag<T>(k4 * ek);
+        const Frag<T> ah[2] = {to_frag<T>(a4[0] * ea), to_frag<T>(a4[1] * ea)};
+        const Frag<T> bh[2] = {to_frag<T>(b4[0] * ek), to_frag<T>(b4[1] * ek)};
+        const Frag<T> qhT = transpose(qh, ident), khT = transpose(kh, ident);
+        const Frag<T> ahT[2] = {transpose(ah[0], ident), transpose(ah[1], ident)};
+        const Frag<T> bhT[2] = {transpose(bh[0], ident), transpose(bh[1], ident)};
         const f32x4 bg4[2] = {b4[0] * edn, b4[1] * edn};
         f32x4 dqh = mm(fin(0), khT, zero4());
         dqh = mm(fin(1), bhT[0], dqh);
@@ -416,9 +432,16 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((sizeof
         const f32x4 dk = dkh * ek + dkg * edn;
         const f32x4 da[2] = {dah[0] * ea + dag[j][0] * ege, dah[1] * ea + dag[j][1] * ege};
         const f32x4 db[2] = {dbh[0] * ek + dbg[0] * edn, dbh[1] * ek + dbg[1] * edn};
-        const f32x4 Dge = da[0] * a4[0] + da[1] * a4[1];
-        const f32x4 Dgi = dq * q4 - dk * k4 - db[0] * b4[0] - db[1] * b4[1];
-        const f32x4 dgl = exp4<T>(gl) * hh4 + sum16(dkg * kg4 + dbg[0] * bg4[0] + dbg[1] * bg4[1]);
+        // The gradient of the log-decay sums, over token pairs (i, j) of the chunk, score-gradient times score with
+        // opposite signs on the two tokens (Dgi: dependence through the inclusive decay sums, Dge: through the
+        // exclusive ones); in the suffix sum below all pairs on one side of a token cancel, and they only do so if
+        // both occurrences are the same number: the score part of each term therefore multiplies the factorised
+        // operand as the products above saw it (rounded to the element type), not its exact value.
+        const f32x4 st = dkg * kg4 + dbg[0] * bg4[0] + dbg[1] * bg4[1];      // the state-path part of k and b
+        const f32x4 Dge = dah[0] * to_f32(ah[0]) + dah[1] * to_f32(ah[1]) + (dag[j][0] * a4[0] + dag[j][1] * a4[1]) * ege;
+        const f32x4 Dgi = dqh * to_f32(qh) + dqg * (q4 * egi * scale) - dkh * to_f32(kh)
+                          - dbh[0] * to_f32(bh[0]) - dbh[1] * to_f32(bh[1]) - st;
+        const f32x4 dgl = exp4<T>(gl) * hh4 + sum16(st);
         const f32x4 dg = rscan16_incl(Dgi + Dge) - Dge + dgl;
         if (STAGE_OUT) {
             put(0, kt, to_frag<T>(dq));
@@ -438,6 +461,8 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((sizeof
             st_frag(at(p.db + ab, ao1 + 16 * kt * ES), to_frag<T>(db[1]));
             st_gk4<GKF32>(dgkp + go + 16 * kt * GS, 0, dg);
         }
+        // the large shapes are at the limit of the register file: keep the two channel tiles from being interleaved
+        if (!EARLY) __builtin_amdgcn_sched_barrier(0);
     }
     if (STAGE_OUT) {
         __syncthreads();                                       // (4) the staged rows are complete
