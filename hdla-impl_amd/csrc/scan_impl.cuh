@@ -28,8 +28,10 @@
 //  * for 2-byte inputs, four "memory waves" per workgroup do nothing but move data: they hold the register ring
 //    of block shares (6 chunks in flight), hand them to LDS, and copy the results, which the computing waves
 //    leave in an LDS outbox laid out like the chunk's record in global memory, out to global memory a step later.
-//    The computing waves then touch global memory only for their own two small tiles per chunk.  Without memory
-//    waves (fp32 inputs, or eight computing waves) the computing waves do all of that themselves.
+//    The computing waves then touch global memory only for the few tiles that are theirs alone (rows of do in the
+//    reverse scan; tiles of u^T and v^T in the forward scans, and for K = 64 these too travel through LDS with the
+//    block).  Without memory waves (fp32 inputs, or eight computing waves) the computing waves do all of that
+//    themselves.
 #pragma once
 #include "hdla_common.cuh"
 #include "scan_shapes.h"
@@ -53,6 +55,11 @@ template <typename T, int K, int V, int NWC> struct ScanCfg {
     static constexpr int NM = (sizeof(T) == 2 && NWC <= 4) ? 4 : 0;   // memory waves
     static constexpr int THREADS = 64 * (NWC + NM);
     static constexpr int NLD = NM ? NM : NWC;             // waves that split the loading of a block
+    // forward scans with memory waves (rows of 128 bytes: the larger ones have no registers to spare): the tiles of
+    // u^T and v^T of the workgroup's column blocks travel through LDS with the shared block (appended to it), so
+    // that the computing waves issue no global loads at all
+    static constexpr int OWN_UT = (NM && KB <= 128) ? NWC * PAIR * (int)sizeof(T) : 0, OWN_VTT = (NM && KB <= 128) ? NWC * TILE * (int)sizeof(T) : 0;
+    static constexpr int OWN_FWD = (OWN_UT + OWN_VTT + 1023) & ~1023;
     // Depth of the register ring of block shares (chunks in flight from global memory) and of the computing
     // waves' own tiles; multiples of the number of slots so that slot numbers are static in the unrolled loops;
     // 0: no ring, one chunk at a time.
@@ -77,6 +84,17 @@ template <int ES> __device__ __forceinline__ int piece_off(int i, int l, bool ti
 struct BlockOne {
     const char* p;
     __device__ __forceinline__ const char* piece(int i, int l, bool) const { return p + i * 1024 + l * 16; }
+};
+// forward scan with memory waves: the block, then the workgroup's tiles of u^T, then those of v^T (the last piece may
+// reach past them: those lanes read inside the tiles again, what they leave in LDS is never looked at)
+template <int NIB, int UTB, int VTB> struct BlockFwd {
+    const char *b, *ut, *vtt;
+    __device__ __forceinline__ const char* piece(int i, int l, bool) const {
+        if (i < NIB) return b + i * 1024 + l * 16;
+        const int off = (i - NIB) * 1024 + l * 16;
+        if (off < UTB) return ut + off;
+        return vtt + (off - UTB) % VTB;
+    }
 };
 // reverse scan: W and BGT (NIF pieces) and the piece holding EGL come from the forward-scan block of the (chunk,
 // head), the rest is the reverse-scan block
@@ -195,7 +213,8 @@ __device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem,
     constexpr BlkF B = blk_fwd(K, sizeof(T), WRITE_O);
     constexpr bool PIPE = C::pipelined(WRITE_O);
     constexpr bool PIPE_UPD = PIPE && C::early_update_reads(WRITE_O);
-    constexpr int NI = B.SIZE / 1024, SLOT = B.SIZE;
+    constexpr int NIB = B.SIZE / 1024, SLOT = B.SIZE + C::OWN_FWD, NI = SLOT / 1024;
+    constexpr bool OWN_LDS = C::OWN_FWD > 0;
     typedef ScanLds<T, K, V, NWC, SLOT, WRITE_O ? OUT_O : OUT_STATE> L;
     constexpr int OROW = L::OROW, OB_HC = L::OB_HC, OB = L::OB;
     char* const outbox = smem + NSLOT * SLOT;
@@ -214,7 +233,13 @@ __device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem,
     // block of step t; steps past the end of the sequence are clamped, so every load is unconditional (a load
     // that may or may not have been issued would make the compiler wait for all outstanding loads)
     auto blk = [&](int t) __attribute__((always_inline)) {
-        return BlockOne{reinterpret_cast<const char*>(p.ws.W) + (chw0 + min(c0 + t, last)) * SLOT};
+        const int64_t chw = chw0 + min(c0 + t, last);
+        const char* b = reinterpret_cast<const char*>(p.ws.W) + chw * B.SIZE;
+        if constexpr (OWN_LDS)
+            return BlockFwd<NIB, C::OWN_UT, C::OWN_VTT>{b, reinterpret_cast<const char*>(p.ws.UT + (chw * VT + vt0) * PAIR),
+                                                        reinterpret_cast<const char*>(p.ws.VTT + (chw * VT + vt0) * TILE)};
+        else
+            return BlockOne{b};
     };
 
     if (NM && wv >= NWC) {
@@ -264,11 +289,13 @@ __device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem,
 #pragma unroll
             for (int i = 0; i < 4; ++i) S[kt][i] = p.h0[soff + (int64_t)(16 * kt + 4 * g + i) * V];
     }
-    struct Own { Frag<T> ut[2], vtt; };                   // the tiles only this wave reads
+    struct Own { Frag<T> ut[2], vtt; };                   // the tiles only this wave reads (from LDS where they travel with the block)
     auto load_own = [&](Own& o, int t) __attribute__((always_inline)) {
-        const int64_t chw = chw0 + min(c0 + t, last);
-        ld_pair(p.ws.UT + (chw * VT + vt) * PAIR, o.ut[0], o.ut[1]);
-        o.vtt = ld_tile(p.ws.VTT + (chw * VT + vt) * TILE);
+        if constexpr (!OWN_LDS) {
+            const int64_t chw = chw0 + min(c0 + t, last);
+            ld_pair(p.ws.UT + (chw * VT + vt) * PAIR, o.ut[0], o.ut[1]);
+            o.vtt = ld_tile(p.ws.VTT + (chw * VT + vt) * TILE);
+        }
     };
 
     Frag<T> w[2][KT];                                     // phase-1 operands; when pipelined, read a step ahead
@@ -289,6 +316,10 @@ __device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem,
         const int64_t chw = chw0 + cid;
         const int64_t tok0 = bos + (int64_t)t * CH;
         const int len = (int)min((int64_t)CH, eos - tok0);
+        if constexpr (OWN_LDS) {
+            ld_pair(reinterpret_cast<const T*>(slot + B.SIZE) + wv * PAIR, own.ut[0], own.ut[1]);
+            own.vtt = ld_tile(reinterpret_cast<const T*>(slot + B.SIZE + C::OWN_UT) + wv * TILE);
+        }
         const T* sBGT = reinterpret_cast<const T*>(slot + B.BGT);
         const T* sKGT = reinterpret_cast<const T*>(slot + B.KGT);
         const float* sEGL = reinterpret_cast<const float*>(slot + B.EGL);
@@ -675,7 +706,7 @@ __device__ __forceinline__ void scan_bwd_body(const ChunkArgs<T>& p, char* smem,
 // grid = (H, N, directions * SPLIT); blockIdx.z = direction * SPLIT + split
 template <typename T, int K, int V, int NWC, bool WRITE_O>
 __global__ __launch_bounds__((ScanCfg<T, K, V, NWC>::THREADS)) void scan_fwd_kernel(ChunkArgs<T> p) {
-    __shared__ __attribute__((aligned(16))) char smem[ScanLds<T, K, V, NWC, blk_fwd(K, sizeof(T), WRITE_O).SIZE, WRITE_O ? OUT_O : OUT_STATE>::BYTES];
+    __shared__ __attribute__((aligned(16))) char smem[ScanLds<T, K, V, NWC, blk_fwd(K, sizeof(T), WRITE_O).SIZE + ScanCfg<T, K, V, NWC>::OWN_FWD, WRITE_O ? OUT_O : OUT_STATE>::BYTES];
     scan_fwd_body<T, K, V, NWC, WRITE_O>(p, smem, blockIdx.z);
 }
 template <typename T, int K, int V, int NWC>
@@ -686,7 +717,7 @@ __global__ __launch_bounds__((ScanCfg<T, K, V, NWC>::THREADS)) void scan_bwd_ker
 // Both scans of the backward pass in one launch: they depend on the prep kernel only, not on each other.
 template <typename T, int K, int V, int NWC>
 __global__ __launch_bounds__((ScanCfg<T, K, V, NWC>::THREADS)) void scan_pair_kernel(ChunkArgs<T> p) {
-    constexpr int NF = ScanLds<T, K, V, NWC, blk_fwd(K, sizeof(T), false).SIZE, OUT_STATE>::BYTES;
+    constexpr int NF = ScanLds<T, K, V, NWC, blk_fwd(K, sizeof(T), false).SIZE + ScanCfg<T, K, V, NWC>::OWN_FWD, OUT_STATE>::BYTES;
     constexpr int NB = ScanLds<T, K, V, NWC, slot_bwd(K, sizeof(T)).SIZE, OUT_GRAD>::BYTES;
     constexpr int SPLIT = ScanCfg<T, K, V, NWC>::SPLIT;
     __shared__ __attribute__((aligned(16))) char smem[NF > NB ? NF : NB];
