@@ -98,7 +98,8 @@ template <typename T>
 int run_chunk(const hdla_dims* d, int pass, const void* q, const void* k, const void* v, const void* a_,
               const void* b, const void* gk, const float* h0, void* o, float* ht, const void* d_o,
               const float* dht, void* dq, void* dk, void* dv, void* da, void* db, void* dgk, float* dh0,
-              void* workspace, size_t workspace_bytes, hipStream_t stream, int stages = HDLA_STAGE_ALL) {
+              void* workspace, size_t workspace_bytes, hipStream_t stream, int stages = HDLA_STAGE_ALL,
+              const void* beta = nullptr, void* dbeta = nullptr) {
     WsLayout L;
     int nch = 0;
     int rc = make_layout(d, pass, L, nch);
@@ -113,6 +114,7 @@ int run_chunk(const hdla_dims* d, int pass, const void* q, const void* k, const 
     a.dout = static_cast<const T*>(d_o); a.dht = dht; a.dh0 = dh0;
     a.dq = static_cast<T*>(dq); a.dk = static_cast<T*>(dk); a.dv = static_cast<T*>(dv);
     a.da = static_cast<T*>(da); a.db = static_cast<T*>(db); a.dgk = dgk;
+    a.beta = static_cast<const T*>(beta); a.dbeta = static_cast<T*>(dbeta);
     bind_ws(a, d, L, nch, workspace);
 #ifdef HDLA_PHASE_TIMING
     a.phase_clk = g_phase_clk;
@@ -229,6 +231,43 @@ int hdla_chunk_bwd(const hdla_dims* dims, const void* q, const void* k, const vo
                                dh0, workspace, workspace_bytes, s);
     return run_chunk<float>(dims, 1, q, k, v, a, b, gk, h0, nullptr, nullptr, d_o, dht, dq, dk, dv, da, db, dgk,
                             dh0, workspace, workspace_bytes, s);
+}
+
+int hdla_param_chunk_fwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* beta,
+                         const void* gk, const float* h0, void* o, float* ht,
+                         void* workspace, size_t workspace_bytes, void* stream) {
+    const int rc = check_dims(dims);
+    if (rc) return rc;
+    if (!beta || (dims->T > 0 && (!q || !k || !v || !gk || !o))) return HDLA_ERR_NULL;
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(gk) || !aligned16(o) || !aligned16(h0) ||
+        !aligned16(ht)) return HDLA_ERR_ALIGN;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dims->in_dtype == HDLA_BF16)
+        return run_chunk<bf16>(dims, 0, q, k, v, nullptr, nullptr, gk, h0, o, ht, nullptr, nullptr, nullptr, nullptr,
+                               nullptr, nullptr, nullptr, nullptr, nullptr, workspace, workspace_bytes, s,
+                               HDLA_STAGE_ALL, beta, nullptr);
+    return run_chunk<float>(dims, 0, q, k, v, nullptr, nullptr, gk, h0, o, ht, nullptr, nullptr, nullptr, nullptr,
+                            nullptr, nullptr, nullptr, nullptr, nullptr, workspace, workspace_bytes, s,
+                            HDLA_STAGE_ALL, beta, nullptr);
+}
+
+int hdla_param_chunk_bwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* beta,
+                         const void* gk, const float* h0, const void* d_o, const float* dht,
+                         void* dq, void* dk, void* dv, void* dbeta, void* dgk, float* dh0,
+                         void* workspace, size_t workspace_bytes, void* stream) {
+    const int rc = check_dims(dims);
+    if (rc) return rc;
+    if (!beta || (dims->T > 0 && (!q || !k || !v || !gk || !d_o || !dq || !dk || !dv || !dbeta || !dgk)))
+        return HDLA_ERR_NULL;
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(gk) || !aligned16(d_o) || !aligned16(dq) ||
+        !aligned16(dk) || !aligned16(dv) || !aligned16(dgk) || !aligned16(h0) || !aligned16(dht) || !aligned16(dh0))
+        return HDLA_ERR_ALIGN;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dims->in_dtype == HDLA_BF16)
+        return run_chunk<bf16>(dims, 1, q, k, v, nullptr, nullptr, gk, h0, nullptr, nullptr, d_o, dht, dq, dk, dv,
+                               nullptr, nullptr, dgk, dh0, workspace, workspace_bytes, s, HDLA_STAGE_ALL, beta, dbeta);
+    return run_chunk<float>(dims, 1, q, k, v, nullptr, nullptr, gk, h0, nullptr, nullptr, d_o, dht, dq, dk, dv,
+                            nullptr, nullptr, dgk, dh0, workspace, workspace_bytes, s, HDLA_STAGE_ALL, beta, dbeta);
 }
 
 int hdla_chunk_stages(const hdla_dims* dims, int pass, int stages, const void* q, const void* k, const void* v,

@@ -45,12 +45,24 @@ template <typename T, int K, int V> struct CgLds {
     static constexpr bool STAGE_OUT = ES == 2;
     static constexpr int OPK = K * ES + 16, OPV = V * ES + 16;       // padded rows
     static constexpr int PART_B = (NW / 2) * 9 * 1024, OUT_B = STAGE_OUT ? (7 * OPK + OPV) * CH : 0;
-    static constexpr int R1 = KG + KG_B, R1_B = PART_B > OUT_B ? PART_B : OUT_B;
+    // per wave and token: three partial sums over channels of the backward of the HDLA parameterisation
+    static constexpr int RED = KG + KG_B, RED_B = NW * 3 * CH * 4;
+    static constexpr int R1 = RED + RED_B, R1_B = PART_B > OUT_B ? PART_B : OUT_B;
     static constexpr int BYTES = R1 + R1_B;
 };
 
-template <typename T, bool GKF32, int K, int V>
-__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((sizeof(T) * K * V <= 2 * 64 * 64) ? 3 : sizeof(T) == 2 ? 2 : 1, (sizeof(T) * K * V <= 2 * 64 * 64) ? 3 : 2))) void chunk_grad_kernel(ChunkArgs<T> p) {
+// waves per SIMD asked of the compiler (lowest, highest): three workgroups per compute unit for the smallest 2-byte
+// shape, two for the other 2-byte shapes; the variant with the HDLA parameterisation carries its backward's
+// partial results across one more barrier and gets one step less
+template <typename T, int K, int V, bool HD> constexpr int cg_waves(bool highest) {
+    const bool small = sizeof(T) * K * V <= 2 * 64 * 64;
+    if (sizeof(T) != 2) return highest ? 2 : 1;
+    if (HD) return small ? 2 : (highest ? 2 : 1);
+    return small ? 3 : 2;
+}
+
+template <typename T, bool GKF32, int K, int V, bool HD>
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(cg_waves<T, K, V, HD>(false), cg_waves<T, K, V, HD>(true)))) void chunk_grad_kernel(ChunkArgs<T> p) {
     constexpr int KT = K / 16, VT = V / 16, KT2 = KT / 2, KTW = KT / NW, VTW = VT / NW;
     static_assert(KT % NW == 0 && VT % NW == 0 && (KTW == 1 || KTW == 2), "a wave owns one channel tile or one stored pair");
     typedef CgLds<T, K, V> L;
@@ -62,6 +74,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((sizeof
     float* const sScore = reinterpret_cast<float*>(smem + L::SCORE);
     T* const sKg = reinterpret_cast<T*>(smem + L::KG);
     T* const sFin = reinterpret_cast<T*>(smem + L::FIN);
+    float* const sRed = reinterpret_cast<float*>(smem + L::RED);
     float* const sPart = reinterpret_cast<float*>(smem + L::R1);
     char* const sOut = smem + L::R1;
 
@@ -108,10 +121,13 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((sizeof
         rg[j] = ld_gk4<GKF32>(gkp + go + ko * GS, 0, rowok);
         rq[j] = ld_frag_sel(at(p.q + qb, qo + ko * ES), rowok);
         rk[j] = ld_frag_sel(at(p.k + qb, qo + ko * ES), rowok);
-        ra[0][j] = ld_frag_sel(at(p.a + ab, ao0 + ko * ES), rowok);
-        ra[1][j] = ld_frag_sel(at(p.a + ab, ao1 + ko * ES), rowok);
+        if (!HD) {
+            ra[0][j] = ld_frag_sel(at(p.a + ab, ao0 + ko * ES), rowok);
+            ra[1][j] = ld_frag_sel(at(p.a + ab, ao1 + ko * ES), rowok);
+        }
     }
     auto load_b = [&]() __attribute__((always_inline)) {       // b is used in the second pass only
+        if (HD) return;
 #pragma unroll
         for (int j = 0; j < KTW; ++j) {
             const uint32_t ko = 16 * (kt0 + j);
@@ -177,6 +193,30 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((sizeof
     for (int s = 0; s < 2; ++s) ld_pair(p.ws.TM + chw * 1024 + s * PAIR, tmT[s][0], tmT[s][1]);
     if (EARLY) { own_kt_tiles(DHC, dhk); own_vt_tiles(DHC, dhv); load_b(); }
 
+    // HDLA parameterisation (hdla_custom.py:19-43): a_1 = -beta k, a_2 = beta k (beta s - f), b_1 = f k, b_2 = k with
+    // f = exp(gk) and s = sum over ALL channels of k^2 f (every wave reads all of k and gk of the chunk for it), rounded
+    // to the element type as the layer's .to(dtype) does, so that everything below sees what the plain operator sees
+    float beta_t = 0.f, s_t = 0.f;
+    if (HD) {
+        beta_t = rowok ? ld_elem(p.beta + (cp.tok0 + row) * H + h) : 0.f;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            const f32x4 g4 = ld_gk4<GKF32>(gkp + go + 16 * kt * GS, 0, rowok);
+            const f32x4 k4 = to_f32(ld_frag_sel(at(p.k + qb, qo + 16 * kt * ES), rowok));
+            const f32x4 kf = k4 * k4 * exp4<T>(g4);
+            s_t += kf[0] + kf[1] + kf[2] + kf[3];
+        }
+        s_t += __shfl_xor(s_t, 16);
+        s_t += __shfl_xor(s_t, 32);
+#pragma unroll
+        for (int j = 0; j < KTW; ++j) {
+            const f32x4 kk = to_f32(rk[j]), f4 = exp4<T>(rg[j]);
+            ra[0][j] = to_frag<T>(kk * (-beta_t));
+            ra[1][j] = to_frag<T>(kk * ((beta_t * s_t - f4) * beta_t));
+            rb[0][j] = to_frag<T>(f4 * kk);
+            rb[1][j] = rk[j];
+        }
+    }
     const Frag<T> ident = ident_frag<T>();
 
     // ---- own channel tiles: part of A_qk^T and A_ak^T (rows j, inner i); kg for everybody ------------------------
@@ -366,6 +406,8 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((sizeof
         else if (rowok) st_frag(at(p.dv + vb, vo + 16 * (vt0 + j) * ES), to_frag<T>(x));
     }
     // ---- own channel tiles, second pass: state products, score backward, final gradients ---------------------------
+    f32x4 dk_pre[HD ? KTW : 1], dg_pre[HD ? KTW : 1];
+    float red[3] = {0.f, 0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < KTW; ++j) {
         const int kt = kt0 + j;
@@ -443,7 +485,19 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((sizeof
                           - dbh[0] * to_f32(bh[0]) - dbh[1] * to_f32(bh[1]) - st;
         const f32x4 dgl = exp4<T>(gl) * hh4 + sum16(st);
         const f32x4 dg = rscan16_incl(Dgi + Dge) - Dge + dgl;
-        if (STAGE_OUT) {
+        if (HD) {
+            // backward of the parameterisation, the part that needs no sum over channels; what does (through s, and
+            // dbeta itself) waits for the sums r1 = sum k da_1, r2 = sum k da_2, r3 = sum k f da_2 of all the waves
+            const f32x4 f4 = exp4<T>(g4);
+            dk_pre[j] = dk - da[0] * beta_t + da[1] * ((beta_t * s_t - f4) * beta_t) + db[0] * f4 + db[1];
+            dg_pre[j] = dg + (db[0] - da[1] * beta_t) * k4 * f4;
+            const f32x4 t1 = k4 * da[0], t2 = k4 * da[1], t3 = t2 * f4;
+            red[0] += t1[0] + t1[1] + t1[2] + t1[3];
+            red[1] += t2[0] + t2[1] + t2[2] + t2[3];
+            red[2] += t3[0] + t3[1] + t3[2] + t3[3];
+            if (STAGE_OUT) put(0, kt, to_frag<T>(dq));
+            else if (rowok) st_frag(at(p.dq + qb, qo + 16 * kt * ES), to_frag<T>(dq));
+        } else if (STAGE_OUT) {
             put(0, kt, to_frag<T>(dq));
             put(1, kt, to_frag<T>(dk));
             put(2, kt, to_frag<T>(da[0]));
@@ -464,18 +518,56 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((sizeof
         // the large shapes are at the limit of the register file: keep the two channel tiles from being interleaved
         if (!EARLY) __builtin_amdgcn_sched_barrier(0);
     }
+    if (HD) {
+        // sums over all channels, per token: within the wave over the four lane groups, then over the waves through LDS
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            red[i] += __shfl_xor(red[i], 16);
+            red[i] += __shfl_xor(red[i], 32);
+            if (g == 0) sRed[(w * 3 + i) * CH + c] = red[i];
+        }
+        __syncthreads();                                       // (3b) the sums of all waves are there
+        float r1 = 0.f, r2 = 0.f, r3 = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < NW; ++ww) {
+            r1 += sRed[(ww * 3 + 0) * CH + c];
+            r2 += sRed[(ww * 3 + 1) * CH + c];
+            r3 += sRed[(ww * 3 + 2) * CH + c];
+        }
+        // a_2 depends on every channel through s: ds = beta^2 r2, and s = sum k^2 f
+        const float ds = beta_t * beta_t * r2;
+#pragma unroll
+        for (int j = 0; j < KTW; ++j) {
+            const int kt = kt0 + j;
+            const f32x4 k4 = to_f32(rk[j]), kf = k4 * exp4<T>(rg[j]);
+            const f32x4 dk = dk_pre[j] + kf * (2.f * ds);
+            const f32x4 dg = dg_pre[j] + kf * k4 * ds;
+            if (STAGE_OUT) {
+                put(1, kt, to_frag<T>(dk));
+                if (!GKF32) put(6, kt, to_frag<T>(dg));
+                else if (rowok) st_gk4<GKF32>(dgkp + go + 16 * kt * GS, 0, dg);
+            } else if (rowok) {
+                st_frag(at(p.dk + qb, qo + 16 * kt * ES), to_frag<T>(dk));
+                st_gk4<GKF32>(dgkp + go + 16 * kt * GS, 0, dg);
+            }
+        }
+        // dbeta = sum_c da_1 (-k) + da_2 k (2 beta s - f)
+        if (w == 0 && g == 0 && rowok) st_elem(p.dbeta + (cp.tok0 + c) * H + h, -r1 + 2.f * beta_t * s_t * r2 - r3);
+    }
     if (STAGE_OUT) {
         __syncthreads();                                       // (4) the staged rows are complete
         // whole rows, 16 bytes a lane; the waves take turns over the instructions
         constexpr int LRK = K * (int)ES / 16, RPK = 64 / LRK, NUK = CH / RPK;   // lanes per row, rows per instruction, instructions per tensor
         constexpr int LRV = V * (int)ES / 16, RPV = 64 / LRV, NUV = CH / RPV;
-        constexpr int NKT = GKF32 ? 6 : 7, NU = NKT * NUK + NUV;
+        // gradients that leave through the staged rows: dq, dk, da (2), db (2), dgk; with the HDLA parameterisation
+        // dq, dk, dgk; dgk goes out directly when it is fp32 next to 2-byte inputs
+        constexpr int NKT = HD ? (GKF32 ? 2 : 3) : (GKF32 ? 6 : 7), NU = NKT * NUK + NUV;
         const uint32_t qpitch = (uint32_t)(H * K) * ES, apitch = qpitch * RANK;
 #pragma unroll
         for (int t = 0; t < (NU + NW - 1) / NW; ++t) {
             const int u = w + t * NW;
             if (u < NKT * NUK) {
-                const int m = u / NUK, r = (u % NUK) * RPK + l / LRK, e = (l % LRK) * 16;
+                const int mi = u / NUK, m = (HD && mi == 2) ? 6 : mi, r = (u % NUK) * RPK + l / LRK, e = (l % LRK) * 16;
                 char* base = reinterpret_cast<char*>(m == 0 ? p.dq + qb : m == 1 ? p.dk + qb : m < 4 ? p.da + ab : m < 6 ? p.db + ab : reinterpret_cast<T*>(dgkp));
                 const uint32_t pitch = (m < 2 || m == 6) ? qpitch : apitch, off = (m == 3 || m == 5) ? qpitch : 0;
                 const i32x4 x = *reinterpret_cast<const i32x4*>(sOut + (m * CH + r) * L::OPK + e);
@@ -489,22 +581,27 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((sizeof
     }
 }
 
-template <typename T, int K, int V>
+template <typename T, int K, int V, bool HD>
 static hipError_t launch_chunk_grad_kv(const ChunkArgs<T>& a, hipStream_t stream) {
     dim3 grid(a.st.nch * a.H), block(64 * NW);
     constexpr bool kAlwaysF32 = sizeof(T) == 4;
-    if (kAlwaysF32 || a.gk_f32) hipLaunchKernelGGL((chunk_grad_kernel<T, true, K, V>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((chunk_grad_kernel<T, kAlwaysF32, K, V>), grid, block, 0, stream, a);
+    if (kAlwaysF32 || a.gk_f32) hipLaunchKernelGGL((chunk_grad_kernel<T, true, K, V, HD>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((chunk_grad_kernel<T, kAlwaysF32, K, V, HD>), grid, block, 0, stream, a);
     return hipGetLastError();
+}
+
+template <typename T, bool HD>
+static hipError_t launch_chunk_grad_hd(const ChunkArgs<T>& a, int K, int V, hipStream_t stream) {
+    if (K == 64 && V == 64) return launch_chunk_grad_kv<T, 64, 64, HD>(a, stream);
+    if (K == 128 && V == 128) return launch_chunk_grad_kv<T, 128, 128, HD>(a, stream);
+    if (K == 64 && V == 128) return launch_chunk_grad_kv<T, 64, 128, HD>(a, stream);
+    if (K == 128 && V == 64) return launch_chunk_grad_kv<T, 128, 64, HD>(a, stream);
+    return hipErrorInvalidValue;
 }
 
 template <typename T>
 hipError_t launch_chunk_grad(const ChunkArgs<T>& a, int K, int V, hipStream_t stream) {
-    if (K == 64 && V == 64) return launch_chunk_grad_kv<T, 64, 64>(a, stream);
-    if (K == 128 && V == 128) return launch_chunk_grad_kv<T, 128, 128>(a, stream);
-    if (K == 64 && V == 128) return launch_chunk_grad_kv<T, 64, 128>(a, stream);
-    if (K == 128 && V == 64) return launch_chunk_grad_kv<T, 128, 64>(a, stream);
-    return hipErrorInvalidValue;
+    return a.beta ? launch_chunk_grad_hd<T, true>(a, K, V, stream) : launch_chunk_grad_hd<T, false>(a, K, V, stream);
 }
 template hipError_t launch_chunk_grad<bf16>(const ChunkArgs<bf16>&, int, int, hipStream_t);
 template hipError_t launch_chunk_grad<float>(const ChunkArgs<float>&, int, int, hipStream_t);

@@ -102,6 +102,10 @@ struct Ws {
 template <typename T>
 struct ChunkArgs {            // inputs of the chunked operator + workspace
     const T *q, *k, *v, *a, *b;
+    // HDLA parameterisation (hdla_custom.py:19-43): when beta is given, a and b are not read but formed in the
+    // kernels from (beta, k, gk), and the backward pass returns dbeta (and folds da, db into dk, dgk) instead of da, db
+    const T* beta;            // nullable [B,T,H]
+    T* dbeta;
     const void* gk;
     int gk_f32;
     int H;

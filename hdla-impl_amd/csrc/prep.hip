@@ -17,7 +17,7 @@ namespace hdla {
 
 constexpr int LDP = 36;   // padded row length of the 32x32 LDS matrices (keeps 16-byte row alignment)
 
-template <typename T, bool GKF32, int K, int V, bool BWD>
+template <typename T, bool GKF32, int K, int V, bool BWD, bool HD>
 __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void prep_kernel(ChunkArgs<T> p) {
     constexpr int NWP = K / 64;                       // waves per (chunk, head)
     constexpr int KTW = 4, VT = V / 16, VTW = VT / NWP, KT2 = K / 32;
@@ -68,16 +68,39 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
     Frag<T> rv[VTW];
 #pragma unroll
     for (int vt = 0; vt < VTW; ++vt) rv[vt] = ld_frag_sel(p.v + voff + 16 * (vt0 + vt), rowok);
+    // HDLA parameterisation: a_1 = -beta k, a_2 = beta k (beta s - f), b_1 = f k, b_2 = k with f = exp(gk) and
+    // s = sum over ALL channels of k^2 f (a wave reads the other waves' channels of k and gk for it as well)
+    float beta_t = 0.f, s_t = 0.f;
+    if (HD) {
+        beta_t = rowok ? ld_elem(p.beta + tok * H + h) : 0.f;
+#pragma unroll
+        for (int kt = 0; kt < K / 16; ++kt) {
+            const f32x4 g4 = ld_gk4<GKF32>(p.gk, qoff + 16 * kt, rowok);
+            const f32x4 k4 = to_f32(ld_frag_sel(p.k + qoff + 16 * kt, rowok));
+            const f32x4 kf = k4 * k4 * exp4<T>(g4);
+            s_t += kf[0] + kf[1] + kf[2] + kf[3];
+        }
+        s_t += __shfl_xor(s_t, 16);
+        s_t += __shfl_xor(s_t, 32);
+    }
 #pragma unroll
     for (int kt = 0; kt < KTW; ++kt) {
         const int ko = 16 * (kt0 + kt);
         const f32x4 g4 = ld_gk4<GKF32>(p.gk, qoff + ko, rowok);
         rq[kt] = ld_frag_sel(p.q + qoff + ko, rowok);
         rk[kt] = ld_frag_sel(p.k + qoff + ko, rowok);
-        ra[0][kt] = ld_frag_sel(p.a + aoff0 + ko, rowok);
-        ra[1][kt] = ld_frag_sel(p.a + aoff1 + ko, rowok);
-        rb[0][kt] = ld_frag_sel(p.b + aoff0 + ko, rowok);
-        rb[1][kt] = ld_frag_sel(p.b + aoff1 + ko, rowok);
+        if (HD) {
+            const f32x4 kk = to_f32(rk[kt]), f4 = exp4<T>(g4);
+            ra[0][kt] = to_frag<T>(kk * (-beta_t));
+            ra[1][kt] = to_frag<T>(kk * ((beta_t * s_t - f4) * beta_t));
+            rb[0][kt] = to_frag<T>(f4 * kk);
+            rb[1][kt] = rk[kt];
+        } else {
+            ra[0][kt] = ld_frag_sel(p.a + aoff0 + ko, rowok);
+            ra[1][kt] = ld_frag_sel(p.a + aoff1 + ko, rowok);
+            rb[0][kt] = ld_frag_sel(p.b + aoff0 + ko, rowok);
+            rb[1][kt] = ld_frag_sel(p.b + aoff1 + ko, rowok);
+        }
         gi[kt] = scan16_incl(g4);
         ge[kt] = gi[kt] - g4;
         const f32x4 m = bcast16(gi[kt], MID);
@@ -268,27 +291,32 @@ __global__ void build_chunk_table_kernel(const int64_t* cu, int N, int nch, int3
     }
 }
 
-template <typename T, int K, int V>
+template <typename T, int K, int V, bool HD>
 static hipError_t launch_prep_kv(const ChunkArgs<T>& a, bool bwd, hipStream_t stream) {
     dim3 grid(a.st.nch * a.H), block(K);
     constexpr bool kAlwaysF32 = sizeof(T) == 4;
     if (kAlwaysF32 || a.gk_f32) {
-        if (bwd) hipLaunchKernelGGL((prep_kernel<T, true, K, V, true>), grid, block, 0, stream, a);
-        else hipLaunchKernelGGL((prep_kernel<T, true, K, V, false>), grid, block, 0, stream, a);
+        if (bwd) hipLaunchKernelGGL((prep_kernel<T, true, K, V, true, HD>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((prep_kernel<T, true, K, V, false, HD>), grid, block, 0, stream, a);
     } else {
-        if (bwd) hipLaunchKernelGGL((prep_kernel<T, kAlwaysF32, K, V, true>), grid, block, 0, stream, a);
-        else hipLaunchKernelGGL((prep_kernel<T, kAlwaysF32, K, V, false>), grid, block, 0, stream, a);
+        if (bwd) hipLaunchKernelGGL((prep_kernel<T, kAlwaysF32, K, V, true, HD>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((prep_kernel<T, kAlwaysF32, K, V, false, HD>), grid, block, 0, stream, a);
     }
     return hipGetLastError();
 }
 
+template <typename T, bool HD>
+static hipError_t launch_prep_hd(const ChunkArgs<T>& a, int K, int V, bool bwd, hipStream_t stream) {
+    if (K == 64 && V == 64) return launch_prep_kv<T, 64, 64, HD>(a, bwd, stream);
+    if (K == 128 && V == 128) return launch_prep_kv<T, 128, 128, HD>(a, bwd, stream);
+    if (K == 64 && V == 128) return launch_prep_kv<T, 64, 128, HD>(a, bwd, stream);
+    if (K == 128 && V == 64) return launch_prep_kv<T, 128, 64, HD>(a, bwd, stream);
+    return hipErrorInvalidValue;
+}
+
 template <typename T>
 hipError_t launch_prep(const ChunkArgs<T>& a, int K, int V, bool bwd, hipStream_t stream) {
-    if (K == 64 && V == 64) return launch_prep_kv<T, 64, 64>(a, bwd, stream);
-    if (K == 128 && V == 128) return launch_prep_kv<T, 128, 128>(a, bwd, stream);
-    if (K == 64 && V == 128) return launch_prep_kv<T, 64, 128>(a, bwd, stream);
-    if (K == 128 && V == 64) return launch_prep_kv<T, 128, 64>(a, bwd, stream);
-    return hipErrorInvalidValue;
+    return a.beta ? launch_prep_hd<T, true>(a, K, V, bwd, stream) : launch_prep_hd<T, false>(a, K, V, bwd, stream);
 }
 template hipError_t launch_prep<bf16>(const ChunkArgs<bf16>&, int, int, bool, hipStream_t);
 template hipError_t launch_prep<float>(const ChunkArgs<float>&, int, int, bool, hipStream_t);

@@ -1,8 +1,10 @@
 """hdla_hip: MI355X-native operators for HDLA's rank-2 DPLR delta-rule linear attention.
 
-Exports the two operators of the reference package (HRDPLR/__init__.py:1-12) with the same signatures.
+Exports the two operators of the reference package (HRDPLR/__init__.py:1-12) with the same signatures, and the
+operator as the HDLA layer calls it (a, b given by beta, k, log_f: HRDPLR/hdla_custom.py:19-43,290-309).
 """
 from .chunk import ChunkDPLRDeltaRuleFunction, chunk_hrdplr_delta_rule
+from .hdla import ChunkHDLAFunction, chunk_hdla_delta_rule, parameterize_a_b
 from .recurrent import FusedRecurrentDPLRDeltaRuleFunction, fused_recurrent_dplr_delta_rule
 
 __all__ = [
@@ -10,4 +12,7 @@ __all__ = [
     "chunk_hrdplr_delta_rule",
     "ChunkDPLRDeltaRuleFunction",
     "FusedRecurrentDPLRDeltaRuleFunction",
+    "chunk_hdla_delta_rule",
+    "parameterize_a_b",
+    "ChunkHDLAFunction",
 ]

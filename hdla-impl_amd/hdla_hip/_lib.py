@@ -61,6 +61,10 @@ def load():
     lib.hdla_chunk_fwd.argtypes = [F] + [P] * 9 + [P, ctypes.c_size_t, P]
     lib.hdla_chunk_bwd.restype = ctypes.c_int
     lib.hdla_chunk_bwd.argtypes = [F] + [P] * 16 + [P, ctypes.c_size_t, P]
+    lib.hdla_param_chunk_fwd.restype = ctypes.c_int
+    lib.hdla_param_chunk_fwd.argtypes = [F] + [P] * 8 + [P, ctypes.c_size_t, P]
+    lib.hdla_param_chunk_bwd.restype = ctypes.c_int
+    lib.hdla_param_chunk_bwd.argtypes = [F] + [P] * 14 + [P, ctypes.c_size_t, P]
     lib.hdla_chunk_stages.restype = ctypes.c_int
     lib.hdla_chunk_stages.argtypes = [F, ctypes.c_int, ctypes.c_int] + [P] * 18 + [P, ctypes.c_size_t, P]
     lib.hdla_calib_stream.restype = ctypes.c_int

@@ -95,6 +95,21 @@ int hdla_chunk_bwd(const hdla_dims* dims, const void* q, const void* k, const vo
                    void* dq, void* dk, void* dv, void* da, void* db, void* dgk, float* dh0,
                    void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same operator with a and b formed inside the kernels the way the HDLA layer forms them
+ * (parameterize_a_b, HRDPLR/hdla_custom.py:19-43, called at :290 right before the operator):
+ *     f = exp(gk),  s = sum_c k_c^2 f_c,   a_1 = -beta k,  a_2 = beta k (beta s - f),   b_1 = f k,  b_2 = k
+ * (identical to the reference's a_2 = a_t2 + a_t1 sum(b_t1 a_t2); the decay is (I - beta k k^T) Diag(f) (I - beta k k^T)),
+ * with a and b rounded to the input dtype as the layer's .to(dtype) does (:301-304).  beta is [B,T,H] in the input
+ * dtype.  a and b are never materialised: neither read here nor written by a caller.  The backward pass returns
+ * dbeta [B,T,H] and folds the gradients of a and b into dk and dgk. */
+int hdla_param_chunk_fwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* beta,
+                         const void* gk, const float* h0, void* o, float* ht,
+                         void* workspace, size_t workspace_bytes, void* stream);
+int hdla_param_chunk_bwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* beta,
+                         const void* gk, const float* h0, const void* d_o, const float* dht,
+                         void* dq, void* dk, void* dv, void* dbeta, void* dgk, float* dh0,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
 /* Profiling / debugging aid with no counterpart in the reference: runs only the kernels selected by `stages`
  * (a bit mask) of the forward (pass 0) or backward (pass 1) launch sequence, in order, on the same workspace, so
  * that a caller can bracket each kernel with events on `stream`.  A stage reads what the earlier stages left

@@ -19,6 +19,11 @@ Parity of the oracle itself is pinned without importing the reference (``tests/t
 closed forms (T = 1; a = b = 0 gives gated linear attention; g = 0 with one rank gives DeltaNet),
 linearity in (v, S0), chunk-size independence, chunk form == recurrence, split-sequence state hand-off,
 reverse == time flip, variable-length == per-sequence calls, and gradients by central finite differences.
+
+* :func:`parameterize_a_b` follows ``HRDPLR/hdla_custom.py:19-43`` (the build of a, b from beta, k, log_f that the
+  layer runs right before the operator, ``:290``), with the ``return`` the reference's function lacks.  It is
+  pinned by the identity its own comment states (``hdla_custom.py:270-288``): the one-step transition
+  ``Diag(f) + b_1 a_1^T + b_2 a_2^T`` equals ``(I - beta k k^T) Diag(f) (I - beta k k^T)``.
 """
 from typing import Optional, Tuple
 
@@ -149,6 +154,24 @@ def chunk_naive(
     o = torch.stack(outs, 2)                                             # [B,H,NT,C,V]
     o = o.permute(0, 2, 3, 1, 4).reshape(B, T, H, V)                     # naive.py:263
     return o, (S if output_final_state else None)
+
+
+def parameterize_a_b(beta: torch.Tensor, k: torch.Tensor, log_f: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """HRDPLR/hdla_custom.py:19-43: beta [B,T,H,1] (or [B,T,H]), k and log_f [B,T,H,K] -> a, b [B,2T,H,K]."""
+    if beta.dim() == 3:
+        beta = beta.unsqueeze(-1)
+    f = torch.exp(log_f)
+    a_t1 = -beta * k                                                   # :24
+    a_t2 = -beta * f * k                                               # :25
+    b_t1, b_t2 = k, k                                                  # :27-28
+    a_1 = a_t1                                                         # :30
+    a_2 = a_t2 + a_t1 * torch.sum(b_t1 * a_t2, dim=-1, keepdim=True)   # :31-33
+    b_1 = f * b_t1                                                     # :35
+    b_2 = b_t2                                                         # :36
+    B, T, H, K = k.shape
+    a = torch.stack([a_1, a_2], dim=2).reshape(B, 2 * T, H, K)         # :38-41: rank-minor rows
+    b = torch.stack([b_1, b_2], dim=2).reshape(B, 2 * T, H, K)
+    return a, b
 
 
 def rel_l2(x: torch.Tensor, ref: torch.Tensor) -> float:

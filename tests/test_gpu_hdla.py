@@ -1,0 +1,105 @@
+"""The operator with a and b formed inside the kernels from (beta, k, log_f) (hdla_hip.chunk_hdla_delta_rule) against
+(1) the float64 recurrence on a, b = oracle.parameterize_a_b(beta, k, log_f) with autograd through both, to the
+stated tolerances (outputs and state 5e-3, gradients 1e-2 for bf16; 1e-5 for fp32), and (2) the plain operator fed
+with the torch-built a and b, which it must reproduce almost to the bit (the kernels round a and b to the input
+type exactly as ``.to(dtype)`` does; only exp() differs in the last place)."""
+import pytest
+import torch
+
+from hdla_hip import chunk_hdla_delta_rule, chunk_hrdplr_delta_rule, parameterize_a_b
+from oracle import hrdplr_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+TOL = {torch.bfloat16: (5e-3, 1e-2), torch.float32: (1e-5, 1e-5)}
+NAMES = ["dq", "dk", "dv", "dbeta", "dlog_f", "dh0"]
+
+
+def _inputs(seed, B, T, H, K, V, N=None, gk_div=4.0):
+    g = torch.Generator().manual_seed(seed)
+    rn = lambda *s: torch.randn(*s, generator=g)
+    q = torch.nn.functional.normalize(rn(B, T, H, K), dim=-1)
+    k = torch.nn.functional.normalize(rn(B, T, H, K), dim=-1)
+    v = rn(B, T, H, V)
+    beta = 2.0 * torch.rand(B, T, H, 1, generator=g)
+    log_f = torch.nn.functional.logsigmoid(rn(B, T, H, K)) / gk_div
+    N = B if N is None else N
+    return q, k, v, beta, log_f, rn(N, H, K, V), rn(B, T, H, V), rn(N, H, K, V)
+
+
+def _oracle(inp, dtype, scale, cu=None):
+    q, k, v, beta, log_f, h0, do, dht = inp
+    leaves = [t.to(dtype).double().requires_grad_() for t in (q, k, v, beta, log_f)]
+    h0 = h0.double().requires_grad_()
+    a, b = O.parameterize_a_b(leaves[3], leaves[1], leaves[4])
+    o, ht = O.recurrence(leaves[0], leaves[1], leaves[2], a, b, leaves[4], scale, h0, cu_seqlens=cu)
+    g = torch.autograd.grad([o, ht], leaves + [h0], [do.to(dtype).double(), dht.double()])
+    return o.detach(), ht.detach(), dict(zip(NAMES, g))
+
+
+def _fused(inp, dtype, scale, cu=None):
+    q, k, v, beta, log_f, h0, do, dht = inp
+    leaves = [t.to(dtype).to(DEV).requires_grad_() for t in (q, k, v, beta, log_f)]
+    h0 = h0.to(DEV).requires_grad_()
+    o, ht = chunk_hdla_delta_rule(*leaves, scale=scale, initial_state=h0, output_final_state=True,
+                                  cu_seqlens=None if cu is None else cu.to(DEV))
+    g = torch.autograd.grad([o, ht], leaves + [h0], [do.to(dtype).to(DEV), dht.to(DEV)])
+    assert g[3].shape == leaves[3].shape and g[3].dtype == dtype
+    return o.detach(), ht.detach(), dict(zip(NAMES, g))
+
+
+def _unfused(inp, dtype, scale, cu=None):
+    q, k, v, beta, log_f, h0, do, dht = inp
+    leaves = [t.to(dtype).to(DEV).requires_grad_() for t in (q, k, v, beta, log_f)]
+    h0 = h0.to(DEV).requires_grad_()
+    a, b = parameterize_a_b(leaves[3].float(), leaves[1].float(), leaves[4].float())       # fp32, then .to(dtype)
+    o, ht = chunk_hrdplr_delta_rule(leaves[0], leaves[1], leaves[2], a.to(dtype), b.to(dtype), leaves[4], 2, scale=scale,
+                                    initial_state=h0, output_final_state=True, chunk_size=16,
+                                    cu_seqlens=None if cu is None else cu.to(DEV))
+    g = torch.autograd.grad([o, ht], leaves + [h0], [do.to(dtype).to(DEV), dht.to(DEV)])
+    return o.detach(), ht.detach(), dict(zip(NAMES, g))
+
+
+def _check(got, ref, tol_o, tol_g, what):
+    errs = {"o": O.rel_l2(got[0], ref[0]), "ht": O.rel_l2(got[1], ref[1])}
+    errs.update({n: O.rel_l2(got[2][n], ref[2][n]) for n in NAMES})
+    print(what, {k: f"{v:.2e}" for k, v in errs.items()}, flush=True)
+    assert errs["o"] <= tol_o and errs["ht"] <= tol_o, errs
+    for n in NAMES:
+        assert errs[n] <= tol_g, (n, errs)
+
+
+CASES = [
+    (torch.float32, 2, 40, 2, 64, 64, 4.0, 1.0),
+    (torch.float32, 1, 50, 2, 128, 128, 1.0, 0.5),
+    (torch.float32, 1, 33, 3, 64, 128, 16.0, 1.0),
+    (torch.bfloat16, 2, 64, 2, 64, 64, 4.0, 1.0),
+    (torch.bfloat16, 1, 100, 3, 128, 64, 1.0, 1.0),
+    (torch.bfloat16, 2, 130, 2, 64, 128, 16.0, 0.125),
+    (torch.bfloat16, 1, 256, 2, 128, 128, 16.0, 1.0),
+    (torch.bfloat16, 1, 17, 40, 64, 64, 2.0, 1.0),
+]
+
+
+@pytest.mark.parametrize("dtype,B,T,H,K,V,gk_div,scale", CASES)
+def test_against_the_recurrence(dtype, B, T, H, K, V, gk_div, scale):
+    inp = _inputs(700 + T, B, T, H, K, V, gk_div=gk_div)
+    _check(_fused(inp, dtype, scale), _oracle(inp, dtype, scale), *TOL[dtype], what=f"{dtype} B{B} T{T} H{H} K{K} V{V}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_reproduces_the_plain_operator_on_torch_built_a_b(dtype):
+    inp = _inputs(11, 2, 96, 3, 64, 64)
+    got, ref = _fused(inp, dtype, 1.0), _unfused(inp, dtype, 1.0)
+    # forward: same kernels on (nearly) the same a, b; gradients of k, beta, log_f: the plain route rounds da, db to the
+    # input type before torch's backward of the parameterisation, the fused one does not
+    _check(got, ref, 1e-3 if dtype == torch.bfloat16 else 1e-5, 8e-3 if dtype == torch.bfloat16 else 1e-5,
+           what=f"fused against plain, {dtype}")
+
+
+def test_packed_sequences_and_padded_head_dims():
+    cu = torch.tensor([0, 17, 17, 60, 100])
+    inp = _inputs(5, 1, 100, 2, 64, 64, N=4)
+    _check(_fused(inp, torch.bfloat16, 1.0, cu), _oracle(inp, torch.bfloat16, 1.0, cu), *TOL[torch.bfloat16], what="packed")
+    inp = _inputs(6, 1, 40, 2, 48, 96)
+    _check(_fused(inp, torch.float32, 1.0), _oracle(inp, torch.float32, 1.0), *TOL[torch.float32], what="K=48 V=96")

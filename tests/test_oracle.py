@@ -162,3 +162,28 @@ def test_golden_fixture_config0():
     assert abs(float(inp.gk.double().sum()) - float(gold["gk_sum"])) < 1e-5
     o2, h2 = O.chunk_naive(inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk, 1.0, None, chunk_size=16, dtype=torch.float32)
     assert O.rel_l2(o2, o) < 1e-5 and O.rel_l2(h2, h) < 1e-5
+
+
+def test_parameterize_a_b_gives_the_two_sided_householder_decay():
+    # hdla_custom.py:270-288: with a, b = parameterize_a_b(beta, k, log_f) one step of the recurrence without input
+    # (k v^T = 0) multiplies the state by (I - beta k k^T) Diag(f) (I - beta k k^T); recurrence() applies
+    # Diag(f) + sum_r b_r a_r^T, so the two must agree for any state (row order r = 0, 1 of a/b included)
+    g = torch.Generator().manual_seed(5)
+    B, T, H, K, V = 2, 1, 3, 7, 4
+    k = torch.randn(B, T, H, K, generator=g, dtype=D)
+    k = k / k.norm(dim=-1, keepdim=True)
+    beta = 2 * torch.rand(B, T, H, 1, generator=g, dtype=D)
+    log_f = -torch.rand(B, T, H, K, generator=g, dtype=D)
+    S0 = torch.randn(B, H, K, V, generator=g, dtype=D)
+    a, b = O.parameterize_a_b(beta, k, log_f)
+    assert a.shape == (B, 2 * T, H, K) and b.shape == a.shape
+    zero = torch.zeros(B, T, H, V, dtype=D)
+    _, S1 = O.recurrence(torch.zeros_like(k), k, zero, a, b, log_f, 1.0, S0)
+    kk = k[:, 0]
+    P = torch.eye(K, dtype=D) - beta[:, 0, :, :, None] * kk[..., :, None] * kk[..., None, :]     # I - beta k k^T
+    Hm = P @ torch.diag_embed(torch.exp(log_f[:, 0])) @ P
+    assert torch.allclose(S1, Hm @ S0, atol=1e-12)
+    # [B,T,H] beta is accepted as well, and the two ranks are not interchangeable
+    a3, b3 = O.parameterize_a_b(beta[..., 0], k, log_f)
+    assert torch.equal(a3, a) and torch.equal(b3, b)
+    assert not torch.allclose(a[:, 0], a[:, 1]) and torch.equal(b[:, 1], k[:, 0])
