@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the HDLA rank-2 DPLR delta-rule hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload train|fwd|varlen|decode|copy] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload train|fwd|varlen|decode|copy|hdla] [--no-cpu-baseline]
 
 Default workload ("train") is the headline configuration: chunked forward + backward at B=4, T=2048, H=16,
 K=V=64, bf16 inputs, fp32 state, random fp32 initial state, upstream gradients do and dht (configuration 2).
@@ -35,7 +35,7 @@ def _args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="train", choices=["train", "fwd", "varlen", "decode", "copy"])
+    ap.add_argument("--workload", default="train", choices=["train", "fwd", "varlen", "decode", "copy", "hdla"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
 
@@ -209,7 +209,7 @@ def main():
         print(json.dumps({"metric": "copy calibration", "bytes_read_per_launch": n, "bytes_written_per_launch": n,
                           "ms_per_step": sec * 1e3, "GB/s": 2 * n / sec / 1e9, "GB/s_by_read_write_mix": mixes}))
         return
-    cfg = {"train": 2, "fwd": 1, "varlen": 3, "decode": 4}[wl]
+    cfg = {"train": 2, "fwd": 1, "varlen": 3, "decode": 4, "hdla": 2}[wl]
     B, T, H, K, V = CONFIG_SHAPES[cfg]
     inp = make_config(cfg)
     dt = torch.bfloat16
@@ -256,6 +256,38 @@ def main():
         print(json.dumps(res))
         return
 
+    if wl == "hdla":
+        # The operator as the HDLA layer calls it (a, b given by beta, k, log_f), on the shape of configuration 2:
+        # a and b formed inside the kernels against the layer's own route (torch builds a, b, the plain operator runs
+        # on them, autograd goes back through both).  Whole-step rates only.
+        from hdla_hip import chunk_hdla_delta_rule, parameterize_a_b
+        g = torch.Generator().manual_seed(0)
+        beta = (2.0 * torch.rand(B, T, H, 1, generator=g)).to(dt).to(dev).requires_grad_()
+        q, k, v, lf = [x.to(dt).to(dev).requires_grad_() for x in (inp.q, inp.k, inp.v, inp.gk)]
+        h0 = inp.h0.to(dev).requires_grad_()
+        do, dht = inp.do.to(dt).to(dev), inp.dht.to(dev)
+
+        def fused():
+            o, ht = chunk_hdla_delta_rule(q, k, v, beta, lf, scale=1.0, initial_state=h0, output_final_state=True)
+            torch.autograd.grad([o, ht], [q, k, v, beta, lf, h0], [do, dht])
+
+        def plain():
+            a, b = parameterize_a_b(beta.float(), k.float(), lf.float())
+            o, ht = chunk_hrdplr_delta_rule(q, k, v, a.to(dt), b.to(dt), lf, 2, scale=1.0, initial_state=h0,
+                                            output_final_state=True, chunk_size=16)
+            torch.autograd.grad([o, ht], [q, k, v, beta, lf, h0], [do, dht])
+
+        sec = time_steps(fused, args.steps, args.warmup)
+        sec_plain = time_steps(plain, args.steps, args.warmup)
+        res.update(metric="chunked fwd+bwd tokens/s with a, b given by (beta, k, log_f)", value=B * T / sec,
+                   ms_per_step=sec * 1e3,
+                   config={"workload": "configuration 2 shape (B=4 T=2048 H=16 K=V=64, bf16), a and b formed in the kernels",
+                           "global_batch": B, "seq_len": T, "heads": H, "K": K, "V": V, "chunk": 16},
+                   plain_route={"what": "torch parameterize_a_b (fp32, eager) + chunk_hrdplr_delta_rule + autograd through both",
+                                "ms_per_step": sec_plain * 1e3, "value": B * T / sec_plain},
+                   roofline=None)
+        print(json.dumps(res))
+        return
     cu = None if inp.cu_seqlens is None else inp.cu_seqlens.to(dev)
     N = B if cu is None else cu.numel() - 1
     leaves = [x.to(dt).to(dev).requires_grad_(wl != "fwd") for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]

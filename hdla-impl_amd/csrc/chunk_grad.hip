@@ -52,17 +52,16 @@ template <typename T, int K, int V> struct CgLds {
 };
 
 // waves per SIMD asked of the compiler (lowest, highest): three workgroups per compute unit for the smallest 2-byte
-// shape, two for the other 2-byte shapes; the variant with the HDLA parameterisation carries its backward's
-// partial results across one more barrier and gets one step less
-template <typename T, int K, int V, bool HD> constexpr int cg_waves(bool highest) {
+// shape, two for the other 2-byte shapes
+template <typename T, bool GKF32, int K, int V, bool HD> constexpr int cg_waves(bool highest) {
     const bool small = sizeof(T) * K * V <= 2 * 64 * 64;
     if (sizeof(T) != 2) return highest ? 2 : 1;
-    if (HD) return small ? 2 : (highest ? 2 : 1);
+    if (HD && GKF32 && small) return 2;                   // fp32 decay next to 2-byte inputs: four more registers a tile
     return small ? 3 : 2;
 }
 
 template <typename T, bool GKF32, int K, int V, bool HD>
-__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(cg_waves<T, K, V, HD>(false), cg_waves<T, K, V, HD>(true)))) void chunk_grad_kernel(ChunkArgs<T> p) {
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(cg_waves<T, GKF32, K, V, HD>(false), cg_waves<T, GKF32, K, V, HD>(true)))) void chunk_grad_kernel(ChunkArgs<T> p) {
     constexpr int KT = K / 16, VT = V / 16, KT2 = KT / 2, KTW = KT / NW, VTW = VT / NW;
     static_assert(KT % NW == 0 && VT % NW == 0 && (KTW == 1 || KTW == 2), "a wave owns one channel tile or one stored pair");
     typedef CgLds<T, K, V> L;
@@ -194,47 +193,54 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(cg_wave
     if (EARLY) { own_kt_tiles(DHC, dhk); own_vt_tiles(DHC, dhv); load_b(); }
 
     // HDLA parameterisation (hdla_custom.py:19-43): a_1 = -beta k, a_2 = beta k (beta s - f), b_1 = f k, b_2 = k with
-    // f = exp(gk) and s = sum over ALL channels of k^2 f (every wave reads all of k and gk of the chunk for it), rounded
-    // to the element type as the layer's .to(dtype) does, so that everything below sees what the plain operator sees
+    // f = exp(gk) and s = sum over ALL channels of k^2 f.  A wave has a quarter of the channels: the waves exchange their
+    // parts of s with the parts of the score tiles below, and until then nothing may depend on a_2.
     float beta_t = 0.f, s_t = 0.f;
-    if (HD) {
-        beta_t = rowok ? ld_elem(p.beta + (cp.tok0 + row) * H + h) : 0.f;
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt) {
-            const f32x4 g4 = ld_gk4<GKF32>(gkp + go + 16 * kt * GS, 0, rowok);
-            const f32x4 k4 = to_f32(ld_frag_sel(at(p.k + qb, qo + 16 * kt * ES), rowok));
-            const f32x4 kf = k4 * k4 * exp4<T>(g4);
-            s_t += kf[0] + kf[1] + kf[2] + kf[3];
-        }
-        s_t += __shfl_xor(s_t, 16);
-        s_t += __shfl_xor(s_t, 32);
-#pragma unroll
-        for (int j = 0; j < KTW; ++j) {
-            const f32x4 kk = to_f32(rk[j]), f4 = exp4<T>(rg[j]);
-            ra[0][j] = to_frag<T>(kk * (-beta_t));
-            ra[1][j] = to_frag<T>(kk * ((beta_t * s_t - f4) * beta_t));
-            rb[0][j] = to_frag<T>(f4 * kk);
-            rb[1][j] = rk[j];
-        }
-    }
+    if (HD) beta_t = rowok ? ld_elem(p.beta + (cp.tok0 + row) * H + h) : 0.f;
+    // a and b of the own channel tiles as the products take them: as loaded, or (HDLA parameterisation) formed on the
+    // spot from k, gk, beta and s, which costs a few instructions and no registers in between
+    auto a_of = [&](int r, int j) __attribute__((always_inline)) {
+        if (!HD) return ra[r][j];
+        const f32x4 kk = to_f32(rk[j]);
+        return r == 0 ? to_frag<T>(kk * (-beta_t)) : to_frag<T>(kk * ((beta_t * s_t - exp4<T>(rg[j])) * beta_t));
+    };
+    auto b_of = [&](int r, int j) __attribute__((always_inline)) {
+        if (!HD) return rb[r][j];
+        return r == 0 ? to_frag<T>(exp4<T>(rg[j]) * to_f32(rk[j])) : rk[j];
+    };
     const Frag<T> ident = ident_frag<T>();
 
     // ---- own channel tiles: part of A_qk^T and A_ak^T (rows j, inner i); kg for everybody ------------------------
     {
+        // HDLA parameterisation: A_ak^r[i][j] = sum_c a_r[i][c] ea k^[j][c] with a_1 = -beta_i k, a_2 = beta_i^2 s_i k -
+        // beta_i f k: the two tiles exchanged are X1 = (k ea) k^^T and X2 = (k f ea) k^^T, which need neither beta nor
+        // s, and A_ak^1 = -beta X1, A_ak^2 = beta^2 s X1 - beta X2 follow from the sums (scaled along the inner index i)
         f32x4 aqkT = zero4(), aakT[2] = {zero4(), zero4()};
+        float sp = 0.f;
 #pragma unroll
         for (int j = 0; j < KTW; ++j) {
             const f32x4 g4 = rg[j];
             const f32x4 gi = scan16_incl(g4), ge = gi - g4;
             const f32x4 m = bcast16(gi, MID);
             const f32x4 eq = exp4<T>(gi - m), ek = exp4<T>(m - gi), ea = exp4<T>(ge - m);
-            const f32x4 q4 = to_f32(rq[j]), k4 = to_f32(rk[j]), a0 = to_f32(ra[0][j]), a1 = to_f32(ra[1][j]);
+            const f32x4 q4 = to_f32(rq[j]), k4 = to_f32(rk[j]);
             const Frag<T> qh = to_frag<T>(q4 * eq * scale), kh = to_frag<T>(k4 * ek);
             aqkT = mm(kh, qh, aqkT);
-            aakT[0] = mm(kh, to_frag<T>(a0 * ea), aakT[0]);
-            aakT[1] = mm(kh, to_frag<T>(a1 * ea), aakT[1]);
+            if (HD) {
+                const f32x4 f4 = exp4<T>(g4), kea = k4 * ea, kf = k4 * k4 * f4;
+                aakT[0] = mm(kh, to_frag<T>(kea), aakT[0]);
+                aakT[1] = mm(kh, to_frag<T>(kea * f4), aakT[1]);
+                sp += kf[0] + kf[1] + kf[2] + kf[3];
+            } else {
+                aakT[0] = mm(kh, to_frag<T>(to_f32(ra[0][j]) * ea), aakT[0]);
+                aakT[1] = mm(kh, to_frag<T>(to_f32(ra[1][j]) * ea), aakT[1]);
+            }
             const f32x4 edn = exp4<T>(bcast16(gi, CH - 1) - gi);
             st_tile(sKg + (kt0 + j) * TILE, to_frag<T>(k4 * edn));
+        }
+        if (HD) {
+            sp = sum_groups(sp);
+            if (g == 0) { sRed[(w * 3 + 0) * CH + c] = sp; sRed[(w * 3 + 1) * CH + c] = beta_t; }
         }
         *reinterpret_cast<f32x4*>(sScore + ((w * 3 + 0) * 64 + l) * 4) = aqkT;
         *reinterpret_cast<f32x4*>(sScore + ((w * 3 + 1) * 64 + l) * 4) = aakT[0];
@@ -280,6 +286,19 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(cg_wave
         for (int ww = 0; ww < NW; ++ww)
 #pragma unroll
             for (int i = 0; i < 3; ++i) t[i] += *reinterpret_cast<const f32x4*>(sScore + ((ww * 3 + i) * 64 + l) * 4);
+        if (HD) {
+            // s of the own token (lane c), and beta, s of the four tokens this lane holds along the inner index
+            f32x4 si = zero4();
+#pragma unroll
+            for (int ww = 0; ww < NW; ++ww) {
+                s_t += sRed[(ww * 3 + 0) * CH + c];
+                si += *reinterpret_cast<const f32x4*>(sRed + (ww * 3 + 0) * CH + 4 * g);
+            }
+            const f32x4 bi = *reinterpret_cast<const f32x4*>(sRed + 1 * CH + 4 * g);
+            const f32x4 x1 = t[1], x2 = t[2];
+            t[1] = -bi * x1;
+            t[2] = bi * bi * si * x1 - bi * x2;
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {          // row j = c, inner i = 4g+i
             const int ii = 4 * g + i;
@@ -406,7 +425,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(cg_wave
         else if (rowok) st_frag(at(p.dv + vb, vo + 16 * (vt0 + j) * ES), to_frag<T>(x));
     }
     // ---- own channel tiles, second pass: state products, score backward, final gradients ---------------------------
-    f32x4 dk_pre[HD ? KTW : 1], dg_pre[HD ? KTW : 1];
+    f32x4 dk_pre[(HD && !STAGE_OUT) ? KTW : 1], dg_pre[(HD && !STAGE_OUT) ? KTW : 1];
     float red[3] = {0.f, 0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < KTW; ++j) {
@@ -443,8 +462,8 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(cg_wave
         const f32x4 eq = exp4<T>(gi - m), ek = exp4<T>(m - gi), ea = exp4<T>(ge - m);
         const f32x4 egi = exp4<T>(gi), ege = exp4<T>(ge);
         const f32x4 q4 = to_f32(rq[j]);
-        const f32x4 a4[2] = {to_f32(ra[0][j]), to_f32(ra[1][j])};
-        const f32x4 b4[2] = {to_f32(rb[0][j]), to_f32(rb[1][j])};
+        const f32x4 a4[2] = {to_f32(a_of(0, j)), to_f32(a_of(1, j))};
+        const f32x4 b4[2] = {to_f32(b_of(0, j)), to_f32(b_of(1, j))};
         const Frag<T> qh = to_frag<T>(q4 * eq * scale), kh = to_frag<T>(k4 * ek);
         const Frag<T> ah[2] = {to_frag<T>(a4[0] * ea), to_frag<T>(a4[1] * ea)};
         const Frag<T> bh[2] = {to_frag<T>(b4[0] * ek), to_frag<T>(b4[1] * ek)};
@@ -489,8 +508,15 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(cg_wave
             // backward of the parameterisation, the part that needs no sum over channels; what does (through s, and
             // dbeta itself) waits for the sums r1 = sum k da_1, r2 = sum k da_2, r3 = sum k f da_2 of all the waves
             const f32x4 f4 = exp4<T>(g4);
-            dk_pre[j] = dk - da[0] * beta_t + da[1] * ((beta_t * s_t - f4) * beta_t) + db[0] * f4 + db[1];
-            dg_pre[j] = dg + (db[0] - da[1] * beta_t) * k4 * f4;
+            const f32x4 dkp = dk - da[0] * beta_t + da[1] * ((beta_t * s_t - f4) * beta_t) + db[0] * f4 + db[1];
+            const f32x4 dgp = dg + (db[0] - da[1] * beta_t) * k4 * f4;
+            if (STAGE_OUT) {       // kept, per lane, in the rows of the staging area that da and db do not use here
+                *reinterpret_cast<f32x4*>(sOut + 2 * CH * L::OPK + ((w * KTW + j) * 2 + 0) * 1024 + l * 16) = dkp;
+                *reinterpret_cast<f32x4*>(sOut + 2 * CH * L::OPK + ((w * KTW + j) * 2 + 1) * 1024 + l * 16) = dgp;
+            } else {
+                dk_pre[j] = dkp;
+                dg_pre[j] = dgp;
+            }
             const f32x4 t1 = k4 * da[0], t2 = k4 * da[1], t3 = t2 * f4;
             red[0] += t1[0] + t1[1] + t1[2] + t1[3];
             red[1] += t2[0] + t2[1] + t2[2] + t2[3];
@@ -522,8 +548,7 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(cg_wave
         // sums over all channels, per token: within the wave over the four lane groups, then over the waves through LDS
 #pragma unroll
         for (int i = 0; i < 3; ++i) {
-            red[i] += __shfl_xor(red[i], 16);
-            red[i] += __shfl_xor(red[i], 32);
+            red[i] = sum_groups(red[i]);
             if (g == 0) sRed[(w * 3 + i) * CH + c] = red[i];
         }
         __syncthreads();                                       // (3b) the sums of all waves are there
@@ -540,8 +565,10 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(cg_wave
         for (int j = 0; j < KTW; ++j) {
             const int kt = kt0 + j;
             const f32x4 k4 = to_f32(rk[j]), kf = k4 * exp4<T>(rg[j]);
-            const f32x4 dk = dk_pre[j] + kf * (2.f * ds);
-            const f32x4 dg = dg_pre[j] + kf * k4 * ds;
+            const f32x4 dkp = STAGE_OUT ? *reinterpret_cast<const f32x4*>(sOut + 2 * CH * L::OPK + ((w * KTW + j) * 2 + 0) * 1024 + l * 16) : dk_pre[j];
+            const f32x4 dgp = STAGE_OUT ? *reinterpret_cast<const f32x4*>(sOut + 2 * CH * L::OPK + ((w * KTW + j) * 2 + 1) * 1024 + l * 16) : dg_pre[j];
+            const f32x4 dk = dkp + kf * (2.f * ds);
+            const f32x4 dg = dgp + kf * k4 * ds;
             if (STAGE_OUT) {
                 put(1, kt, to_frag<T>(dk));
                 if (!GKF32) put(6, kt, to_frag<T>(dg));

@@ -293,4 +293,18 @@ __device__ __forceinline__ float xor32(float x) {
     return __int_as_float(lane_id() < 32 ? r[1] : r[0]);
 }
 
+// value held by the lane 16 positions away within each half of the wave (v_permlane16_swap exchanges odd and even
+// rows of 16 lanes between two registers)
+__device__ __forceinline__ float xor16(float x) {
+    const int xi = __float_as_int(x);
+    auto r = __builtin_amdgcn_permlane16_swap(xi, xi, false, false);     // r[0] rows: x0 x0 x2 x2, r[1]: x1 x1 x3 x3
+    return __int_as_float((lane_id() & 16) ? r[0] : r[1]);
+}
+// sum over the four lanes c, c+16, c+32, c+48, on all of them
+__device__ __forceinline__ float sum_groups(float x) {
+    x += xor16(x);
+    x += xor32(x);
+    return x;
+}
+
 }  // namespace hdla
