@@ -30,7 +30,8 @@ def test_library_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "hdla_hip.h")).read()
     names = set(re.findall(r"\b(hdla_[a-z_]+)\s*\(", header))
     assert {"hdla_version", "hdla_strerror", "hdla_workspace_bytes", "hdla_workspace_layout", "hdla_chunk_fwd",
-            "hdla_chunk_bwd", "hdla_chunk_stages", "hdla_recurrent_fwd"} <= names
+            "hdla_chunk_bwd", "hdla_chunk_stages", "hdla_recurrent_fwd", "hdla_param_chunk_fwd", "hdla_param_chunk_bwd",
+            "hdla_calib_stream"} <= names
     for n in names:
         assert hasattr(lib, n), n
     assert lib.hdla_version() == 100
@@ -87,6 +88,37 @@ def test_null_misaligned_and_small_workspace():
     assert lib.hdla_chunk_bwd(ctypes.byref(d), ok, ok, ok, ok, ok, ok, None, None, None, ok, ok, ok, ok, ok, ok, None,
                               ok, 1 << 40, None) == -1
     assert lib.hdla_workspace_layout(ctypes.byref(d), 0, None) == -1
+
+
+def test_parameterised_entry_points_check_their_arguments():
+    lib = _lib.load()
+    d = _dims()
+    ok, bad = ctypes.c_void_p(4096), ctypes.c_void_p(4096 + 8)
+    f = lib.hdla_param_chunk_fwd
+    assert f(ctypes.byref(d), ok, ok, ok, None, ok, None, ok, None, ok, 1 << 40, None) == -1      # beta is required
+    assert f(ctypes.byref(d), ok, None, ok, ok, ok, None, ok, None, ok, 1 << 40, None) == -1
+    assert f(ctypes.byref(d), ok, bad, ok, ok, ok, None, ok, None, ok, 1 << 40, None) == -6
+    assert f(ctypes.byref(d), ok, ok, ok, ok, ok, None, ok, None, ok, 1024, None) == -5
+    assert f(ctypes.byref(_dims(K=96)), ok, ok, ok, ok, ok, None, ok, None, ok, 1 << 40, None) == -2
+    g = lib.hdla_param_chunk_bwd
+    assert g(ctypes.byref(d), ok, ok, ok, ok, ok, None, ok, None, ok, ok, ok, None, ok, None, ok, 1 << 40, None) == -1   # dbeta
+    assert g(ctypes.byref(d), ok, ok, ok, ok, ok, None, ok, None, ok, ok, ok, ok, ok, None, None, 1 << 40, None) == -5
+
+
+def test_parameterised_python_entry_validates_and_needs_a_gpu():
+    from hdla_hip import chunk_hdla_delta_rule, parameterize_a_b
+    x = make_inputs(3, 2, 32, 2, 64, 64)
+    q, k, v, gk = [t.bfloat16() for t in (x.q, x.k, x.v, x.gk)]
+    beta = torch.rand(2, 32, 2, 1).bfloat16()
+    with pytest.raises(ValueError):
+        chunk_hdla_delta_rule(q, k, v, beta[:, :5], gk)
+    with pytest.raises(ValueError):
+        chunk_hdla_delta_rule(q, k[:, :5], v, beta, gk)
+    with pytest.raises(_lib.HdlaError):
+        chunk_hdla_delta_rule(q, k, v, beta, gk)                      # CPU tensors: no fallback
+    a, b = parameterize_a_b(beta.float(), k.float(), gk.float())       # the reference's helper, with its return
+    assert a.shape == (2, 64, 2, 64) and b.shape == a.shape
+    assert torch.equal(b[:, 1::2], k.float()) and torch.allclose(a[:, 0::2], -beta.float() * k.float())
 
 
 def _cpu_args(T=32, K=64, V=64, R=2, B=2):
