@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the HDLA rank-2 DPLR delta-rule hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload train|fwd|varlen|decode|copy|hdla] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload train|fwd|varlen|decode|copy|hdla|hdla_decode] [--no-cpu-baseline]
 
 Default workload ("train") is the headline configuration: chunked forward + backward at B=4, T=2048, H=16,
 K=V=64, bf16 inputs, fp32 state, random fp32 initial state, upstream gradients do and dht (configuration 2).
@@ -35,7 +35,7 @@ def _args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="train", choices=["train", "fwd", "varlen", "decode", "copy", "hdla"])
+    ap.add_argument("--workload", default="train", choices=["train", "fwd", "varlen", "decode", "copy", "hdla", "hdla_decode"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
 
@@ -209,7 +209,7 @@ def main():
         print(json.dumps({"metric": "copy calibration", "bytes_read_per_launch": n, "bytes_written_per_launch": n,
                           "ms_per_step": sec * 1e3, "GB/s": 2 * n / sec / 1e9, "GB/s_by_read_write_mix": mixes}))
         return
-    cfg = {"train": 2, "fwd": 1, "varlen": 3, "decode": 4, "hdla": 2}[wl]
+    cfg = {"train": 2, "fwd": 1, "varlen": 3, "decode": 4, "hdla": 2, "hdla_decode": 4}[wl]
     B, T, H, K, V = CONFIG_SHAPES[cfg]
     inp = make_config(cfg)
     dt = torch.bfloat16
@@ -253,6 +253,46 @@ def main():
                              "traffic": measured_traffic("decode", "recurrent", K, V), "bytes_per_launch": nbytes, "ms_per_launch": kms})
         if not args.no_cpu_baseline:
             res["cpu_baseline"] = cpu_baseline_decode()
+        print(json.dumps(res))
+        return
+
+    if wl == "hdla_decode":
+        # One decode step of the HDLA layer on the shape of configuration 4: a and b formed per token inside the
+        # token-serial kernel, against the layer's own route (torch builds a, b from beta, k, log_f, then the plain
+        # recurrent operator).  Whole-step rates only; the kernel's traffic is the state, as for "decode".
+        from hdla_hip import fused_recurrent_hdla_delta_rule, parameterize_a_b
+        from hdla_hip.synthetic import make_inputs
+        ncycle = 8
+        gen = [inp] + [make_inputs(2000 + i, B, 1, H, K, V, h0_std=0.1) for i in range(1, ncycle)]
+        g = torch.Generator().manual_seed(0)
+        steps_in = [[x.to(dt).to(dev) for x in (c.q, c.k, c.v, 2.0 * torch.rand(B, 1, H, 1, generator=g), c.gk)] for c in gen]
+        state = {"S": inp.h0.to(dev), "i": 0}
+
+        def fused():
+            t = steps_in[state["i"] % ncycle]
+            state["i"] += 1
+            _, state["S"] = fused_recurrent_hdla_delta_rule(*t, scale=1.0, initial_state=state["S"], output_final_state=True)
+
+        def plain():
+            q, k, v, beta, lf = steps_in[state["i"] % ncycle]
+            state["i"] += 1
+            a, b = parameterize_a_b(beta.float(), k.float(), lf.float())
+            _, state["S"] = fused_recurrent_dplr_delta_rule(q, k, v, a.to(dt), b.to(dt), lf, 2, scale=1.0,
+                                                            initial_state=state["S"], output_final_state=True)
+
+        sec = time_steps(fused, args.steps, args.warmup)
+        state["S"] = inp.h0.to(dev)
+        sec_plain = time_steps(plain, args.steps, args.warmup)
+        nbytes = 2 * B * H * K * V * 4 + B * H * (3 * K + V + V + 1) * 2
+        res.update(metric="decode tokens/s with a, b given by (beta, k, log_f)", value=B / sec, ms_per_step=sec * 1e3,
+                   config={"workload": "configuration 4 shape (B=256 H=32 K=V=128, one token per call, persistent fp32 "
+                                       "state), a and b formed in the kernel", "batch": B, "heads": H, "K": K, "V": V},
+                   plain_route={"what": "torch parameterize_a_b (fp32, eager) + fused_recurrent_dplr_delta_rule",
+                                "ms_per_step": sec_plain * 1e3, "value": B / sec_plain},
+                   roofline={"bound": "hbm", "kernel": "recurrent_kernel", "achieved": nbytes / sec / 1e9,
+                             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / sec / 1e9 / HBM_PEAK_GBS,
+                             "traffic": None, "bytes_per_launch": nbytes, "ms_per_launch": sec * 1e3,
+                             "note": "whole step on the host clock (one kernel per step)"})
         print(json.dumps(res))
         return
 

@@ -287,19 +287,16 @@ int hdla_chunk_stages(const hdla_dims* dims, int pass, int stages, const void* q
                             workspace, workspace_bytes, s, stages);
 }
 
-int hdla_recurrent_fwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
-                       const void* b, const void* gk, int reverse, const float* h0, void* o, float* ht,
-                       void* stream) {
-    const int rc = check_dims(dims);
-    if (rc) return rc;
-    if (dims->T > 0 && (!q || !k || !v || !a || !b || !gk || !o)) return HDLA_ERR_NULL;
-    if (!aligned16(h0) || !aligned16(ht)) return HDLA_ERR_ALIGN;
+static int run_recurrent(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
+                         const void* b, const void* beta, const void* gk, int reverse, const float* h0, void* o,
+                         float* ht, void* stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e;
     if (dims->in_dtype == HDLA_BF16) {
         RecurrentArgs<bf16> r{};
         r.q = static_cast<const bf16*>(q); r.k = static_cast<const bf16*>(k); r.v = static_cast<const bf16*>(v);
         r.a = static_cast<const bf16*>(a); r.b = static_cast<const bf16*>(b);
+        r.beta = static_cast<const bf16*>(beta);
         r.gk = gk; r.gk_f32 = dims->gk_dtype == HDLA_FP32;
         r.H = dims->H; r.T_ = dims->T; r.N = dims->N; r.scale = dims->scale; r.reverse = reverse;
         r.cu = dims->cu_seqlens; r.h0 = h0; r.ht = ht; r.o = static_cast<bf16*>(o);
@@ -308,12 +305,33 @@ int hdla_recurrent_fwd(const hdla_dims* dims, const void* q, const void* k, cons
         RecurrentArgs<float> r{};
         r.q = static_cast<const float*>(q); r.k = static_cast<const float*>(k); r.v = static_cast<const float*>(v);
         r.a = static_cast<const float*>(a); r.b = static_cast<const float*>(b);
+        r.beta = static_cast<const float*>(beta);
         r.gk = gk; r.gk_f32 = 1;
         r.H = dims->H; r.T_ = dims->T; r.N = dims->N; r.scale = dims->scale; r.reverse = reverse;
         r.cu = dims->cu_seqlens; r.h0 = h0; r.ht = ht; r.o = static_cast<float*>(o);
         e = launch_recurrent<float>(r, dims->K, dims->V, s);
     }
     return e == hipSuccess ? HDLA_OK : (int)e;
+}
+
+int hdla_recurrent_fwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
+                       const void* b, const void* gk, int reverse, const float* h0, void* o, float* ht,
+                       void* stream) {
+    const int rc = check_dims(dims);
+    if (rc) return rc;
+    if (dims->T > 0 && (!q || !k || !v || !a || !b || !gk || !o)) return HDLA_ERR_NULL;
+    if (!aligned16(h0) || !aligned16(ht)) return HDLA_ERR_ALIGN;
+    return run_recurrent(dims, q, k, v, a, b, nullptr, gk, reverse, h0, o, ht, stream);
+}
+
+int hdla_param_recurrent_fwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* beta,
+                             const void* gk, int reverse, const float* h0, void* o, float* ht, void* stream) {
+    const int rc = check_dims(dims);
+    if (rc) return rc;
+    if (!beta) return HDLA_ERR_NULL;
+    if (dims->T > 0 && (!q || !k || !v || !gk || !o)) return HDLA_ERR_NULL;
+    if (!aligned16(h0) || !aligned16(ht)) return HDLA_ERR_ALIGN;
+    return run_recurrent(dims, q, k, v, nullptr, nullptr, beta, gk, reverse, h0, o, ht, stream);
 }
 
 }  // extern "C"

@@ -128,6 +128,7 @@ struct ChunkArgs {            // inputs of the chunked operator + workspace
 template <typename T>
 struct RecurrentArgs {
     const T *q, *k, *v, *a, *b;
+    const T* beta;            // non-null: a, b formed per token from (beta, k, gk); a and b are not read
     const void* gk;
     int gk_f32;
     int H, T_, N;

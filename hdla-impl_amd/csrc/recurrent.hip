@@ -9,6 +9,11 @@
 // row segments, and all of a block's loads are in flight before the first use.  The two reductions over K
 // (a^T S and q^T S) run as in-lane partial sums, two cross-lane butterfly steps and one LDS exchange between
 // the four wavefronts.
+//
+// HD mode (p.beta given) forms the rank terms of the HDLA layer per token from (beta, k, gk) instead of reading
+// them (HRDPLR/hdla_custom.py:19-43): with f = exp(gk) and s = sum_c k_c^2 f_c,
+//     a_1 = -beta k,  a_2 = beta k (beta s - f),  b_1 = f k,  b_2 = k,
+// each rounded to the input type as the stored tensors would be.
 #include "hdla_common.cuh"
 #include "hdla_launch.h"
 
@@ -16,16 +21,19 @@ namespace hdla {
 
 __device__ __forceinline__ float ld_as_float(const bf16* p) { return bf2f(p->x); }
 __device__ __forceinline__ float ld_as_float(const float* p) { return *p; }
+__device__ __forceinline__ float round_as(const bf16*, float x) { return bf2f(f2bf(x)); }
+__device__ __forceinline__ float round_as(const float*, float x) { return x; }
 __device__ __forceinline__ float ld_gk1(const void* base, int64_t off, int is_f32) {
     return is_f32 ? reinterpret_cast<const float*>(base)[off] : bf2f(reinterpret_cast<const bf16*>(base)[off].x);
 }
 
-template <typename T, int K, int V, int BV>
+template <typename T, int K, int V, int BV, bool HD>
 __global__ __launch_bounds__(256) void recurrent_kernel(RecurrentArgs<T> p) {
     constexpr int CG = BV / 4;        // lanes across a row segment (float4 each)
     constexpr int RG = 256 / CG;      // row groups
     constexpr int RPT = K / RG;       // state rows per thread
     static_assert(K % RG == 0 && RPT >= 1, "tile shape");
+    static_assert(K <= 256, "one channel per thread in the per-token fill");
     __shared__ float sq[K], sk[K], seg[K], sa[2][K], sb[2][K], sv[BV];
     __shared__ float red[4][3][BV];
 
@@ -47,16 +55,41 @@ __global__ __launch_bounds__(256) void recurrent_kernel(RecurrentArgs<T> p) {
     for (int step = 0; step < len; ++step) {
         const int64_t t = p.reverse ? (eos - 1 - step) : (bos + step);
         __syncthreads();
-        for (int idx = tid; idx < K; idx += 256) {
-            const int64_t off = (t * H + h) * K + idx;
-            const int64_t off0 = ((t * RANK + 0) * H + h) * K + idx, off1 = ((t * RANK + 1) * H + h) * K + idx;
-            sq[idx] = ld_as_float(p.q + off) * p.scale;
-            sk[idx] = ld_as_float(p.k + off);
-            seg[idx] = exp_t<T>(ld_gk1(p.gk, off, p.gk_f32));
-            sa[0][idx] = ld_as_float(p.a + off0);
-            sa[1][idx] = ld_as_float(p.a + off1);
-            sb[0][idx] = ld_as_float(p.b + off0);
-            sb[1][idx] = ld_as_float(p.b + off1);
+        if constexpr (HD) {
+            const int64_t off = (t * H + h) * K + tid;
+            float kk = 0.f, f = 0.f;
+            if (tid < K) {
+                kk = ld_as_float(p.k + off);
+                f = exp_t<T>(ld_gk1(p.gk, off, p.gk_f32));
+                sq[tid] = ld_as_float(p.q + off) * p.scale;
+            }
+            float part = kk * kk * f;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) part += __shfl_xor(part, o);
+            if (lane == 0) red[wave][0][0] = part;
+            __syncthreads();
+            if (tid < K) {
+                const float s = red[0][0][0] + red[1][0][0] + red[2][0][0] + red[3][0][0];
+                const float beta = ld_as_float(p.beta + t * H + h);
+                sk[tid] = kk;
+                seg[tid] = f;
+                sa[0][tid] = round_as(p.k, -beta * kk);
+                sa[1][tid] = round_as(p.k, (beta * s - f) * beta * kk);
+                sb[0][tid] = round_as(p.k, f * kk);
+                sb[1][tid] = kk;
+            }
+        } else {
+            for (int idx = tid; idx < K; idx += 256) {
+                const int64_t off = (t * H + h) * K + idx;
+                const int64_t off0 = ((t * RANK + 0) * H + h) * K + idx, off1 = ((t * RANK + 1) * H + h) * K + idx;
+                sq[idx] = ld_as_float(p.q + off) * p.scale;
+                sk[idx] = ld_as_float(p.k + off);
+                seg[idx] = exp_t<T>(ld_gk1(p.gk, off, p.gk_f32));
+                sa[0][idx] = ld_as_float(p.a + off0);
+                sa[1][idx] = ld_as_float(p.a + off1);
+                sb[0][idx] = ld_as_float(p.b + off0);
+                sb[1][idx] = ld_as_float(p.b + off1);
+            }
         }
         if (tid < BV) sv[tid] = ld_as_float(p.v + (t * H + h) * V + vb * BV + tid);
         __syncthreads();
@@ -116,7 +149,8 @@ template <typename T, int K, int V>
 static hipError_t launch_recurrent_kv(const RecurrentArgs<T>& a, hipStream_t stream) {
     constexpr int BV = 64;
     dim3 grid(a.N * a.H, V / BV), block(256);
-    hipLaunchKernelGGL((recurrent_kernel<T, K, V, BV>), grid, block, 0, stream, a);
+    if (a.beta) hipLaunchKernelGGL((recurrent_kernel<T, K, V, BV, true>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((recurrent_kernel<T, K, V, BV, false>), grid, block, 0, stream, a);
     return hipGetLastError();
 }
 

@@ -4,7 +4,7 @@ Exports the two operators of the reference package (HRDPLR/__init__.py:1-12) wit
 operator as the HDLA layer calls it (a, b given by beta, k, log_f: HRDPLR/hdla_custom.py:19-43,290-309).
 """
 from .chunk import ChunkDPLRDeltaRuleFunction, chunk_hrdplr_delta_rule
-from .hdla import ChunkHDLAFunction, chunk_hdla_delta_rule, parameterize_a_b
+from .hdla import ChunkHDLAFunction, chunk_hdla_delta_rule, fused_recurrent_hdla_delta_rule, parameterize_a_b
 from .recurrent import FusedRecurrentDPLRDeltaRuleFunction, fused_recurrent_dplr_delta_rule
 
 __all__ = [
@@ -13,6 +13,7 @@ __all__ = [
     "ChunkDPLRDeltaRuleFunction",
     "FusedRecurrentDPLRDeltaRuleFunction",
     "chunk_hdla_delta_rule",
+    "fused_recurrent_hdla_delta_rule",
     "parameterize_a_b",
     "ChunkHDLAFunction",
 ]

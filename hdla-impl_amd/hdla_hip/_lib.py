@@ -71,6 +71,8 @@ def load():
     lib.hdla_calib_stream.argtypes = [ctypes.POINTER(P), ctypes.c_int, ctypes.POINTER(P), ctypes.c_int, ctypes.c_size_t, P]
     lib.hdla_recurrent_fwd.restype = ctypes.c_int
     lib.hdla_recurrent_fwd.argtypes = [F] + [P] * 6 + [ctypes.c_int] + [P] * 4
+    lib.hdla_param_recurrent_fwd.restype = ctypes.c_int
+    lib.hdla_param_recurrent_fwd.argtypes = [F] + [P] * 5 + [ctypes.c_int] + [P] * 4
     _lib = lib
     return lib
 

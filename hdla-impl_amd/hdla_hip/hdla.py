@@ -7,6 +7,10 @@
   b: the kernels form them from (beta, k, log_f) where they are used, and the backward pass returns the gradients of
   (q, k, v, beta, log_f) directly (C ABI: ``hdla_param_chunk_fwd`` / ``hdla_param_chunk_bwd``).
 
+* ``fused_recurrent_hdla_delta_rule`` <- the same pair for the token-serial operator (``parameterize_a_b`` +
+  ``fused_recurrent_dplr_delta_rule``, HRDPLR/recurrent.py:227-319), forward only, for decode steps that carry the
+  state a chunked prefill returned (C ABI: ``hdla_param_recurrent_fwd``).
+
 a and b are half of the operator's input bytes and da, db half of its gradient bytes; the layer also saves the
 elementwise kernels (and their backward) that would build them.
 """
@@ -161,3 +165,76 @@ def chunk_hdla_delta_rule(
     if final_state is not None and (Kn != K or Vn != V):
         final_state = final_state[:, :, :K, :V]
     return o.to(out_dtype), final_state
+
+
+@torch.compiler.disable
+def fused_recurrent_hdla_delta_rule(
+    q: torch.Tensor,                 # [B, T, H, K]
+    k: torch.Tensor,                 # [B, T, H, K]
+    v: torch.Tensor,                 # [B, T, H, V]
+    beta: torch.Tensor,              # [B, T, H, 1] or [B, T, H]
+    log_f: torch.Tensor,             # [B, T, H, K], log-space decay
+    scale: Optional[float] = None,
+    initial_state: Optional[torch.Tensor] = None,    # [N, H, K, V]
+    output_final_state: bool = False,
+    reverse: bool = False,
+    cu_seqlens: Optional[torch.Tensor] = None,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """``fused_recurrent_dplr_delta_rule(q, k, v, *parameterize_a_b(beta, k, log_f), gk=log_f, rank_ab=2, ...)``
+    with a and b (rounded to q's dtype) formed per token inside the kernel.  Inference only: no gradients, like
+    the plain recurrent operator (HRDPLR/recurrent.py:219-224)."""
+    assert q.dtype == k.dtype == v.dtype
+    if q.dim() != 4 or v.dim() != 4:
+        raise ValueError("q, k, v must be 4-dimensional [B, T, H, D]")
+    B, T, H, K = q.shape
+    V = v.shape[-1]
+    if k.shape != q.shape or log_f.shape != q.shape or v.shape[:3] != q.shape[:3]:
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)} log_f {tuple(log_f.shape)}")
+    if beta.shape not in ((B, T, H, 1), (B, T, H)):
+        raise ValueError(f"beta must be [B, T, H, 1] or [B, T, H], got {tuple(beta.shape)}")
+    if cu_seqlens is not None:
+        if B != 1:
+            raise ValueError(f"The batch size is expected to be 1 rather than {B} when using `cu_seqlens`."
+                             f"Please flatten variable-length inputs before processing.")
+        if initial_state is not None and initial_state.shape[0] != len(cu_seqlens) - 1:
+            raise ValueError(f"The number of initial states is expected to be equal to the number of input sequences, "
+                             f"i.e., {len(cu_seqlens) - 1} rather than {initial_state.shape[0]}.")
+        cu_seqlens = cu_seqlens.to(device=q.device, dtype=torch.int64).contiguous()
+    elif initial_state is not None and initial_state.shape[0] != B:
+        raise ValueError(f"initial_state must hold one state per sequence ({B}), got {initial_state.shape[0]}")
+    if any(x.requires_grad for x in (q, k, v, beta, log_f)) and torch.is_grad_enabled():
+        raise NotImplementedError("fused_recurrent_hdla_delta_rule is only for inference. "
+                                  "For training, please use `chunk_hdla_delta_rule`.")
+    _require_gpu(q, k, v, beta, log_f, initial_state)
+    scale = K ** -0.5 if scale is None else scale
+
+    out_dtype = v.dtype
+    if q.dtype == torch.float16:
+        q, k, v, beta, log_f = (x.float() for x in (q, k, v, beta, log_f))
+    elif q.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError(f"unsupported dtype {q.dtype}")
+    beta = beta.to(q.dtype).reshape(B, T, H).contiguous()
+    gk = log_f
+    if gk.dtype != torch.float32 and gk.dtype != q.dtype:
+        gk = gk.float()
+    Kn, Vn = _native_dim(K), _native_dim(V)
+    h0 = None if initial_state is None else initial_state.to(torch.float32)
+    if h0 is not None and (Kn != K or Vn != V):
+        h0 = F.pad(h0, (0, Vn - V, 0, Kn - K))
+    q, k, v, gk = (_pad_last(x, n).contiguous() for x, n in ((q, Kn), (k, Kn), (v, Vn), (gk, Kn)))
+    N = B if cu_seqlens is None else cu_seqlens.numel() - 1
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        dims = _dims(q, v, gk, scale, cu_seqlens, N)
+        h0 = None if h0 is None else h0.contiguous()
+        ht = torch.empty(N, H, Kn, Vn, dtype=torch.float32, device=q.device) if output_final_state else None
+        o = torch.empty_like(v)
+        rc = lib.hdla_param_recurrent_fwd(ctypes.byref(dims), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(beta),
+                                          _lib.ptr(gk), int(bool(reverse)), _lib.ptr(h0), _lib.ptr(o), _lib.ptr(ht),
+                                          _lib.current_stream(q.device))
+        _lib.check(rc, "hdla_param_recurrent_fwd")
+    if Vn != V:
+        o = o[..., :V]
+    if ht is not None and (Kn != K or Vn != V):
+        ht = ht[:, :, :K, :V]
+    return o.to(out_dtype), ht

@@ -11,6 +11,7 @@
  *                           (chunk_dplr_bwd_dAu HRDPLR/bwd_func.py:18, _dhu :63, _dv :125, _bwd_o :155,
  *                            _bwd_wy :218, _bwd_dqk_intra :274)
  *   hdla_recurrent_fwd  <-  fused_recurrent_dplr_delta_rule_fwd   HRDPLR/recurrent.py:121-177
+ *   hdla_param_*        <-  the same three with parameterize_a_b (HRDPLR/hdla_custom.py:19-43) folded in
  *
  * Conventions
  *   - All tensor pointers are DEVICE pointers to contiguous, 16-byte aligned buffers owned by the caller.
@@ -131,6 +132,13 @@ int hdla_chunk_stages(const hdla_dims* dims, int pass, int stages, const void* q
 int hdla_recurrent_fwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
                        const void* b, const void* gk, int reverse, const float* h0, void* o, float* ht,
                        void* stream);
+
+/* The same recurrence with the rank terms of the HDLA layer formed per token inside the kernel from
+ * (beta [B,T,H], k, gk = log f) instead of read from a and b: parameterize_a_b, HRDPLR/hdla_custom.py:19-43,
+ * followed by fused_recurrent_dplr_delta_rule_fwd, HRDPLR/recurrent.py:121-177.  beta has the input dtype and
+ * must not be NULL (also when T = 0: it selects the mode). */
+int hdla_param_recurrent_fwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* beta,
+                             const void* gk, int reverse, const float* h0, void* o, float* ht, void* stream);
 
 /* Measurement aid; it has no counterpart in the reference.  One launch of a kernel that reads `n_read` (0..3)
  * buffers and writes `n_write` (0..2) buffers of `bytes` bytes each (a multiple of 16; every pointer 16-byte

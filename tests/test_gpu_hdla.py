@@ -2,11 +2,13 @@
 (1) the float64 recurrence on a, b = oracle.parameterize_a_b(beta, k, log_f) with autograd through both, to the
 stated tolerances (outputs and state 5e-3, gradients 1e-2 for bf16; 1e-5 for fp32), and (2) the plain operator fed
 with the torch-built a and b, which it must reproduce almost to the bit (the kernels round a and b to the input
-type exactly as ``.to(dtype)`` does; only exp() differs in the last place)."""
+type exactly as ``.to(dtype)`` does; only exp() differs in the last place).  The token-serial operator (hdla_hip.fused_recurrent_hdla_delta_rule) is held
+to the same two references, forward only, and to the chunked one across a prefill -> decode hand-over."""
 import pytest
 import torch
 
-from hdla_hip import chunk_hdla_delta_rule, chunk_hrdplr_delta_rule, parameterize_a_b
+from hdla_hip import (chunk_hdla_delta_rule, chunk_hrdplr_delta_rule, fused_recurrent_dplr_delta_rule,
+                      fused_recurrent_hdla_delta_rule, parameterize_a_b)
 from oracle import hrdplr_oracle as O
 
 pytestmark = pytest.mark.gpu
@@ -103,3 +105,70 @@ def test_packed_sequences_and_padded_head_dims():
     _check(_fused(inp, torch.bfloat16, 1.0, cu), _oracle(inp, torch.bfloat16, 1.0, cu), *TOL[torch.bfloat16], what="packed")
     inp = _inputs(6, 1, 40, 2, 48, 96)
     _check(_fused(inp, torch.float32, 1.0), _oracle(inp, torch.float32, 1.0), *TOL[torch.float32], what="K=48 V=96")
+
+
+REC_CASES = [
+    (torch.float32, 2, 9, 2, 64, 64, 4.0, 1.0, False),
+    (torch.float32, 1, 5, 3, 128, 128, 1.0, 0.5, True),
+    (torch.bfloat16, 3, 1, 4, 128, 128, 4.0, 1.0, False),
+    (torch.bfloat16, 2, 20, 2, 64, 128, 16.0, 0.125, False),
+    (torch.bfloat16, 1, 12, 3, 128, 64, 1.0, 1.0, True),
+    (torch.bfloat16, 2, 7, 2, 48, 96, 4.0, 1.0, False),
+]
+
+
+@pytest.mark.parametrize("dtype,B,T,H,K,V,gk_div,scale,reverse", REC_CASES)
+def test_recurrent_against_the_recurrence(dtype, B, T, H, K, V, gk_div, scale, reverse):
+    q, k, v, beta, log_f, h0, _, _ = _inputs(900 + T, B, T, H, K, V, gk_div=gk_div)
+    lo = [t.to(dtype) for t in (q, k, v, beta, log_f)]
+    a, b = O.parameterize_a_b(lo[3].double(), lo[1].double(), lo[4].double())
+    ro, rht = O.recurrence(lo[0], lo[1], lo[2], a, b, lo[4], scale, h0.double(), reverse=reverse)
+    o, ht = fused_recurrent_hdla_delta_rule(*[t.to(DEV) for t in lo], scale=scale, initial_state=h0.to(DEV),
+                                            output_final_state=True, reverse=reverse)
+    assert o.dtype == dtype and ht.dtype == torch.float32 and ht.shape == (B, H, K, V)
+    eo, eh = O.rel_l2(o, ro), O.rel_l2(ht, rht)
+    print(f"recurrent {dtype} B{B} T{T} H{H} K{K} V{V} rev{reverse}: o {eo:.2e} ht {eh:.2e}", flush=True)
+    assert eo <= TOL[dtype][0] and eh <= TOL[dtype][0]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_recurrent_reproduces_the_plain_operator_on_torch_built_a_b(dtype):
+    q, k, v, beta, log_f, h0, _, _ = _inputs(21, 1, 30, 2, 128, 128, N=3)
+    cu = torch.tensor([0, 11, 11, 30], device=DEV)
+    lo = [t.to(dtype).to(DEV) for t in (q, k, v, beta, log_f)]
+    a, b = parameterize_a_b(lo[3].float(), lo[1].float(), lo[4].float())
+    ro, rht = fused_recurrent_dplr_delta_rule(lo[0], lo[1], lo[2], a.to(dtype), b.to(dtype), lo[4], rank_ab=2, scale=1.0,
+                                              initial_state=h0.to(DEV), output_final_state=True, cu_seqlens=cu)
+    o, ht = fused_recurrent_hdla_delta_rule(*lo, scale=1.0, initial_state=h0.to(DEV), output_final_state=True,
+                                            cu_seqlens=cu)
+    tol = 1e-3 if dtype == torch.bfloat16 else 1e-5
+    eo, eh = O.rel_l2(o, ro), O.rel_l2(ht, rht)
+    print(f"recurrent fused against plain {dtype}: o {eo:.2e} ht {eh:.2e}", flush=True)
+    assert eo <= tol and eh <= tol
+
+
+def test_prefill_then_decode_equals_one_pass():
+    """A chunked prefill of 70 tokens hands its state to 6 single-token steps of the token-serial operator; outputs
+    and the last state must match one chunked pass over all 76 tokens."""
+    dtype, B, T, H, K, V, P = torch.bfloat16, 2, 76, 3, 128, 128, 70
+    q, k, v, beta, log_f, h0, _, _ = _inputs(31, B, T, H, K, V)
+    lo = [t.to(dtype).to(DEV) for t in (q, k, v, beta, log_f)]
+    with torch.no_grad():
+        ro, rht = chunk_hdla_delta_rule(*lo, scale=1.0, initial_state=h0.to(DEV), output_final_state=True)
+        o, S = chunk_hdla_delta_rule(*[t[:, :P] for t in lo], scale=1.0, initial_state=h0.to(DEV), output_final_state=True)
+        outs = [o]
+        for t in range(P, T):
+            o, S = fused_recurrent_hdla_delta_rule(*[x[:, t:t + 1] for x in lo], scale=1.0, initial_state=S,
+                                                   output_final_state=True)
+            outs.append(o)
+    eo, eh = O.rel_l2(torch.cat(outs, 1), ro), O.rel_l2(S, rht)
+    print(f"prefill+decode against one pass: o {eo:.2e} ht {eh:.2e}", flush=True)
+    assert eo <= 5e-3 and eh <= 5e-3
+
+
+def test_recurrent_is_inference_only():
+    q, k, v, beta, log_f, *_ = _inputs(1, 1, 2, 1, 64, 64)
+    lo = [t.bfloat16().to(DEV) for t in (q, k, v, beta, log_f)]
+    lo[1].requires_grad_()
+    with pytest.raises(NotImplementedError):
+        fused_recurrent_hdla_delta_rule(*lo)

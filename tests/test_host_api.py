@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
     names = set(re.findall(r"\b(hdla_[a-z_]+)\s*\(", header))
     assert {"hdla_version", "hdla_strerror", "hdla_workspace_bytes", "hdla_workspace_layout", "hdla_chunk_fwd",
             "hdla_chunk_bwd", "hdla_chunk_stages", "hdla_recurrent_fwd", "hdla_param_chunk_fwd", "hdla_param_chunk_bwd",
-            "hdla_calib_stream"} <= names
+            "hdla_param_recurrent_fwd", "hdla_calib_stream"} <= names
     for n in names:
         assert hasattr(lib, n), n
     assert lib.hdla_version() == 100
@@ -103,10 +103,15 @@ def test_parameterised_entry_points_check_their_arguments():
     g = lib.hdla_param_chunk_bwd
     assert g(ctypes.byref(d), ok, ok, ok, ok, ok, None, ok, None, ok, ok, ok, None, ok, None, ok, 1 << 40, None) == -1   # dbeta
     assert g(ctypes.byref(d), ok, ok, ok, ok, ok, None, ok, None, ok, ok, ok, ok, ok, None, None, 1 << 40, None) == -5
+    r = lib.hdla_param_recurrent_fwd
+    assert r(ctypes.byref(d), ok, ok, ok, None, ok, 0, None, ok, None, None) == -1                    # beta is required
+    assert r(ctypes.byref(d), ok, ok, ok, ok, None, 0, None, ok, None, None) == -1
+    assert r(ctypes.byref(d), ok, ok, ok, ok, ok, 0, bad, ok, None, None) == -6
+    assert r(ctypes.byref(_dims(V=96)), ok, ok, ok, ok, ok, 0, None, ok, None, None) == -2
 
 
 def test_parameterised_python_entry_validates_and_needs_a_gpu():
-    from hdla_hip import chunk_hdla_delta_rule, parameterize_a_b
+    from hdla_hip import chunk_hdla_delta_rule, fused_recurrent_hdla_delta_rule, parameterize_a_b
     x = make_inputs(3, 2, 32, 2, 64, 64)
     q, k, v, gk = [t.bfloat16() for t in (x.q, x.k, x.v, x.gk)]
     beta = torch.rand(2, 32, 2, 1).bfloat16()
@@ -116,6 +121,12 @@ def test_parameterised_python_entry_validates_and_needs_a_gpu():
         chunk_hdla_delta_rule(q, k[:, :5], v, beta, gk)
     with pytest.raises(_lib.HdlaError):
         chunk_hdla_delta_rule(q, k, v, beta, gk)                      # CPU tensors: no fallback
+    with pytest.raises(ValueError):
+        fused_recurrent_hdla_delta_rule(q, k, v, beta[:, :5], gk)
+    with pytest.raises(ValueError, match="batch size is expected to be 1"):
+        fused_recurrent_hdla_delta_rule(q, k, v, beta, gk, cu_seqlens=torch.tensor([0, 16, 32]))
+    with pytest.raises(_lib.HdlaError):
+        fused_recurrent_hdla_delta_rule(q, k, v, beta, gk)
     a, b = parameterize_a_b(beta.float(), k.float(), gk.float())       # the reference's helper, with its return
     assert a.shape == (2, 64, 2, 64) and b.shape == a.shape
     assert torch.equal(b[:, 1::2], k.float()) and torch.allclose(a[:, 0::2], -beta.float() * k.float())
