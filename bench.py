@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the HDLA rank-2 DPLR delta-rule hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload train|fwd|varlen|decode|copy|hdla|hdla_decode] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload train|fwd|varlen|decode|copy|hdla|hdla_decode|norm] [--no-cpu-baseline]
 
 Default workload ("train") is the headline configuration: chunked forward + backward at B=4, T=2048, H=16,
 K=V=64, bf16 inputs, fp32 state, random fp32 initial state, upstream gradients do and dht (configuration 2).
@@ -35,7 +35,7 @@ def _args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="train", choices=["train", "fwd", "varlen", "decode", "copy", "hdla", "hdla_decode"])
+    ap.add_argument("--workload", default="train", choices=["train", "fwd", "varlen", "decode", "copy", "hdla", "hdla_decode", "norm"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
 
@@ -208,6 +208,95 @@ def main():
             mixes[f"{nr}:{nw}"] = round((nr + nw) * n / sec / 1e9)
         print(json.dumps({"metric": "copy calibration", "bytes_read_per_launch": n, "bytes_written_per_launch": n,
                           "ms_per_step": sec * 1e3, "GB/s": 2 * n / sec / 1e9, "GB/s_by_read_write_mix": mixes}))
+        return
+    if wl == "norm":
+        # The gated RMS norm the HDLA layer applies to the operator's output (hdla_custom.py:341-345), forward +
+        # backward, on the layer's shape for configuration 2 (B*T = 8192 rows of H*V = 1024 channels, bf16; the five
+        # tensors of the backward pass are 80 MiB together and stay in the last-level cache) and on 32x the rows,
+        # which is what HBM sees; the roofline entry is the backward kernel on the large shape.
+        from hdla_hip.normalize import normalize_fn
+        g = torch.Generator().manual_seed(0)
+        out = {}
+        for name, rows in (("config2", 8192), ("hbm", 262144)):
+            D = 1024
+            x = torch.randn(rows, D, generator=g).bfloat16().to(dev).requires_grad_()
+            gate = torch.randn(rows, D, generator=g).bfloat16().to(dev).requires_grad_()
+            w = torch.ones(D, device=dev, requires_grad=True)
+            do = torch.randn(rows, D, generator=g).bfloat16().to(dev)
+            res = {}
+
+            def fwd():
+                res["o"] = normalize_fn(x, w, gate=gate, gate_pos="pre", c=D ** 0.5, eps=1e-5)
+
+            def bwd():
+                torch.autograd.grad(res["o"], [x, gate, w], do, retain_graph=True)
+
+            def both():
+                fwd()
+                torch.autograd.grad(res["o"], [x, gate, w], do)
+            sec = time_steps(both, args.steps, args.warmup)
+            # the two passes by themselves: C entry points on preallocated tensors, events on the launch stream
+            import ctypes
+            from hdla_hip import _lib
+            lib = _lib.load()
+            dims = _lib.HdlaNormDims(rows, 1, D, 0, 1, 1, D ** 0.5, 1e-5)
+            o, dx, dg = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+            dw = torch.empty(D, dtype=torch.float32, device=dev)
+            nws = lib.hdla_normalize_workspace_bytes(ctypes.byref(dims))
+            ws = torch.empty(nws, dtype=torch.uint8, device=dev)
+            P, stream = _lib.ptr, _lib.current_stream(dev)
+
+            def fwd_c():
+                _lib.check(lib.hdla_normalize_fwd(ctypes.byref(dims), P(x), P(w), P(gate), P(o), stream), "hdla_normalize_fwd")
+
+            def bwd_c():
+                _lib.check(lib.hdla_normalize_bwd(ctypes.byref(dims), P(x), P(w), P(gate), P(do), P(dx), P(dg), P(dw),
+                                                  P(ws), nws, stream), "hdla_normalize_bwd")
+            ms = {}
+            for nm, fn in (("fwd", fwd_c), ("bwd", bwd_c)):
+                fn()
+                evs = []
+                for _ in range(args.steps):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(); fn(); e1.record()
+                    evs.append((e0, e1))
+                torch.cuda.synchronize()
+                ms[nm] = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+            del o, dx, dg, ws
+            nb = {"fwd": 3 * rows * D * 2 + D * 4, "bwd": 5 * rows * D * 2 + D * 8}
+            out[name] = {"rows": rows, "channels": D, "ms_per_step": sec * 1e3, "rows/s": rows / sec,
+                         "fwd_ms": ms["fwd"], "bwd_ms": ms["bwd"], "fwd_bytes": nb["fwd"], "bwd_bytes": nb["bwd"],
+                         "fwd_GB/s": nb["fwd"] / ms["fwd"] / 1e6, "bwd_GB/s": nb["bwd"] / ms["bwd"] / 1e6}
+            del x, gate, do, res
+        big = out["hbm"]
+        line = {"metric": "gated rms norm fwd+bwd rows/s", "value": out["config2"]["rows/s"], "unit": "rows/s", "n_gpus": 1,
+                "steps": args.steps, "warmup": args.warmup, "ms_per_step": out["config2"]["ms_per_step"],
+                "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+                "config": {"workload": "gated RMS norm of the layer at configuration 2's shape: 8192 rows x 1024 channels, "
+                                       "bf16 tensors, fp32 weight, gate before the norm; forward + backward"},
+                "shapes": out,
+                "roofline": {"bound": "hbm", "kernel": "normalize_bwd_kernel (+ normalize_dw_kernel), 262144 rows",
+                             "achieved": big["bwd_GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": big["bwd_GB/s"] / HBM_PEAK_GBS, "traffic": None,
+                             "bytes_per_launch": big["bwd_bytes"], "ms_per_launch": big["bwd_ms"],
+                             "note": "one call of hdla_normalize_bwd: the backward kernel and the small weight-gradient reduction after it"}}
+        if not args.no_cpu_baseline:
+            from oracle import normalize_oracle as NO
+            cores = os.cpu_count() or 1
+            torch.set_num_threads(cores)
+            rows = 8192
+            xc = torch.randn(rows, 1024, generator=g).bfloat16().float().requires_grad_()
+            gc_ = torch.randn(rows, 1024, generator=g).bfloat16().float().requires_grad_()
+            wc = torch.ones(1024, requires_grad=True)
+            t0 = time.perf_counter()
+            reps = 5
+            for _ in range(reps):
+                o = NO.rms_norm_fused_gate(xc, gc_, wc, dtype=torch.float32)
+                torch.autograd.grad(o, [xc, gc_, wc], torch.ones_like(o))
+            dtc = (time.perf_counter() - t0) / reps
+            line["cpu_baseline"] = {"value": rows / dtc, "unit": "rows/s", "cores": cores, "kind": "port",
+                                    "sample": f"{reps} runs of the config-2 shape (8192 x 1024), fp32 torch oracle fwd + autograd bwd"}
+        print(json.dumps(line))
         return
     cfg = {"train": 2, "fwd": 1, "varlen": 3, "decode": 4, "hdla": 2, "hdla_decode": 4}[wl]
     B, T, H, K, V = CONFIG_SHAPES[cfg]

@@ -29,6 +29,13 @@ class HdlaWsLayout(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int64) for n in _names]
 
 
+class HdlaNormDims(ctypes.Structure):
+    """struct hdla_norm_dims of include/hdla_hip.h."""
+    _fields_ = [("rows", ctypes.c_int64), ("G", ctypes.c_int32), ("E", ctypes.c_int32), ("dtype", ctypes.c_int32),
+                ("weight_dtype", ctypes.c_int32), ("gate_pos", ctypes.c_int32), ("c", ctypes.c_float),
+                ("eps", ctypes.c_float)]
+
+
 class HdlaError(RuntimeError):
     pass
 
@@ -73,6 +80,13 @@ def load():
     lib.hdla_recurrent_fwd.argtypes = [F] + [P] * 6 + [ctypes.c_int] + [P] * 4
     lib.hdla_param_recurrent_fwd.restype = ctypes.c_int
     lib.hdla_param_recurrent_fwd.argtypes = [F] + [P] * 5 + [ctypes.c_int] + [P] * 4
+    NF = ctypes.POINTER(HdlaNormDims)
+    lib.hdla_normalize_workspace_bytes.restype = ctypes.c_size_t
+    lib.hdla_normalize_workspace_bytes.argtypes = [NF]
+    lib.hdla_normalize_fwd.restype = ctypes.c_int
+    lib.hdla_normalize_fwd.argtypes = [NF] + [P] * 5
+    lib.hdla_normalize_bwd.restype = ctypes.c_int
+    lib.hdla_normalize_bwd.argtypes = [NF] + [P] * 8 + [ctypes.c_size_t, P]
     _lib = lib
     return lib
 

@@ -140,6 +140,35 @@ int hdla_recurrent_fwd(const hdla_dims* dims, const void* q, const void* k, cons
 int hdla_param_recurrent_fwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* beta,
                              const void* gk, int reverse, const float* h0, void* o, float* ht, void* stream);
 
+/* Fused normalisation with an optional sigmoid gate, the operator the HDLA layer applies around the attention
+ * operator: _normalize_fwd / _normalize_bwd, HRDPLR/normalizations/normalize/normalize/normalize_triton.py:21-253
+ * (NormalizeTriton.forward :256-352, .backward :354-449) for use_mean = False, no bias, no residual.
+ * A tensor is `rows` rows of G groups of E channels, contiguous; per group
+ *     x' = x * sigmoid(gate) (gate_pos 1),  sigma = sqrt(sum x'^2 / E + eps),
+ *     o = (c / sqrt(E)) * x' / sigma * weight  [* sigmoid(gate), gate_pos 2].
+ * rms norm over a row: G = 1, c = sqrt(E) (normalizations/utils.py:35-39); group rms norm: c = sqrt(E), G groups
+ * (:47-50); l2_norm: G = 1, c = 1, no weight (normalizations/l2_norm.py:4-14).
+ * E must be a multiple of 16 bytes' worth of elements and at most 4096 (bf16) / 2048 (fp32). */
+typedef struct hdla_norm_dims {
+    int64_t rows;              /* product of the leading dimensions */
+    int32_t G, E;              /* groups per row, channels per group */
+    int32_t dtype;             /* x, gate, o, do, dx, dgate */
+    int32_t weight_dtype;      /* weight [G*E] (ignored when weight is NULL) */
+    int32_t gate_pos;          /* 0 = no gate, 1 = before the norm ("pre"), 2 = after it ("post") */
+    float c, eps;
+} hdla_norm_dims;
+
+/* weight and gate may be NULL (gate only with gate_pos 0). */
+int hdla_normalize_fwd(const hdla_norm_dims* dims, const void* x, const void* weight, const void* gate, void* o,
+                       void* stream);
+/* Backward pass; sigma is recomputed.  dw: fp32 [G*E], required iff weight is given; it is summed over rows in a
+ * fixed order through `workspace` (hdla_normalize_workspace_bytes() bytes, 16-byte aligned; not needed without a
+ * weight).  dgate is required iff gate_pos != 0. */
+int hdla_normalize_bwd(const hdla_norm_dims* dims, const void* x, const void* weight, const void* gate,
+                       const void* d_o, void* dx, void* dgate, float* dw, void* workspace, size_t workspace_bytes,
+                       void* stream);
+size_t hdla_normalize_workspace_bytes(const hdla_norm_dims* dims);
+
 /* Measurement aid; it has no counterpart in the reference.  One launch of a kernel that reads `n_read` (0..3)
  * buffers and writes `n_write` (0..2) buffers of `bytes` bytes each (a multiple of 16; every pointer 16-byte
  * aligned) and does nothing else.  Supported mixes (reads:writes): 1:0, 0:1, 1:1, 2:1, 3:1, 1:2; others return

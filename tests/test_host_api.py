@@ -31,7 +31,8 @@ def test_library_exports_every_declared_symbol():
     names = set(re.findall(r"\b(hdla_[a-z_]+)\s*\(", header))
     assert {"hdla_version", "hdla_strerror", "hdla_workspace_bytes", "hdla_workspace_layout", "hdla_chunk_fwd",
             "hdla_chunk_bwd", "hdla_chunk_stages", "hdla_recurrent_fwd", "hdla_param_chunk_fwd", "hdla_param_chunk_bwd",
-            "hdla_param_recurrent_fwd", "hdla_calib_stream"} <= names
+            "hdla_param_recurrent_fwd", "hdla_calib_stream", "hdla_normalize_fwd", "hdla_normalize_bwd",
+            "hdla_normalize_workspace_bytes"} <= names
     for n in names:
         assert hasattr(lib, n), n
     assert lib.hdla_version() == 100
@@ -108,6 +109,47 @@ def test_parameterised_entry_points_check_their_arguments():
     assert r(ctypes.byref(d), ok, ok, ok, ok, None, 0, None, ok, None, None) == -1
     assert r(ctypes.byref(d), ok, ok, ok, ok, ok, 0, bad, ok, None, None) == -6
     assert r(ctypes.byref(_dims(V=96)), ok, ok, ok, ok, ok, 0, None, ok, None, None) == -2
+
+
+def test_normalize_entry_points_check_their_arguments():
+    lib = _lib.load()
+    ok, bad = ctypes.c_void_p(4096), ctypes.c_void_p(4096 + 8)
+    nd = lambda **kw: _lib.HdlaNormDims(**{**dict(rows=8, G=1, E=1024, dtype=0, weight_dtype=1, gate_pos=1, c=32.0,
+                                                  eps=1e-5), **kw})
+    f, b, wsb = lib.hdla_normalize_fwd, lib.hdla_normalize_bwd, lib.hdla_normalize_workspace_bytes
+    assert f(ctypes.byref(nd()), None, ok, ok, ok, None) == -1
+    assert f(ctypes.byref(nd()), ok, ok, None, ok, None) == -1                       # gate_pos 1 needs a gate
+    assert f(ctypes.byref(nd()), ok, ok, bad, ok, None) == -6
+    assert f(ctypes.byref(nd(E=1020)), ok, ok, ok, ok, None) == -2                   # groups must start on 16 bytes
+    assert f(ctypes.byref(nd(E=8192)), ok, ok, ok, ok, None) == -2                   # longer than one wavefront holds
+    assert f(ctypes.byref(nd(dtype=3)), ok, ok, ok, ok, None) == -4
+    assert f(ctypes.byref(nd(gate_pos=3)), ok, ok, ok, ok, None) == -2
+    assert f(ctypes.byref(nd(rows=0)), None, None, None, None, None) == 0            # nothing to do
+    need = wsb(ctypes.byref(nd()))
+    assert need > 0 and need % (1024 * 4) == 0 and wsb(ctypes.byref(nd(E=1020))) == 0
+    assert wsb(ctypes.byref(nd(rows=1 << 20))) <= 8192 * 4 * 1024 * 4                # bounded however many rows
+    assert b(ctypes.byref(nd()), ok, ok, ok, ok, ok, ok, None, ok, need, None) == -1           # weight without dw
+    assert b(ctypes.byref(nd()), ok, ok, ok, ok, ok, None, ok, ok, need, None) == -1           # gate without dgate
+    assert b(ctypes.byref(nd()), ok, ok, ok, ok, ok, ok, ok, ok, need - 1, None) == -5
+    assert b(ctypes.byref(nd()), ok, ok, ok, ok, ok, ok, ok, None, need, None) == -5
+
+
+def test_normalize_python_entry_validates_and_needs_a_gpu():
+    from hdla_hip import normalize as NZ
+    x = torch.randn(4, 64)
+    with pytest.raises(NotImplementedError):
+        NZ.normalize_fn(x, use_mean=True)
+    with pytest.raises(NotImplementedError):
+        NZ.normalize_fn(x, bias=torch.zeros(64))
+    with pytest.raises(NotImplementedError):
+        NZ.normalize_fn(x, gate=x, gate_act="silu")
+    with pytest.raises(ValueError):
+        NZ.normalize_fn(x, gate=x[:2])
+    with pytest.raises(AssertionError):
+        NZ.normalize_fn(x, num_groups=3)
+    with pytest.raises(_lib.HdlaError):
+        NZ.l2_norm(x)                                                   # CPU tensor: no fallback
+    assert isinstance(NZ.get_norm_fn("rmsnorm_fused_gate")(64, bias=False, num_groups=2), NZ.RMSNormFusedGate)
 
 
 def test_parameterised_python_entry_validates_and_needs_a_gpu():
