@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the HDLA rank-2 DPLR delta-rule hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload train|fwd|varlen|decode|copy|hdla|hdla_decode|norm] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload train|fwd|varlen|decode|copy|hdla|hdla_decode|norm|layer] [--no-cpu-baseline]
 
 Default workload ("train") is the headline configuration: chunked forward + backward at B=4, T=2048, H=16,
 K=V=64, bf16 inputs, fp32 state, random fp32 initial state, upstream gradients do and dht (configuration 2).
@@ -35,7 +35,7 @@ def _args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="train", choices=["train", "fwd", "varlen", "decode", "copy", "hdla", "hdla_decode", "norm"])
+    ap.add_argument("--workload", default="train", choices=["train", "fwd", "varlen", "decode", "copy", "hdla", "hdla_decode", "norm", "layer"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
 
@@ -208,6 +208,35 @@ def main():
             mixes[f"{nr}:{nw}"] = round((nr + nw) * n / sec / 1e9)
         print(json.dumps({"metric": "copy calibration", "bytes_read_per_launch": n, "bytes_written_per_launch": n,
                           "ms_per_step": sec * 1e3, "GB/s": 2 * n / sec / 1e9, "GB/s_by_read_write_mix": mixes}))
+        return
+    if wl == "layer":
+        # The whole HDLA token mixer (projections, activations, normalisations, the operator, output gate and
+        # projection) on the layer shape of configuration 2: embed_dim = H*K = 1024, 16 heads, B=4, T=2048, bf16
+        # parameters; forward + backward (gradients of x and of every parameter).  Whole-step rates only: the GEMMs are
+        # the BLAS library's, and the step is partly bound by the host issuing ~90 small launches.
+        from hdla_hip.layer import HDLA_Custom
+        B, T, H, D = 4, 2048, 16, 64
+        d = H * D
+        torch.manual_seed(0)
+        x = torch.randn(B, T, d, device=dev, dtype=torch.bfloat16, requires_grad=True)
+        do = torch.randn(B, T, d, device=dev, dtype=torch.bfloat16)
+        out = {}
+        for name, kw in (("fused", {}), ("plain_route", {"fuse_ab": False})):
+            m = HDLA_Custom(d, H, token_mixer_init_type=2, rescale_type=0, **kw).to(dev).bfloat16().train()
+
+            def step():
+                y, _ = m(x)
+                y.backward(do)
+            out[name] = time_steps(step, args.steps, args.warmup)
+        print(json.dumps({"metric": "HDLA layer fwd+bwd tokens/s", "value": B * T / out["fused"], "unit": "tokens/s",
+                          "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": out["fused"] * 1e3,
+                          "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+                          "data": "synthetic",
+                          "config": {"workload": "HDLA_Custom layer, embed_dim 1024, 16 heads of 64, B=4 T=2048, bf16; "
+                                                 "forward + backward", "global_batch": B, "seq_len": T},
+                          "plain_route": {"what": "same layer with fuse_ab=False: torch parameterize_a_b + the plain operator",
+                                          "ms_per_step": out["plain_route"] * 1e3, "value": B * T / out["plain_route"]},
+                          "roofline": None}))
         return
     if wl == "norm":
         # The gated RMS norm the HDLA layer applies to the operator's output (hdla_custom.py:341-345), forward +

@@ -6,6 +6,7 @@ fused normalisation the layer applies around it (HRDPLR/normalizations/normalize
 """
 from .chunk import ChunkDPLRDeltaRuleFunction, chunk_hrdplr_delta_rule
 from .hdla import ChunkHDLAFunction, chunk_hdla_delta_rule, fused_recurrent_hdla_delta_rule, parameterize_a_b
+from .layer import HDLA_Custom, RecurrentCache, get_activation_fn
 from .normalize import (GroupRMSNorm, GroupRMSNormFusedGate, NormalizeFunction, RMSNorm, RMSNormFusedGate, SRMSNorm,
                         get_norm_fn, l2_norm, normalize_fn)
 from .recurrent import FusedRecurrentDPLRDeltaRuleFunction, fused_recurrent_dplr_delta_rule
@@ -28,4 +29,7 @@ __all__ = [
     "GroupRMSNorm",
     "GroupRMSNormFusedGate",
     "NormalizeFunction",
+    "HDLA_Custom",
+    "RecurrentCache",
+    "get_activation_fn",
 ]
