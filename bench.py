@@ -75,14 +75,32 @@ def measured_traffic(workload, kernel_key, K, V):
         return None
     pass_, name = kernel_key.split(".") if "." in kernel_key else ("", kernel_key)
     for k, rec in table.items():
-        if not k.startswith(name + "_kernel<") or f" {K}, {V}" not in k:
+        if not k.startswith(name + "_kernel<"):
             continue
-        if name in ("prep", "scan_fwd"):
-            forward_variant = k.endswith("false>") if name == "prep" else k.endswith("true>")
-            if forward_variant != (pass_ == "fwd"):
-                continue
+        targs = [a.strip() for a in k[k.index("<") + 1:k.rindex(">")].split(",")]
+        # prep<T, GKF32, K, V, BWD, HD>, scan_fwd<T, K, V, NWC, WRITE_O>, scan_pair<T, K, V, NWC>,
+        # chunk_grad<T, GKF32, K, V, HD>, recurrent<T, K, V, BV, HD>
+        kv = targs[2:4] if name in ("prep", "chunk_grad") else targs[1:3]
+        if kv != [str(K), str(V)]:
+            continue
+        if name == "prep" and ((targs[4] == "true") != (pass_ == "bwd") or targs[5:] == ["true"]):
+            continue
+        if name == "scan_fwd" and (targs[4] == "true") != (pass_ == "fwd"):
+            continue
+        if name in ("chunk_grad", "recurrent") and targs[4:] == ["true"]:
+            continue
         return rec["hbm_bytes_per_launch"]
     return None
+
+
+def norm_traffic(rows):
+    """HBM bytes of one backward call of the gated norm at `rows` rows (backward kernel + weight-gradient reduction)
+    from the committed counter summary, or None."""
+    try:
+        table = json.load(open(os.path.join(ROOT, "profiles", "hbm_traffic.json"))).get("norm", {})
+        return sum(table[f"{k}@{rows}rows"]["hbm_bytes_per_launch"] for k in ("normalize_bwd_kernel<bf16, 2>", "normalize_dw_kernel"))
+    except (OSError, ValueError, KeyError):
+        return None
 
 
 def time_steps(fn, steps, warmup):
@@ -224,18 +242,17 @@ def main():
         for name, kw in (("fused", {}), ("plain_route", {"fuse_ab": False})):
             m = HDLA_Custom(d, H, token_mixer_init_type=2, rescale_type=0, **kw).to(dev).bfloat16().train()
 
-            def step():
+            params = [p for p in m.parameters()]
+
+            def grads():
+                # gradients of x and of every parameter, handed over as new tensors (what an optimizer step that
+                # clears gradients with set_to_none sees), not accumulated into existing ones
                 y, _ = m(x)
-                y.backward(do)
-            out[name] = time_steps(step, args.steps, args.warmup)
+                return [y.detach()] + list(torch.autograd.grad(y, [x] + params, do))
+            out[name] = time_steps(grads, args.steps, args.warmup)
             if name == "fused":
                 # the same step as one HIP graph (the library only launches kernels, so it can be captured): removes the
                 # host's share; every replay is checked against the eager step before it is timed
-                params = [p for p in m.parameters()]
-
-                def grads():
-                    y, _ = m(x)
-                    return [y.detach()] + list(torch.autograd.grad(y, [x] + params, do))
                 side = torch.cuda.Stream()
                 side.wait_stream(torch.cuda.current_stream())
                 with torch.cuda.stream(side):
@@ -335,7 +352,7 @@ def main():
                 "shapes": out,
                 "roofline": {"bound": "hbm", "kernel": "normalize_bwd_kernel (+ normalize_dw_kernel), 262144 rows",
                              "achieved": big["bwd_GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                             "frac": big["bwd_GB/s"] / HBM_PEAK_GBS, "traffic": None,
+                             "frac": big["bwd_GB/s"] / HBM_PEAK_GBS, "traffic": norm_traffic(262144),
                              "bytes_per_launch": big["bwd_bytes"], "ms_per_launch": big["bwd_ms"],
                              "note": "one call of hdla_normalize_bwd: the backward kernel and the small weight-gradient reduction after it"}}
         if not args.no_cpu_baseline:
@@ -520,7 +537,7 @@ def main():
                        "global_batch": B, "seq_len": T, "heads": H, "K": K, "V": V, "chunk": 16},
                roofline={"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS,
                          "unit": "GB/s", "frac": dom["frac_hbm"],
-                         "traffic": measured_traffic("train", dom["kernel"], K, V) if wl == "train" else None,
+                         "traffic": measured_traffic(wl, dom["kernel"], K, V),
                          "bytes_per_launch": dom["bytes"], "ms_per_launch": dom["ms"]},
                kernels=klist,
                whole_step={"compulsory_bytes": whole, "GB/s": whole / sec / 1e9, "frac_hbm": whole / sec / 1e9 / HBM_PEAK_GBS,

@@ -28,6 +28,7 @@ struct NormArgs {
     long long nsg;             // wavefront passes: ceil(nslot / (64 >> lpr_log2))
     int G, E, lpr_log2, w_f32, gate_pos;
     int wg_reduce;             // the four wavefronts of a workgroup meet the same weight columns: one partial row set
+    int wg_row;                // long groups: the four wavefronts of a workgroup share one group, 256 lanes across it
     float cn, inv_e, eps;      // c / sqrt(E), 1 / E
 };
 
@@ -75,25 +76,51 @@ template <int N> __device__ __forceinline__ void ld_weight(const void* w, int w_
 
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.f / (1.f + __expf(-x)); }
 
-// Where a lane stands: lane sl of the LPR lanes across one group, group position rw of the 64/LPR groups of a pass.
+// Where a lane stands: lane sl of the LPR lanes across one group, group position rw of the 64/LPR groups of a pass;
+// `wave` counts passes' owners (wavefronts, or workgroups when a workgroup shares one long group).
 struct NormLane {
-    int lpr, rpw, sl, rw;
+    int lpr, rpw, sl, rw, wg_row;
     long long wave, nwave;
     __device__ __forceinline__ explicit NormLane(const NormArgs& p) {
         const int lane = threadIdx.x & 63;
-        lpr = 1 << p.lpr_log2;
-        rpw = 64 >> p.lpr_log2;
-        sl = lane & (lpr - 1);
-        rw = lane >> p.lpr_log2;
-        nwave = (long long)gridDim.x * 4;
-        wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+        wg_row = p.wg_row;
+        if (wg_row) {
+            lpr = 256; rpw = 1; sl = threadIdx.x; rw = 0;
+            nwave = gridDim.x;
+            wave = blockIdx.x;
+        } else {
+            lpr = 1 << p.lpr_log2;
+            rpw = 64 >> p.lpr_log2;
+            sl = lane & (lpr - 1);
+            rw = lane >> p.lpr_log2;
+            nwave = (long long)gridDim.x * 4;
+            wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+        }
     }
 };
+
+// Sums of a and b over the lanes of one group, on all of them.  Across the wavefronts of a workgroup the partial
+// sums go through `sred` ([2][4][2] floats, alternating halves, so one barrier per call is enough); every thread of
+// the workgroup makes the same calls.
+__device__ __forceinline__ void group_sum(const NormLane& L, float& a, float& b, float* sred, int& buf) {
+    const int width = L.wg_row ? 64 : L.lpr;
+    for (int o = 1; o < width; o <<= 1) { a += __shfl_xor(a, o); b += __shfl_xor(b, o); }
+    if (L.wg_row) {
+        float* s = sred + buf * 8;
+        if ((threadIdx.x & 63) == 0) { s[2 * (threadIdx.x >> 6)] = a; s[2 * (threadIdx.x >> 6) + 1] = b; }
+        __syncthreads();
+        a = (s[0] + s[2]) + (s[4] + s[6]);
+        b = (s[1] + s[3]) + (s[5] + s[7]);
+        buf ^= 1;
+    }
+}
 
 template <typename T, int NV>
 __global__ __launch_bounds__(256) void normalize_fwd_kernel(NormArgs p) {
     constexpr int N = Piece<T>::N;
     const NormLane L(p);
+    __shared__ float sred[16];
+    int buf = 0;
     const bool pre = p.gate_pos == 1, post = p.gate_pos == 2;
     const int E = p.E;
     // the launch makes nwave * rpw a multiple of G: the group index of a lane's slots never changes
@@ -132,7 +159,8 @@ __global__ __launch_bounds__(256) void normalize_fwd_kernel(NormArgs p) {
                 if (pre) x[i][j] *= gs[i][j];
                 ss += x[i][j] * x[i][j];
             }
-        for (int o = 1; o < L.lpr; o <<= 1) ss += __shfl_xor(ss, o);
+        float unused = 0.f;
+        group_sum(L, ss, unused, sred, buf);
         const float rs = p.cn / sqrtf(ss * p.inv_e + p.eps);
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
@@ -152,6 +180,8 @@ template <typename T, int NV>
 __global__ __launch_bounds__(256) void normalize_bwd_kernel(NormArgs p) {
     constexpr int N = Piece<T>::N;
     const NormLane L(p);
+    __shared__ float sred[16];
+    int buf = 0;
     const bool pre = p.gate_pos == 1, post = p.gate_pos == 2, has_w = p.weight != nullptr;
     const int E = p.E;
     const int g = (int)((L.wave * L.rpw + L.rw) % p.G);
@@ -196,7 +226,7 @@ __global__ __launch_bounds__(256) void normalize_bwd_kernel(NormArgs p) {
                 ss += x[i][j] * x[i][j];
                 sd += x[i][j] * dr[i][j] * w[i][j];
             }
-        for (int o = 1; o < L.lpr; o <<= 1) { ss += __shfl_xor(ss, o); sd += __shfl_xor(sd, o); }
+        group_sum(L, ss, sd, sred, buf);
         const float inv = 1.f / sqrtf(ss * p.inv_e + p.eps);          // 1 / sigma
         const float proj = sd * inv * p.inv_e;                         // sum(r * dr * w) / E, r = x / sigma
 #pragma unroll
@@ -295,9 +325,9 @@ __global__ __launch_bounds__(256) void normalize_dw_kernel(const float* __restri
 
 // Launch shape shared by both passes and by the workspace size.
 struct NormCfg {
-    int n, nv, lpr_log2, rpw, wg_reduce;
+    int n, nv, lpr_log2, rpw, wg_reduce, wg_row;
     long long nslot, nsg, nwg;
-    long long partial_rows() const { return nwg * (wg_reduce ? 1 : 4) * rpw; }
+    long long partial_rows() const { return wg_row ? nwg : nwg * (wg_reduce ? 1 : 4) * rpw; }
 };
 
 static long long gcd_ll(long long a, long long b) { while (b) { const long long t = a % b; a = b; b = t; } return a; }
@@ -311,24 +341,32 @@ static int norm_config(const hdla_norm_dims* d, bool bwd, NormCfg& c) {
     c.n = d->dtype == HDLA_BF16 ? 8 : 4;
     if (d->E % c.n) return HDLA_ERR_SHAPE;                      // groups start on 16-byte boundaries
     const int pieces = d->E / c.n;
-    if (pieces > 64 * 8) return HDLA_ERR_SHAPE;                 // a group lives in one wavefront's registers
-    c.nv = 1;
-    while (c.nv * 64 < pieces) c.nv *= 2;
-    const int per = (pieces + c.nv - 1) / c.nv;
-    c.lpr_log2 = 0;
-    while ((1 << c.lpr_log2) < per) ++c.lpr_log2;
-    c.rpw = 64 >> c.lpr_log2;
+    if (pieces > 256 * 8) return HDLA_ERR_SHAPE;                // a group lives in one workgroup's registers
     if (d->rows > (1LL << 40) / d->G) return HDLA_ERR_SHAPE;
     c.nslot = d->rows * d->G;
-    c.nsg = (c.nslot + c.rpw - 1) / c.rpw;
-    c.wg_reduce = c.rpw % d->G == 0;
+    c.wg_row = pieces > 64 * 8;
+    if (c.wg_row) {
+        // long groups: one per workgroup pass, 256 lanes across it
+        c.nv = pieces <= 256 * 4 ? 4 : 8;
+        c.lpr_log2 = 8; c.rpw = 1; c.wg_reduce = 0;
+        c.nsg = c.nslot;
+    } else {
+        c.nv = 1;
+        while (c.nv * 64 < pieces) c.nv *= 2;
+        const int per = (pieces + c.nv - 1) / c.nv;
+        c.lpr_log2 = 0;
+        while ((1 << c.lpr_log2) < per) ++c.lpr_log2;
+        c.rpw = 64 >> c.lpr_log2;
+        c.nsg = (c.nslot + c.rpw - 1) / c.rpw;
+        c.wg_reduce = c.rpw % d->G == 0;
+    }
     // a few passes per wavefront to amortise the weight loads, enough workgroups to fill the chip, and, backward, a
     // bound on the partial rows of the weight gradient; then a multiple of what keeps a lane on one weight column
-    const long long per_wave = 4, cap = bwd ? 1024 : 8192;
-    long long nwg = (c.nsg + 4 * per_wave - 1) / (4 * per_wave);
+    const long long per_wave = 4, cap = bwd ? 1024 : 8192, owners = c.wg_row ? 1 : 4;
+    long long nwg = (c.nsg + owners * per_wave - 1) / (owners * per_wave);
     if (nwg < 1) nwg = 1;
     if (nwg > cap) nwg = cap;
-    const long long m = d->G / gcd_ll(d->G, 4LL * c.rpw);
+    const long long m = d->G / gcd_ll(d->G, owners * c.rpw);
     if (m > 65536) return HDLA_ERR_SHAPE;
     c.nwg = (nwg + m - 1) / m * m;
     return HDLA_OK;
@@ -356,7 +394,7 @@ static hipError_t launch_norm(const NormArgs& a, const NormCfg& c, bool bwd, hip
 static NormArgs norm_args(const hdla_norm_dims* d, const NormCfg& c) {
     NormArgs a{};
     a.nslot = c.nslot; a.nsg = c.nsg; a.G = d->G; a.E = d->E; a.lpr_log2 = c.lpr_log2;
-    a.w_f32 = d->weight_dtype == HDLA_FP32; a.gate_pos = d->gate_pos; a.wg_reduce = c.wg_reduce;
+    a.w_f32 = d->weight_dtype == HDLA_FP32; a.gate_pos = d->gate_pos; a.wg_reduce = c.wg_reduce; a.wg_row = c.wg_row;
     a.cn = d->c / sqrtf((float)d->E); a.inv_e = 1.f / (float)d->E; a.eps = d->eps;
     return a;
 }

@@ -148,7 +148,7 @@ int hdla_param_recurrent_fwd(const hdla_dims* dims, const void* q, const void* k
  *     o = (c / sqrt(E)) * x' / sigma * weight  [* sigmoid(gate), gate_pos 2].
  * rms norm over a row: G = 1, c = sqrt(E) (normalizations/utils.py:35-39); group rms norm: c = sqrt(E), G groups
  * (:47-50); l2_norm: G = 1, c = 1, no weight (normalizations/l2_norm.py:4-14).
- * E must be a multiple of 16 bytes' worth of elements and at most 4096 (bf16) / 2048 (fp32). */
+ * E must be a multiple of 16 bytes' worth of elements and at most 16384 (bf16) / 8192 (fp32). */
 typedef struct hdla_norm_dims {
     int64_t rows;              /* product of the leading dimensions */
     int32_t G, E;              /* groups per row, channels per group */

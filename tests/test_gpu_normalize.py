@@ -52,7 +52,10 @@ CASES = [
     # dtype, shape, G, weight, gate_pos, c, eps
     (torch.bfloat16, (4, 64, 1024), 1, True, "pre", 32.0, 1e-5),       # the layer's gated RMS norm, 16 heads x 64
     (torch.bfloat16, (2, 33, 2048), 1, True, "post", 2048 ** 0.5, 1e-5),
-    (torch.bfloat16, (3, 17, 4096), 1, True, "pre", 64.0, 1e-5),       # largest bf16 row
+    (torch.bfloat16, (3, 17, 4096), 1, True, "pre", 64.0, 1e-5),       # largest row one wavefront holds
+    (torch.bfloat16, (2, 9, 8192), 1, True, "pre", 8192 ** 0.5, 1e-5),  # a workgroup per row, four pieces a lane
+    (torch.bfloat16, (11, 16384), 1, True, "post", 128.0, 1e-5),       # largest bf16 row
+    (torch.bfloat16, (6, 10240), 2, True, "pre", 5120 ** 0.5, 1e-5),   # two long groups a row, ragged over 256 lanes
     (torch.bfloat16, (2, 50, 16, 64), 1, False, None, 1.0, 1e-5),      # l2_norm of a [B,T,H,K] tensor
     (torch.bfloat16, (2, 50, 3, 128), 1, False, None, 1.0, 1e-5),
     (torch.bfloat16, (1, 77, 768), 12, True, "pre", 8.0, 1e-5),        # group rms norm, 12 groups of 64
@@ -63,6 +66,8 @@ CASES = [
     (torch.float32, (3, 40, 4, 64), 1, False, None, 1.0, 1e-5),
     (torch.float32, (2, 19, 512), 8, True, "pre", 8.0, 1e-5),
     (torch.float32, (7, 36), 3, True, None, 12 ** 0.5, 1e-5),
+    (torch.float32, (5, 3, 4096), 1, True, "pre", 64.0, 1e-5),
+    (torch.float32, (4, 8192), 1, False, None, 1.0, 1e-5),
 ]
 
 

@@ -121,7 +121,7 @@ def test_normalize_entry_points_check_their_arguments():
     assert f(ctypes.byref(nd()), ok, ok, None, ok, None) == -1                       # gate_pos 1 needs a gate
     assert f(ctypes.byref(nd()), ok, ok, bad, ok, None) == -6
     assert f(ctypes.byref(nd(E=1020)), ok, ok, ok, ok, None) == -2                   # groups must start on 16 bytes
-    assert f(ctypes.byref(nd(E=8192)), ok, ok, ok, ok, None) == -2                   # longer than one wavefront holds
+    assert f(ctypes.byref(nd(E=32768)), ok, ok, ok, ok, None) == -2                  # longer than one workgroup holds
     assert f(ctypes.byref(nd(dtype=3)), ok, ok, ok, ok, None) == -4
     assert f(ctypes.byref(nd(gate_pos=3)), ok, ok, ok, ok, None) == -2
     assert f(ctypes.byref(nd(rows=0)), None, None, None, None, None) == 0            # nothing to do
