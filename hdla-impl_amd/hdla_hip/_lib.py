@@ -36,6 +36,13 @@ class HdlaNormDims(ctypes.Structure):
                 ("eps", ctypes.c_float)]
 
 
+class HdlaPreDims(ctypes.Structure):
+    """struct hdla_pre_dims of include/hdla_hip.h."""
+    _fields_ = [("rows", ctypes.c_int64)] + [(n, ctypes.c_int32) for n in (
+        "H", "D", "dtype", "ldy", "col_q", "col_k", "col_v", "col_beta", "norm_q", "norm_k", "norm_v")] + [
+        ("beta_scale", ctypes.c_float), ("eps", ctypes.c_float)]
+
+
 class HdlaError(RuntimeError):
     pass
 
@@ -87,6 +94,15 @@ def load():
     lib.hdla_normalize_fwd.argtypes = [NF] + [P] * 5
     lib.hdla_normalize_bwd.restype = ctypes.c_int
     lib.hdla_normalize_bwd.argtypes = [NF] + [P] * 8 + [ctypes.c_size_t, P]
+    PF = ctypes.POINTER(HdlaPreDims)
+    lib.hdla_layer_pre_fwd.restype = ctypes.c_int
+    lib.hdla_layer_pre_fwd.argtypes = [PF] + [P] * 6
+    lib.hdla_layer_pre_bwd.restype = ctypes.c_int
+    lib.hdla_layer_pre_bwd.argtypes = [PF] + [P] * 7
+    lib.hdla_logsigmoid_fwd.restype = ctypes.c_int
+    lib.hdla_logsigmoid_fwd.argtypes = [ctypes.c_int, ctypes.c_int64, P, P, P]
+    lib.hdla_logsigmoid_bwd.restype = ctypes.c_int
+    lib.hdla_logsigmoid_bwd.argtypes = [ctypes.c_int, ctypes.c_int64, P, P, P, P]
     _lib = lib
     return lib
 

@@ -5,8 +5,10 @@ Same constructor arguments, parameter names (so a reference ``state_dict`` loads
 
 * projections: the BLAS library through torch, as in the reference (hdla_custom.py:206-213), but with everything
   that multiplies x gathered into one GEMM
-* per-head l2 normalisation of q, k, v and the gated RMS norm after the operator: ``hdla_hip.normalize``
-  (hdla_custom.py:247-251, 341-345)
+* activations, head split, per-head l2 normalisation of q, k, v, beta and the log decay: two kernels each way
+  (``hdla_hip.layer_pre``; hdla_custom.py:214-251) in the default configuration (silu activations, one block);
+  otherwise, or with ``fuse_pre=False``, torch's elementwise operators and ``hdla_hip.normalize.l2_norm``
+* the gated RMS norm after the operator: ``hdla_hip.normalize`` (hdla_custom.py:341-345)
 * the recurrence: ``chunk_hdla_delta_rule`` / ``fused_recurrent_hdla_delta_rule``, which form a and b from
   (beta, k, log_f) inside the kernels; the reference calls ``parameterize_a_b`` first (hdla_custom.py:290, a function
   that as shipped returns nothing) and hands a, b to the plain operators (:296-323).  ``fuse_ab=False`` takes that
@@ -29,6 +31,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .chunk import chunk_hrdplr_delta_rule
+from . import layer_pre as _pre
 from .hdla import chunk_hdla_delta_rule, fused_recurrent_hdla_delta_rule, parameterize_a_b
 from .normalize import get_norm_fn, l2_norm
 from .recurrent import fused_recurrent_dplr_delta_rule
@@ -105,6 +108,7 @@ class HDLA_Custom(nn.Module):
         num_blocks: int = 1,
         fuse_ab: bool = True,
         dispatch: str = "auto",
+        fuse_pre: bool = True,
         **kwargs,
     ):
         super().__init__()
@@ -135,7 +139,8 @@ class HDLA_Custom(nn.Module):
         self.token_mixer_init_type, self.rescale_type = token_mixer_init_type, rescale_type
         self.num_hidden_layers, self.init_std, self.gain = num_hidden_layers, init_std, gain
         self.num_blocks = num_blocks
-        self.fuse_ab, self.dispatch = fuse_ab, dispatch
+        self.fuse_ab, self.dispatch, self.fuse_pre = fuse_ab, dispatch, fuse_pre
+        self._all_silu = all(a in ("silu", "swish") for a in (q_activation, k_activation, v_activation))
         self._init_weights()
 
     # ---- initialisation: hdla_custom.py:159-187 and normalization_utils.py:115-211 (the branches a module of this
@@ -182,18 +187,41 @@ class HDLA_Custom(nn.Module):
         """x [b, n, d] -> q, k, v [b, n, H, D], beta [b, n, H, 1], log_f [b, n, H, D] with H = num_heads * num_blocks,
         and the inner activations of the output gate [b, n, head_dim] (None without a gate)."""
         b, n, d = x.shape
-        # every projection of x in one GEMM (q, k, v, the first halves of the decay and gate projections, beta): one
+        # every projection of x in one GEMM (q, k, v, beta, the first halves of the decay and gate projections): one
         # read of x forward, one GEMM each for dx and dW backward instead of six and their sums
-        heads = [self.q_proj, self.k_proj, self.v_proj, self.f_proj[0]]
-        if self.use_output_gate:
-            heads.append(self.output_gate[0])
+        heads = [self.q_proj, self.k_proj, self.v_proj]
         if self.use_beta:
             heads.append(self.bet_proj)
+        heads.append(self.f_proj[0])
+        if self.use_output_gate:
+            heads.append(self.output_gate[0])
         w = torch.cat([m.weight for m in heads], dim=0)
         bias = torch.cat([m.bias for m in heads], dim=0) if heads[0].bias is not None else None
-        parts = list(F.linear(x, w, bias).split([m.out_features for m in heads], dim=-1))
-        q, k, v, f0 = parts[:4]
-        gate0 = parts[4] if self.use_output_gate else None
+        y = F.linear(x, w, bias)
+        ldy, hd = y.shape[-1], self.head_dim
+        if (self.fuse_pre and self._all_silu and self.num_blocks == 1 and lower_bound is None and x.is_cuda
+                and _pre.supported(y.dtype, hd, ldy, (d, 2 * d, 3 * d))):
+            # activations, head split, l2 normalisation and beta in one kernel each way; its backward pass writes the
+            # gradient of y in place
+            col_tail = 3 * d + (self.num_heads if self.use_beta else 0)
+            q, k, v, beta, tail = _pre.layer_pre(
+                y.reshape(b * n, ldy), self.num_heads, hd, 0, d, 2 * d, 3 * d if self.use_beta else -1, col_tail,
+                self.norm_q, True, self.norm_v, 2.0 if self.beta_activation == "neg" else 1.0)
+            q, k, v = (t.view(b, n, self.num_heads, hd) for t in (q, k, v))
+            beta = beta.view(b, n, self.num_heads, 1) if self.use_beta else x.new_full((b, n, self.num_heads, 1), 2.0)
+            f = self.f_proj[1](tail[:, :hd]).view(b, n, d)
+            if self.use_offset:
+                f = f + self.offset
+            log_f = _pre.logsigmoid(f).view(b, n, self.num_heads, hd)
+            gate0 = tail[:, hd:].view(b, n, hd) if self.use_output_gate else None
+            if attention_mask is not None and not attention_mask.all() and n > 1:        # left padding
+                keep = attention_mask[:, q_offset:].unsqueeze(-1).unsqueeze(-1) != 0
+                k = k.masked_fill(~keep, 0)
+                log_f = log_f.masked_fill(~keep, 0)
+            return q, k, v, beta, log_f, gate0
+        parts = dict(zip([id(m) for m in heads], y.split([m.out_features for m in heads], dim=-1)))
+        q, k, v, f0 = (parts[id(m)] for m in (self.q_proj, self.k_proj, self.v_proj, self.f_proj[0]))
+        gate0 = parts[id(self.output_gate[0])] if self.use_output_gate else None
         f = self.f_proj[1](f0)
         if self.use_offset:
             f = f + self.offset
@@ -202,7 +230,7 @@ class HDLA_Custom(nn.Module):
         else:
             log_f = F.logsigmoid(f)
         if self.use_beta:
-            beta = torch.sigmoid(parts[-1]).unsqueeze(-1)
+            beta = torch.sigmoid(parts[id(self.bet_proj)]).unsqueeze(-1)
             if self.beta_activation == "neg":
                 beta = beta * 2
         else:

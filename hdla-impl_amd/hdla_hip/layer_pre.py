@@ -1,0 +1,115 @@
+"""The elementwise stage of the HDLA layer between its projections and the operator, as two fused operators.
+
+* ``layer_pre``   : (y, ...) -> q, k, v, beta, tail.  ``y [rows, ldy]`` is the output of the layer's one projection
+  GEMM; q, k, v are ``silu`` of three of its column ranges, split into heads and l2-normalised where asked
+  (HRDPLR/hdla_custom.py:228-251), beta is ``beta_scale * sigmoid`` of a fourth (:221-224), and ``tail`` is a
+  contiguous copy of the columns from ``col_tail`` on (the inner activations of the low-rank decay and gate
+  projections).  Its backward pass writes the gradient of all of y once (C ABI ``hdla_layer_pre_fwd/_bwd``).
+* ``logsigmoid``  : HRDPLR/hdla_custom.py:219 (C ABI ``hdla_logsigmoid_fwd/_bwd``).
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from .chunk import _require_gpu
+
+
+def supported(dtype: torch.dtype, D: int, ldy: int, cols) -> bool:
+    """Shapes the kernels take: a head is 16 bytes times a power of two (<= 64) of lanes, rows and column ranges
+    start on 16-byte boundaries."""
+    if dtype not in (torch.bfloat16, torch.float32):
+        return False
+    n = 8 if dtype == torch.bfloat16 else 4
+    if D % n:
+        return False
+    lanes = D // n
+    return lanes <= 64 and lanes & (lanes - 1) == 0 and ldy % n == 0 and all(c % n == 0 for c in cols)
+
+
+class LayerPreFunction(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx, y, H, D, col_q, col_k, col_v, col_beta, col_tail, norm_q, norm_k, norm_v, beta_scale, eps):
+        assert y.dim() == 2 and y.is_contiguous()
+        lib = _lib.load()
+        rows, ldy = y.shape
+        dims = _lib.HdlaPreDims(rows, H, D, _lib.dtype_code(y.dtype), ldy, col_q, col_k, col_v, col_beta,
+                                int(norm_q), int(norm_k), int(norm_v), float(beta_scale), float(eps))
+        with torch.cuda.device(y.device):
+            q, k, v = (torch.empty(rows, H, D, dtype=y.dtype, device=y.device) for _ in range(3))
+            beta = torch.empty(rows, H, 1, dtype=y.dtype, device=y.device) if col_beta >= 0 else None
+            rc = lib.hdla_layer_pre_fwd(ctypes.byref(dims), _lib.ptr(y), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v),
+                                        _lib.ptr(beta), _lib.current_stream(y.device))
+            _lib.check(rc, "hdla_layer_pre_fwd")
+            tail = y[:, col_tail:].contiguous() if col_tail < ldy else None
+        ctx.save_for_backward(y)
+        ctx.dims, ctx.col_tail = dims, col_tail
+        return q, k, v, beta, tail
+
+    @staticmethod
+    def backward(ctx, dq, dk, dv, dbeta, dtail):
+        (y,) = ctx.saved_tensors
+        dims, col_tail = ctx.dims, ctx.col_tail
+        lib = _lib.load()
+        rows, ldy = y.shape
+        H, D = dims.H, dims.D
+        z = lambda g, *shape: (torch.zeros(*shape, dtype=y.dtype, device=y.device) if g is None
+                               else g.to(y.dtype).contiguous())
+        dq, dk, dv = z(dq, rows, H, D), z(dk, rows, H, D), z(dv, rows, H, D)
+        if dims.col_beta >= 0:
+            dbeta = z(dbeta, rows, H, 1)
+        with torch.cuda.device(y.device):
+            covered = 3 * H * D + (H if dims.col_beta >= 0 else 0) + (ldy - col_tail)
+            dy = torch.empty_like(y) if covered == ldy else torch.zeros_like(y)      # gaps between the ranges stay zero
+            rc = lib.hdla_layer_pre_bwd(ctypes.byref(dims), _lib.ptr(y), _lib.ptr(dq), _lib.ptr(dk), _lib.ptr(dv),
+                                        _lib.ptr(dbeta) if dims.col_beta >= 0 else None, _lib.ptr(dy),
+                                        _lib.current_stream(y.device))
+            _lib.check(rc, "hdla_layer_pre_bwd")
+            if col_tail < ldy:
+                if dtail is None:
+                    dy[:, col_tail:].zero_()
+                else:
+                    dy[:, col_tail:].copy_(dtail)
+        return (dy,) + (None,) * 12
+
+
+def layer_pre(y, H, D, col_q, col_k, col_v, col_beta, col_tail, norm_q, norm_k, norm_v, beta_scale, eps=1e-5):
+    """y [rows, ldy] -> q, k, v [rows, H, D], beta [rows, H, 1] (None when col_beta < 0), tail [rows, ldy - col_tail]
+    (None when col_tail == ldy).  The column ranges must not overlap."""
+    _require_gpu(y)
+    return LayerPreFunction.apply(y, H, D, col_q, col_k, col_v, col_beta, col_tail, norm_q, norm_k, norm_v,
+                                  beta_scale, eps)
+
+
+class LogSigmoidFunction(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx, x):
+        x = x.contiguous()
+        lib = _lib.load()
+        with torch.cuda.device(x.device):
+            y = torch.empty_like(x)
+            rc = lib.hdla_logsigmoid_fwd(_lib.dtype_code(x.dtype), x.numel(), _lib.ptr(x), _lib.ptr(y),
+                                         _lib.current_stream(x.device))
+            _lib.check(rc, "hdla_logsigmoid_fwd")
+        ctx.save_for_backward(x)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        (x,) = ctx.saved_tensors
+        dy = dy.to(x.dtype).contiguous()
+        lib = _lib.load()
+        with torch.cuda.device(x.device):
+            dx = torch.empty_like(x)
+            rc = lib.hdla_logsigmoid_bwd(_lib.dtype_code(x.dtype), x.numel(), _lib.ptr(x), _lib.ptr(dy), _lib.ptr(dx),
+                                         _lib.current_stream(x.device))
+            _lib.check(rc, "hdla_logsigmoid_bwd")
+        return dx
+
+
+def logsigmoid(x: torch.Tensor) -> torch.Tensor:
+    """log(sigmoid(x)) elementwise; the element count must be a multiple of 16 bytes' worth."""
+    _require_gpu(x)
+    return LogSigmoidFunction.apply(x)

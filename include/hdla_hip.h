@@ -169,6 +169,31 @@ int hdla_normalize_bwd(const hdla_norm_dims* dims, const void* x, const void* we
                        void* stream);
 size_t hdla_normalize_workspace_bytes(const hdla_norm_dims* dims);
 
+/* What the HDLA layer does between its projections and the operator, one pass per direction
+ * (HRDPLR/hdla_custom.py:214-251): q = silu(q_raw), k = silu(k_raw), v = silu(v_raw), each l2-normalised per head when
+ * its flag is set (x / sqrt(sum x^2 + D eps), HRDPLR/normalizations/l2_norm.py:4-14; the layer always sets norm_k), and
+ * beta = beta_scale * sigmoid(bet_raw).  The raw inputs are column ranges of one row-major matrix y [rows, ldy]
+ * (a projection output): q_raw of head h at columns col_q + h*D .. + D, likewise k, v; bet_raw at col_beta + h
+ * (col_beta < 0: no beta).  Outputs are contiguous [rows, H, D] (q, k, v) and [rows, H] (beta).
+ * D * element size must be 16 bytes times a power of two <= 64; ldy and the q/k/v column offsets multiples of 16 bytes. */
+typedef struct hdla_pre_dims {
+    int64_t rows;
+    int32_t H, D;
+    int32_t dtype;
+    int32_t ldy, col_q, col_k, col_v, col_beta;
+    int32_t norm_q, norm_k, norm_v;
+    float beta_scale, eps;
+} hdla_pre_dims;
+int hdla_layer_pre_fwd(const hdla_pre_dims* dims, const void* y, void* q, void* k, void* v, void* beta, void* stream);
+/* Backward pass: from y and the gradients of the four outputs, the gradient of y's four column ranges, written in
+ * place into dy [rows, ldy]; the other columns of dy are not touched. */
+int hdla_layer_pre_bwd(const hdla_pre_dims* dims, const void* y, const void* dq, const void* dk, const void* dv,
+                       const void* dbeta, void* dy, void* stream);
+/* log_f = logsigmoid(f) (HRDPLR/hdla_custom.py:219) and its gradient df = dlog_f * sigmoid(-f), elementwise over n
+ * contiguous elements (n a multiple of 16 bytes' worth). */
+int hdla_logsigmoid_fwd(int dtype, int64_t n, const void* x, void* y, void* stream);
+int hdla_logsigmoid_bwd(int dtype, int64_t n, const void* x, const void* dy, void* dx, void* stream);
+
 /* Measurement aid; it has no counterpart in the reference.  One launch of a kernel that reads `n_read` (0..3)
  * buffers and writes `n_write` (0..2) buffers of `bytes` bytes each (a multiple of 16; every pointer 16-byte
  * aligned) and does nothing else.  Supported mixes (reads:writes): 1:0, 0:1, 1:1, 2:1, 3:1, 1:2; others return

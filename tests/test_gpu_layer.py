@@ -44,6 +44,8 @@ def _oracle(m, x, do, H, **kw):
     (torch.float32, 256, 2, 37, {"num_blocks": 2, "norm_q": True, "norm_v": True}),
     (torch.float32, 192, 3, 50, {"use_beta": False, "use_output_gate": False, "use_offset": True}),
     (torch.bfloat16, 512, 8, 128, {}),
+    (torch.bfloat16, 512, 8, 128, {"fuse_pre": False}),
+    (torch.float32, 256, 4, 80, {"fuse_pre": False, "fuse_ab": False}),
     (torch.bfloat16, 256, 2, 96, {"gate_pos": "post"}),
 ])
 def test_training_step_against_the_oracle(dtype, d, H, n, kw):

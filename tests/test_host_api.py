@@ -32,7 +32,8 @@ def test_library_exports_every_declared_symbol():
     assert {"hdla_version", "hdla_strerror", "hdla_workspace_bytes", "hdla_workspace_layout", "hdla_chunk_fwd",
             "hdla_chunk_bwd", "hdla_chunk_stages", "hdla_recurrent_fwd", "hdla_param_chunk_fwd", "hdla_param_chunk_bwd",
             "hdla_param_recurrent_fwd", "hdla_calib_stream", "hdla_normalize_fwd", "hdla_normalize_bwd",
-            "hdla_normalize_workspace_bytes"} <= names
+            "hdla_normalize_workspace_bytes", "hdla_layer_pre_fwd", "hdla_layer_pre_bwd", "hdla_logsigmoid_fwd",
+            "hdla_logsigmoid_bwd"} <= names
     for n in names:
         assert hasattr(lib, n), n
     assert lib.hdla_version() == 100
@@ -132,6 +133,32 @@ def test_normalize_entry_points_check_their_arguments():
     assert b(ctypes.byref(nd()), ok, ok, ok, ok, ok, None, ok, ok, need, None) == -1           # gate without dgate
     assert b(ctypes.byref(nd()), ok, ok, ok, ok, ok, ok, ok, ok, need - 1, None) == -5
     assert b(ctypes.byref(nd()), ok, ok, ok, ok, ok, ok, ok, None, need, None) == -5
+
+
+def test_layer_pre_entry_points_check_their_arguments():
+    lib = _lib.load()
+    ok, bad = ctypes.c_void_p(4096), ctypes.c_void_p(4096 + 8)
+    pd = lambda **kw: _lib.HdlaPreDims(**{**dict(rows=8, H=16, D=64, dtype=0, ldy=3216, col_q=0, col_k=1024, col_v=2048,
+                                                 col_beta=3072, norm_q=0, norm_k=1, norm_v=0, beta_scale=2.0, eps=1e-5),
+                                          **kw})
+    f, b = lib.hdla_layer_pre_fwd, lib.hdla_layer_pre_bwd
+    assert f(ctypes.byref(pd()), None, ok, ok, ok, ok, None) == -1
+    assert f(ctypes.byref(pd()), ok, ok, ok, ok, None, None) == -1                   # beta columns given, no beta output
+    assert f(ctypes.byref(pd(col_beta=-1)), ok, ok, bad, ok, None, None) == -6
+    assert f(ctypes.byref(pd(D=48)), ok, ok, ok, ok, ok, None) == -2                 # 6 lanes a head: not a power of two
+    assert f(ctypes.byref(pd(D=1024, H=1)), ok, ok, ok, ok, ok, None) == -2          # more than one wavefront a head
+    assert f(ctypes.byref(pd(ldy=3210)), ok, ok, ok, ok, ok, None) == -6             # rows off 16-byte boundaries
+    assert f(ctypes.byref(pd(col_k=1028)), ok, ok, ok, ok, ok, None) == -6
+    assert f(ctypes.byref(pd(col_v=2200)), ok, ok, ok, ok, ok, None) == -2           # range runs past the row
+    assert f(ctypes.byref(pd(col_beta=3208)), ok, ok, ok, ok, ok, None) == -2
+    assert f(ctypes.byref(pd(dtype=7)), ok, ok, ok, ok, ok, None) == -4
+    assert f(ctypes.byref(pd(rows=0)), None, None, None, None, None, None) == 0
+    assert b(ctypes.byref(pd()), ok, ok, ok, ok, None, ok, None) == -1               # dbeta missing
+    assert b(ctypes.byref(pd()), ok, ok, ok, ok, ok, None, None) == -1
+    lf, lb = lib.hdla_logsigmoid_fwd, lib.hdla_logsigmoid_bwd
+    assert lf(0, 12, ok, ok, None) == -2
+    assert lf(0, 16, None, ok, None) == -1 and lf(5, 16, ok, ok, None) == -4 and lf(0, 0, None, None, None) == 0
+    assert lb(0, 16, ok, None, ok, None) == -1 and lb(0, 16, ok, bad, ok, None) == -6
 
 
 def test_normalize_python_entry_validates_and_needs_a_gpu():
