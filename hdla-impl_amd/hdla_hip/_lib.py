@@ -103,6 +103,11 @@ def load():
     lib.hdla_logsigmoid_fwd.argtypes = [ctypes.c_int, ctypes.c_int64, P, P, P]
     lib.hdla_logsigmoid_bwd.restype = ctypes.c_int
     lib.hdla_logsigmoid_bwd.argtypes = [ctypes.c_int, ctypes.c_int64, P, P, P, P]
+    lib.hdla_skinny_wgrad.restype = ctypes.c_int
+    lib.hdla_skinny_wgrad.argtypes = [ctypes.c_int, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, P, ctypes.c_int64, P,
+                                      ctypes.c_int64, P, P, ctypes.c_size_t, P]
+    lib.hdla_skinny_wgrad_workspace_bytes.restype = ctypes.c_size_t
+    lib.hdla_skinny_wgrad_workspace_bytes.argtypes = [ctypes.c_int, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]
     _lib = lib
     return lib
 

@@ -182,6 +182,12 @@ class HDLA_Custom(nn.Module):
         return (f"embed_dim={self.embed_dim}, num_heads={self.num_heads}, num_blocks={self.num_blocks}, "
                 f"fuse_ab={self.fuse_ab}, dispatch={self.dispatch}")
 
+    def _up(self, lin: nn.Linear, x0: torch.Tensor) -> torch.Tensor:
+        """Second half of a low-rank projection (head_dim -> embed_dim)."""
+        if self.fuse_pre and lin.bias is None and x0.is_cuda and x0.dtype == torch.bfloat16 == lin.weight.dtype:
+            return _pre.low_rank_up(x0, lin.weight)
+        return lin(x0)
+
     # ---- the part of forward() before the recurrence (hdla_custom.py:202-267) --------------------------------------
     def project(self, x, attention_mask=None, q_offset=0, lower_bound=None):
         """x [b, n, d] -> q, k, v [b, n, H, D], beta [b, n, H, 1], log_f [b, n, H, D] with H = num_heads * num_blocks,
@@ -209,7 +215,7 @@ class HDLA_Custom(nn.Module):
                 self.norm_q, True, self.norm_v, 2.0 if self.beta_activation == "neg" else 1.0)
             q, k, v = (t.view(b, n, self.num_heads, hd) for t in (q, k, v))
             beta = beta.view(b, n, self.num_heads, 1) if self.use_beta else x.new_full((b, n, self.num_heads, 1), 2.0)
-            f = self.f_proj[1](tail[:, :hd]).view(b, n, d)
+            f = self._up(self.f_proj[1], tail[:, :hd]).view(b, n, d)
             if self.use_offset:
                 f = f + self.offset
             log_f = _pre.logsigmoid(f).view(b, n, self.num_heads, hd)
@@ -291,7 +297,7 @@ class HDLA_Custom(nn.Module):
             past_key_values.update(recurrent_state=[recurrent_state], layer_idx=self.layer_idx, offset=n)
         output = output.flatten(2, 3)
         if self.use_output_gate:
-            output = self.norm(output, self.output_gate[1](gate0))
+            output = self.norm(output, self._up(self.output_gate[1], gate0))
         else:
             output = self.norm(output)
         return self.o_proj(output), past_key_values

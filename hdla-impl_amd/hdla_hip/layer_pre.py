@@ -6,10 +6,15 @@
   contiguous copy of the columns from ``col_tail`` on (the inner activations of the low-rank decay and gate
   projections).  Its backward pass writes the gradient of all of y once (C ABI ``hdla_layer_pre_fwd/_bwd``).
 * ``logsigmoid``  : HRDPLR/hdla_custom.py:219 (C ABI ``hdla_logsigmoid_fwd/_bwd``).
+* ``low_rank_up`` : ``F.linear(x0, W)`` for the second half of a low-rank projection (head_dim -> embed_dim,
+  hdla_custom.py:117-121,151-155) whose weight gradient ``dY^T @ x0`` — a tiny output contracted over all rows, for
+  which a BLAS kernel tiled over the output has 16 workgroups — runs in a kernel of this library that also splits the
+  rows (C ABI ``hdla_skinny_wgrad``); forward and input gradient stay BLAS calls.
 """
 import ctypes
 
 import torch
+import torch.nn.functional as F
 
 from . import _lib
 from .chunk import _require_gpu
@@ -113,3 +118,47 @@ def logsigmoid(x: torch.Tensor) -> torch.Tensor:
     """log(sigmoid(x)) elementwise; the element count must be a multiple of 16 bytes' worth."""
     _require_gpu(x)
     return LogSigmoidFunction.apply(x)
+
+
+def skinny_ok(dy: torch.Tensor, n_cols: int) -> bool:
+    return (dy.is_cuda and dy.dtype == torch.bfloat16 and n_cols in (64, 128) and dy.shape[-1] % 64 == 0
+            and dy.shape[0] > 0)
+
+
+class LowRankUpFunction(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx, x0, weight):
+        ctx.save_for_backward(x0, weight)
+        return F.linear(x0, weight)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x0, weight = ctx.saved_tensors
+        K, N = weight.shape                                   # embed_dim, head_dim
+        dy2 = dy.reshape(-1, K)
+        dx0 = dw = None
+        if ctx.needs_input_grad[0]:
+            dx0 = (dy2 @ weight).reshape(x0.shape)
+        if ctx.needs_input_grad[1]:
+            x2 = x0.reshape(-1, N)
+            if (skinny_ok(dy2, N) and weight.dtype == x2.dtype == torch.bfloat16 and dy2.stride(1) == 1 and x2.stride(1) == 1
+                    and dy2.stride(0) % 4 == 0 and x2.stride(0) % 4 == 0 and dy2.data_ptr() % 8 == 0 and x2.data_ptr() % 8 == 0):
+                lib = _lib.load()
+                M = dy2.shape[0]
+                with torch.cuda.device(dy2.device):
+                    nws = lib.hdla_skinny_wgrad_workspace_bytes(_lib.HDLA_BF16, M, N, K)
+                    ws = torch.empty(nws, dtype=torch.uint8, device=dy2.device)
+                    dw = torch.empty(K, N, dtype=torch.bfloat16, device=dy2.device)
+                    rc = lib.hdla_skinny_wgrad(_lib.HDLA_BF16, M, N, K, _lib.ptr(dy2), dy2.stride(0), _lib.ptr(x2),
+                                               x2.stride(0), _lib.ptr(dw), _lib.ptr(ws), nws,
+                                               _lib.current_stream(dy2.device))
+                    _lib.check(rc, "hdla_skinny_wgrad")
+            else:
+                dw = dy2.t() @ x2
+        return dx0, dw
+
+
+def low_rank_up(x0: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """``x0 [..., head_dim] @ weight[embed_dim, head_dim]^T`` with this library's kernel for the weight gradient."""
+    return LowRankUpFunction.apply(x0, weight)

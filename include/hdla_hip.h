@@ -194,6 +194,16 @@ int hdla_layer_pre_bwd(const hdla_pre_dims* dims, const void* y, const void* dq,
 int hdla_logsigmoid_fwd(int dtype, int64_t n, const void* x, void* y, void* stream);
 int hdla_logsigmoid_bwd(int dtype, int64_t n, const void* x, const void* dy, void* dx, void* stream);
 
+/* dW [K, N] = dY [M, K]^T * X0 [M, N], bf16 with fp32 accumulation, for N = 64 or 128 and K a multiple of 64: the
+ * weight gradient of the layer's Linear(head_dim -> embed_dim) projections (second halves of f_proj and output_gate,
+ * HRDPLR/hdla_custom.py:117-121,151-155; in the reference a BLAS call inside autograd) with dY [M, embed_dim] the
+ * gradient of their output and X0 [M, head_dim] their input.  ldy, ldx: row strides in elements (multiples of 4);
+ * dW is contiguous [K, N] (the weight's layout).  The rows are split over workgroups; partial results go through
+ * `workspace` (hdla_skinny_wgrad_workspace_bytes() bytes, 16-byte aligned) and are added in a fixed order. */
+int hdla_skinny_wgrad(int dtype, int64_t M, int32_t N, int32_t K, const void* dY, int64_t ldy, const void* X0,
+                      int64_t ldx, void* dW, void* workspace, size_t workspace_bytes, void* stream);
+size_t hdla_skinny_wgrad_workspace_bytes(int dtype, int64_t M, int32_t N, int32_t K);
+
 /* Measurement aid; it has no counterpart in the reference.  One launch of a kernel that reads `n_read` (0..3)
  * buffers and writes `n_write` (0..2) buffers of `bytes` bytes each (a multiple of 16; every pointer 16-byte
  * aligned) and does nothing else.  Supported mixes (reads:writes): 1:0, 0:1, 1:1, 2:1, 3:1, 1:2; others return

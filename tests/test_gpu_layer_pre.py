@@ -103,3 +103,36 @@ def test_empty_input():
     q, k, v, beta, tail = LP.layer_pre(y, 2, 64, 0, 128, 256, 384, 386, False, True, False, 2.0)
     assert q.shape == (0, 2, 64) and beta.shape == (0, 2, 1) and tail.shape == (0, 6)
     assert LP.logsigmoid(torch.empty(0, 8, device=DEV)).shape == (0, 8)
+
+
+@pytest.mark.parametrize("M,N,K,strided", [(8192, 64, 1024, True), (100, 64, 128, False), (33, 128, 512, True),
+                                              (1, 128, 4096, False), (4097, 64, 2048, False), (70000, 64, 64, False)])
+def test_low_rank_up_weight_gradient_against_float64_matmul(M, N, K, strided):
+    """hdla_skinny_wgrad through LowRankUpFunction's backward: dW = dY^T @ X0 against the float64 product of the same
+    bf16 operands; the result is rounded to bf16 once (2^-9 relative per element)."""
+    g = torch.Generator().manual_seed(M + N)
+    dy = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(K, N, generator=g) / K ** 0.5).bfloat16()
+    x0 = torch.randn(M, N, generator=g).bfloat16()
+    wd = w.to(DEV).requires_grad_()
+    if strided:                                             # the layer's case: x0 is a column range of a wider tensor
+        wide = torch.cat([x0, x0 + 1], dim=1).to(DEV).requires_grad_()
+        xd = wide[:, :N]
+    else:
+        xd = x0.to(DEV).requires_grad_()
+    y = LP.low_rank_up(xd, wd)
+    assert torch.equal(y, F.linear(xd, wd))
+    gx, gw = torch.autograd.grad(y, [xd, wd], dy.to(DEV))
+    rx, rw = dy.double() @ w.double(), dy.double().T @ x0.double()
+    ex, ew = O.rel_l2(gx, rx), O.rel_l2(gw, rw)
+    print(M, N, K, f"dx0 {ex:.2e} dw {ew:.2e}", flush=True)
+    assert gw.dtype == torch.bfloat16 and gw.shape == (K, N) and gx.shape == (M, N)
+    assert ex <= 3e-3 and ew <= 3e-3
+    # exactness on small integers: every partial and final sum is an integer that fp32 and bf16 hold exactly
+    picked = torch.arange(0, M, max(1, M // 7))[:7]          # at most seven non-zero rows spread over the row ranges
+    a = torch.zeros(M, K)
+    a[picked] = torch.randint(-2, 3, (len(picked), K), generator=g).float()
+    b = torch.randint(-2, 3, (M, N), generator=g).float()
+    yi = LP.low_rank_up(b.bfloat16().to(DEV), wd)
+    (gi,) = torch.autograd.grad(yi, wd, a.bfloat16().to(DEV))
+    assert torch.equal(gi.float().cpu(), a.T @ b)

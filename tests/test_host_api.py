@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol():
             "hdla_chunk_bwd", "hdla_chunk_stages", "hdla_recurrent_fwd", "hdla_param_chunk_fwd", "hdla_param_chunk_bwd",
             "hdla_param_recurrent_fwd", "hdla_calib_stream", "hdla_normalize_fwd", "hdla_normalize_bwd",
             "hdla_normalize_workspace_bytes", "hdla_layer_pre_fwd", "hdla_layer_pre_bwd", "hdla_logsigmoid_fwd",
-            "hdla_logsigmoid_bwd"} <= names
+            "hdla_logsigmoid_bwd", "hdla_skinny_wgrad", "hdla_skinny_wgrad_workspace_bytes"} <= names
     for n in names:
         assert hasattr(lib, n), n
     assert lib.hdla_version() == 100
@@ -159,6 +159,19 @@ def test_layer_pre_entry_points_check_their_arguments():
     assert lf(0, 12, ok, ok, None) == -2
     assert lf(0, 16, None, ok, None) == -1 and lf(5, 16, ok, ok, None) == -4 and lf(0, 0, None, None, None) == 0
     assert lb(0, 16, ok, None, ok, None) == -1 and lb(0, 16, ok, bad, ok, None) == -6
+    sg, sw = lib.hdla_skinny_wgrad, lib.hdla_skinny_wgrad_workspace_bytes
+    need = sw(0, 8192, 64, 1024)
+    assert need == 16 * 1024 * 64 * 4 and sw(1, 8192, 64, 1024) == 0 and sw(0, 8192, 48, 1024) == 0
+    assert sw(0, 5, 128, 64) == 1 * 64 * 128 * 4                                    # fewer rows than one tile: one range
+    assert sg(0, 8192, 64, 1024, None, 1024, ok, 64, ok, ok, need, None) == -1
+    assert sg(1, 8192, 64, 1024, ok, 1024, ok, 64, ok, ok, need, None) == -4         # bf16 only
+    assert sg(0, 8192, 48, 1024, ok, 1024, ok, 48, ok, ok, need, None) == -2
+    assert sg(0, 8192, 64, 1000, ok, 1000, ok, 64, ok, ok, need, None) == -2
+    assert sg(0, 8192, 64, 1024, ok, 512, ok, 64, ok, ok, need, None) == -2          # row stride shorter than a row
+    assert sg(0, 8192, 64, 1024, ok, 1026, ok, 64, ok, ok, need, None) == -6
+    assert sg(0, 8192, 64, 1024, ok, 1024, ok, 64, bad, ok, need, None) == -6
+    assert sg(0, 8192, 64, 1024, ok, 1024, ok, 64, ok, ok, need - 1, None) == -5
+    assert sg(0, 8192, 64, 1024, ok, 1024, ok, 64, ok, None, need, None) == -5
 
 
 def test_normalize_python_entry_validates_and_needs_a_gpu():
