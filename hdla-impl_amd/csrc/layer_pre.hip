@@ -186,7 +186,13 @@ __global__ __launch_bounds__(256) void logsigmoid_kernel(const void* x, const vo
 #pragma unroll
         for (int j = 0; j < N; ++j) {
             if (BWD) f[j] = g[j] * pre_sigmoid<T>(-f[j]);
-            else f[j] = fminf(f[j], 0.f) - log1pf(exp_t<T>(-fabsf(f[j])));
+            else {
+                // log(1 + e) for e = exp(-|f|) in (0, 1]: the accurate routine for fp32 results; for bf16 results the
+                // hardware logarithm, with the first term of the series where 1 + e would round e away
+                const float e = exp_t<T>(-fabsf(f[j]));
+                const float l = sizeof(T) == 4 ? log1pf(e) : (e < 1e-4f ? e : __logf(1.f + e));
+                f[j] = fminf(f[j], 0.f) - l;
+            }
         }
         PrePiece<T>::st(out, i * N, f);
     }

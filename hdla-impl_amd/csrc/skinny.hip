@@ -4,8 +4,9 @@
 // Linear(embed_dim -> head_dim) followed by Linear(head_dim -> embed_dim), HRDPLR/hdla_custom.py:117-121,151-155; in the
 // reference a BLAS call inside autograd).  The output is tiny (K x N) and the contraction runs over all rows, so a
 // BLAS kernel tiled over the output has 16 workgroups to work with; here the rows are split as well: a workgroup owns
-// 64 columns of dY (one 16-column tile per wavefront) and one range of rows, streams its part of dY once, and leaves a
-// fp32 partial result; a second small kernel adds the partial results in a fixed order.
+// 32 columns of dY and one range of rows, its four wavefronts take every fourth 16-row tile of that range (16 bytes a
+// lane from dY and from X0), add their sums through LDS, and leave a fp32 partial result; a second small kernel adds
+// the partial results of the row ranges in a fixed order.
 //
 // The contraction index (the row) must be the inner index of both MFMA operands, and both are stored with the row
 // outermost, so each 16 x 16 tile is transposed on its way in by one product with the identity (exact in bf16).
@@ -14,34 +15,71 @@
 
 namespace hdla {
 
+// Two 16 x 16 tiles from one 16-byte load per lane: lane (g, c) reads elements 8g .. 8g+7 of row c of a 16 x 32 block;
+// the first four are the fragment of tile A, the last four of tile B, where tile A holds the block's columns
+// 8j + 0..3 and tile B the columns 8j + 4..7 (j = 0..3).  Element e = 0..15 of a tile's column index is therefore
+// column 8 (e / 4) + e % 4 (+ 4 for tile B) of the block.
+__device__ __forceinline__ void ld_two_tiles(const bf16* p, bool ok, Frag<bf16>& a, Frag<bf16>& b) {
+    s16x8 x = *reinterpret_cast<const s16x8*>(p);
+    const s16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+    x = ok ? x : z;
+    a.v = __builtin_shufflevector(x, x, 0, 1, 2, 3);
+    b.v = __builtin_shufflevector(x, x, 4, 5, 6, 7);
+}
+
 template <int N>
 __global__ __launch_bounds__(256) void skinny_wgrad_kernel(const bf16* __restrict__ dY, long long ldy,
                                                            const bf16* __restrict__ X0, long long ldx,
                                                            float* __restrict__ part, int M, int K, int rows_per) {
-    constexpr int CT = N / 16;
+    constexpr int ZP = N / 32;                                 // 32-column blocks of X0
+    __shared__ f32x4 red[3][2 * 2 * ZP][64];
     const int w = threadIdx.x >> 6, lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
-    const int k0 = blockIdx.x * 64 + 16 * w, s = blockIdx.y;
+    const int k0 = blockIdx.x * 32, s = blockIdx.y;
     const long long rbeg = (long long)s * rows_per;
     const long long rend = rbeg + rows_per < M ? rbeg + rows_per : M;
     const Frag<bf16> id = ident_frag<bf16>();
-    f32x4 acc[CT];
+    f32x4 acc[2][2 * ZP];                                      // [tile of dY's 32 columns][tile of X0's columns]
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) acc[ct] = zero4();
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2 * ZP; ++b) acc[a][b] = zero4();
+    // the four wavefronts take every fourth 16-row tile of the range
 #pragma unroll 2
-    for (long long r0 = rbeg; r0 < rend; r0 += 16) {
+    for (long long r0 = rbeg + 16 * w; r0 < rend; r0 += 64) {
         const bool ok = r0 + c < rend;
-        const long long row = ok ? r0 + c : rbeg;                          // a readable row on every lane
-        // F(X), X[c][4g+i] = dY[r0+c][k0+4g+i]; transposed: rows = columns of dY, inner index = row
-        const Frag<bf16> xt = transpose(ld_frag_sel(dY + row * ldy + k0 + 4 * g, ok), id);
+        const long long row = ok ? r0 + c : rbeg;              // a readable row on every lane
+        Frag<bf16> x[2], z[2 * ZP];
+        ld_two_tiles(dY + row * ldy + k0 + 8 * g, ok, x[0], x[1]);
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            const Frag<bf16> zt = transpose(ld_frag_sel(X0 + row * ldx + ct * 16 + 4 * g, ok), id);
-            acc[ct] = mm(xt, zt, acc[ct]);                                  // += sum_r dY[r][k0+c] * X0[r][16 ct + 4g + i]
+        for (int b = 0; b < ZP; ++b) ld_two_tiles(X0 + row * ldx + 32 * b + 8 * g, ok, z[2 * b], z[2 * b + 1]);
+        // transposed tiles: rows = columns of the block, inner index = row of the range
+        x[0] = transpose(x[0], id);
+        x[1] = transpose(x[1], id);
+#pragma unroll
+        for (int b = 0; b < 2 * ZP; ++b) {
+            const Frag<bf16> zt = transpose(z[b], id);
+            acc[0][b] = mm(x[0], zt, acc[0][b]);
+            acc[1][b] = mm(x[1], zt, acc[1][b]);
         }
     }
+    if (w) {
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct)
-        *reinterpret_cast<f32x4*>(part + ((long long)s * K + k0 + c) * N + ct * 16 + 4 * g) = acc[ct];
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < 2 * ZP; ++b) red[w - 1][a * 2 * ZP + b][lane] = acc[a][b];
+    }
+    __syncthreads();
+    if (w) return;
+    // lane (g, c) register i of acc[a][b]: dY column k0 + 8 (c / 4) + c % 4 + 4 a,
+    //                                      X0 column 32 (b / 2) + 8 g + 4 (b % 2) + i
+    const int krow = k0 + 8 * (c >> 2) + (c & 3);
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2 * ZP; ++b) {
+            const f32x4 v = acc[a][b] + red[0][a * 2 * ZP + b][lane] + red[1][a * 2 * ZP + b][lane] + red[2][a * 2 * ZP + b][lane];
+            *reinterpret_cast<f32x4*>(part + ((long long)s * K + krow + 4 * a) * N + 32 * (b >> 1) + 8 * g + 4 * (b & 1)) = v;
+        }
 }
 
 // dW = sum over the row ranges of their partial results, eight outputs a thread
@@ -65,7 +103,7 @@ __global__ __launch_bounds__(256) void skinny_wgrad_sum_kernel(const float* __re
 
 // row ranges: enough workgroups for the chip, whole 16-row tiles each
 static int wgrad_split(long long M, int K, int& rows_per) {
-    const int kb = K / 64;
+    const int kb = K / 32;
     long long S = (256 + kb - 1) / kb;
     const long long tiles = (M + 15) / 16;
     if (S > tiles) S = tiles;
@@ -100,13 +138,13 @@ extern "C" int hdla_skinny_wgrad(int dtype, int64_t M, int32_t N, int32_t K, con
     if (ldy < K || ldx < N) return HDLA_ERR_SHAPE;
     if (!dY || !X0 || !dW) return HDLA_ERR_NULL;
     const auto al = [](const void* p, int a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; };
-    if (!al(dY, 8) || !al(X0, 8) || !al(dW, 16) || ldy % 4 || ldx % 4) return HDLA_ERR_ALIGN;
+    if (!al(dY, 16) || !al(X0, 16) || !al(dW, 16) || ldy % 8 || ldx % 8) return HDLA_ERR_ALIGN;
     int rows_per;
     const int S = wgrad_split(M, K, rows_per);
     const size_t need = (size_t)S * K * N * sizeof(float);
     if (!workspace || !al(workspace, 16) || workspace_bytes < need) return HDLA_ERR_WORKSPACE;
     const hipStream_t s = static_cast<hipStream_t>(stream);
-    const dim3 grid(K / 64, S), block(256);
+    const dim3 grid(K / 32, S), block(256);
     float* part = static_cast<float*>(workspace);
     const bf16* a = static_cast<const bf16*>(dY);
     const bf16* b = static_cast<const bf16*>(X0);

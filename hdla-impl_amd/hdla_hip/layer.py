@@ -210,16 +210,17 @@ class HDLA_Custom(nn.Module):
             # activations, head split, l2 normalisation and beta in one kernel each way; its backward pass writes the
             # gradient of y in place
             col_tail = 3 * d + (self.num_heads if self.use_beta else 0)
-            q, k, v, beta, tail = _pre.layer_pre(
+            q, k, v, beta, f0, *rest = _pre.layer_pre(
                 y.reshape(b * n, ldy), self.num_heads, hd, 0, d, 2 * d, 3 * d if self.use_beta else -1, col_tail,
-                self.norm_q, True, self.norm_v, 2.0 if self.beta_activation == "neg" else 1.0)
+                (hd, hd) if self.use_output_gate else (hd,), self.norm_q, True, self.norm_v,
+                2.0 if self.beta_activation == "neg" else 1.0)
             q, k, v = (t.view(b, n, self.num_heads, hd) for t in (q, k, v))
             beta = beta.view(b, n, self.num_heads, 1) if self.use_beta else x.new_full((b, n, self.num_heads, 1), 2.0)
-            f = self._up(self.f_proj[1], tail[:, :hd]).view(b, n, d)
+            f = self._up(self.f_proj[1], f0).view(b, n, d)
             if self.use_offset:
                 f = f + self.offset
             log_f = _pre.logsigmoid(f).view(b, n, self.num_heads, hd)
-            gate0 = tail[:, hd:].view(b, n, hd) if self.use_output_gate else None
+            gate0 = rest[0].view(b, n, hd) if self.use_output_gate else None
             if attention_mask is not None and not attention_mask.all() and n > 1:        # left padding
                 keep = attention_mask[:, q_offset:].unsqueeze(-1).unsqueeze(-1) != 0
                 k = k.masked_fill(~keep, 0)

@@ -1,9 +1,9 @@
 """The elementwise stage of the HDLA layer between its projections and the operator, as two fused operators.
 
-* ``layer_pre``   : (y, ...) -> q, k, v, beta, tail.  ``y [rows, ldy]`` is the output of the layer's one projection
+* ``layer_pre``   : (y, ...) -> q, k, v, beta, tails.  ``y [rows, ldy]`` is the output of the layer's one projection
   GEMM; q, k, v are ``silu`` of three of its column ranges, split into heads and l2-normalised where asked
-  (HRDPLR/hdla_custom.py:228-251), beta is ``beta_scale * sigmoid`` of a fourth (:221-224), and ``tail`` is a
-  contiguous copy of the columns from ``col_tail`` on (the inner activations of the low-rank decay and gate
+  (HRDPLR/hdla_custom.py:228-251), beta is ``beta_scale * sigmoid`` of a fourth (:221-224), and the tails are
+  contiguous copies of the column ranges from ``col_tail`` on (the inner activations of the low-rank decay and gate
   projections).  Its backward pass writes the gradient of all of y once (C ABI ``hdla_layer_pre_fwd/_bwd``).
 * ``logsigmoid``  : HRDPLR/hdla_custom.py:219 (C ABI ``hdla_logsigmoid_fwd/_bwd``).
 * ``low_rank_up`` : ``F.linear(x0, W)`` for the second half of a low-rank projection (head_dim -> embed_dim,
@@ -35,10 +35,12 @@ def supported(dtype: torch.dtype, D: int, ldy: int, cols) -> bool:
 class LayerPreFunction(torch.autograd.Function):
 
     @staticmethod
-    def forward(ctx, y, H, D, col_q, col_k, col_v, col_beta, col_tail, norm_q, norm_k, norm_v, beta_scale, eps):
+    def forward(ctx, y, H, D, col_q, col_k, col_v, col_beta, col_tail, tail_widths, norm_q, norm_k, norm_v, beta_scale,
+                eps):
         assert y.dim() == 2 and y.is_contiguous()
         lib = _lib.load()
         rows, ldy = y.shape
+        assert col_tail + sum(tail_widths) == ldy
         dims = _lib.HdlaPreDims(rows, H, D, _lib.dtype_code(y.dtype), ldy, col_q, col_k, col_v, col_beta,
                                 int(norm_q), int(norm_k), int(norm_v), float(beta_scale), float(eps))
         with torch.cuda.device(y.device):
@@ -47,13 +49,16 @@ class LayerPreFunction(torch.autograd.Function):
             rc = lib.hdla_layer_pre_fwd(ctypes.byref(dims), _lib.ptr(y), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v),
                                         _lib.ptr(beta), _lib.current_stream(y.device))
             _lib.check(rc, "hdla_layer_pre_fwd")
-            tail = y[:, col_tail:].contiguous() if col_tail < ldy else None
+            tails, c = [], col_tail
+            for wdt in tail_widths:
+                tails.append(y[:, c:c + wdt].contiguous())
+                c += wdt
         ctx.save_for_backward(y)
-        ctx.dims, ctx.col_tail = dims, col_tail
-        return q, k, v, beta, tail
+        ctx.dims, ctx.col_tail, ctx.tail_widths = dims, col_tail, tuple(tail_widths)
+        return (q, k, v, beta) + tuple(tails)
 
     @staticmethod
-    def backward(ctx, dq, dk, dv, dbeta, dtail):
+    def backward(ctx, dq, dk, dv, dbeta, *dtails):
         (y,) = ctx.saved_tensors
         dims, col_tail = ctx.dims, ctx.col_tail
         lib = _lib.load()
@@ -71,20 +76,24 @@ class LayerPreFunction(torch.autograd.Function):
                                         _lib.ptr(dbeta) if dims.col_beta >= 0 else None, _lib.ptr(dy),
                                         _lib.current_stream(y.device))
             _lib.check(rc, "hdla_layer_pre_bwd")
-            if col_tail < ldy:
-                if dtail is None:
-                    dy[:, col_tail:].zero_()
+            c = col_tail
+            for wdt, g in zip(ctx.tail_widths, dtails):
+                if g is None:
+                    dy[:, c:c + wdt].zero_()
                 else:
-                    dy[:, col_tail:].copy_(dtail)
-        return (dy,) + (None,) * 12
+                    dy[:, c:c + wdt].copy_(g)
+                c += wdt
+        return (dy,) + (None,) * 13
 
 
-def layer_pre(y, H, D, col_q, col_k, col_v, col_beta, col_tail, norm_q, norm_k, norm_v, beta_scale, eps=1e-5):
-    """y [rows, ldy] -> q, k, v [rows, H, D], beta [rows, H, 1] (None when col_beta < 0), tail [rows, ldy - col_tail]
-    (None when col_tail == ldy).  The column ranges must not overlap."""
+def layer_pre(y, H, D, col_q, col_k, col_v, col_beta, col_tail, tail_widths, norm_q, norm_k, norm_v, beta_scale,
+              eps=1e-5):
+    """y [rows, ldy] -> q, k, v [rows, H, D], beta [rows, H, 1] (None when col_beta < 0), then one contiguous copy per
+    entry of ``tail_widths`` of consecutive column ranges starting at ``col_tail`` (together they must reach ldy).
+    The column ranges must not overlap."""
     _require_gpu(y)
-    return LayerPreFunction.apply(y, H, D, col_q, col_k, col_v, col_beta, col_tail, norm_q, norm_k, norm_v,
-                                  beta_scale, eps)
+    return LayerPreFunction.apply(y, H, D, col_q, col_k, col_v, col_beta, col_tail, tuple(tail_widths), norm_q, norm_k,
+                                  norm_v, beta_scale, eps)
 
 
 class LogSigmoidFunction(torch.autograd.Function):
@@ -143,7 +152,7 @@ class LowRankUpFunction(torch.autograd.Function):
         if ctx.needs_input_grad[1]:
             x2 = x0.reshape(-1, N)
             if (skinny_ok(dy2, N) and weight.dtype == x2.dtype == torch.bfloat16 and dy2.stride(1) == 1 and x2.stride(1) == 1
-                    and dy2.stride(0) % 4 == 0 and x2.stride(0) % 4 == 0 and dy2.data_ptr() % 8 == 0 and x2.data_ptr() % 8 == 0):
+                    and dy2.stride(0) % 8 == 0 and x2.stride(0) % 8 == 0 and dy2.data_ptr() % 16 == 0 and x2.data_ptr() % 16 == 0):
                 lib = _lib.load()
                 M = dy2.shape[0]
                 with torch.cuda.device(dy2.device):

@@ -197,7 +197,7 @@ int hdla_logsigmoid_bwd(int dtype, int64_t n, const void* x, const void* dy, voi
 /* dW [K, N] = dY [M, K]^T * X0 [M, N], bf16 with fp32 accumulation, for N = 64 or 128 and K a multiple of 64: the
  * weight gradient of the layer's Linear(head_dim -> embed_dim) projections (second halves of f_proj and output_gate,
  * HRDPLR/hdla_custom.py:117-121,151-155; in the reference a BLAS call inside autograd) with dY [M, embed_dim] the
- * gradient of their output and X0 [M, head_dim] their input.  ldy, ldx: row strides in elements (multiples of 4);
+ * gradient of their output and X0 [M, head_dim] their input.  ldy, ldx: row strides in elements (multiples of 8);
  * dW is contiguous [K, N] (the weight's layout).  The rows are split over workgroups; partial results go through
  * `workspace` (hdla_skinny_wgrad_workspace_bytes() bytes, 16-byte aligned) and are added in a fixed order. */
 int hdla_skinny_wgrad(int dtype, int64_t M, int32_t N, int32_t K, const void* dY, int64_t ldy, const void* X0,

@@ -53,7 +53,8 @@ def test_layer_pre_against_torch(dtype, rows, H, D, layout, flags):
     yo = y.double().requires_grad_()
     ref = _ref(yo, H, D, cq, ck, cv, cb, ct, nq, nk, nv, 2.0)
     yd = y.to(DEV).requires_grad_()
-    got = LP.layer_pre(yd, H, D, cq, ck, cv, cb, ct, nq, nk, nv, 2.0)
+    got = LP.layer_pre(yd, H, D, cq, ck, cv, cb, ct, (ldy - ct,) if ct < ldy else (), nq, nk, nv, 2.0)
+    got = tuple(got) + (None,) * (5 - len(got))
     cot = [torch.randn(t.shape, generator=g).to(dtype) if t is not None else None for t in ref]
     live = [i for i, t in enumerate(ref) if t is not None]
     (dref,) = torch.autograd.grad([ref[i] for i in live], yo, [cot[i].double() for i in live])
@@ -100,8 +101,8 @@ def test_logsigmoid(dtype):
 
 def test_empty_input():
     y = torch.empty(0, 3 * 128 + 8, device=DEV, dtype=torch.bfloat16)
-    q, k, v, beta, tail = LP.layer_pre(y, 2, 64, 0, 128, 256, 384, 386, False, True, False, 2.0)
-    assert q.shape == (0, 2, 64) and beta.shape == (0, 2, 1) and tail.shape == (0, 6)
+    q, k, v, beta, t0, t1 = LP.layer_pre(y, 2, 64, 0, 128, 256, 384, 386, (2, 4), False, True, False, 2.0)
+    assert q.shape == (0, 2, 64) and beta.shape == (0, 2, 1) and t0.shape == (0, 2) and t1.shape == (0, 4)
     assert LP.logsigmoid(torch.empty(0, 8, device=DEV)).shape == (0, 8)
 
 
