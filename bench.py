@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the HDLA rank-2 DPLR delta-rule hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload train|fwd|varlen|decode|copy|hdla|hdla_decode|norm|layer] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload train|fwd|varlen|decode|copy|hdla|hdla_decode|norm|layer|layer_decode] [--no-cpu-baseline]
 
 Default workload ("train") is the headline configuration: chunked forward + backward at B=4, T=2048, H=16,
 K=V=64, bf16 inputs, fp32 state, random fp32 initial state, upstream gradients do and dht (configuration 2).
@@ -35,7 +35,7 @@ def _args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="train", choices=["train", "fwd", "varlen", "decode", "copy", "hdla", "hdla_decode", "norm", "layer"])
+    ap.add_argument("--workload", default="train", choices=["train", "fwd", "varlen", "decode", "copy", "hdla", "hdla_decode", "norm", "layer", "layer_decode"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     return ap.parse_args()
 
@@ -226,6 +226,34 @@ def main():
             mixes[f"{nr}:{nw}"] = round((nr + nw) * n / sec / 1e9)
         print(json.dumps({"metric": "copy calibration", "bytes_read_per_launch": n, "bytes_written_per_launch": n,
                           "ms_per_step": sec * 1e3, "GB/s": 2 * n / sec / 1e9, "GB/s_by_read_write_mix": mixes}))
+        return
+    if wl == "layer_decode":
+        # One cached decode step of the whole HDLA_Custom layer on the layer shape of configuration 4: embed_dim =
+        # H*K = 4096, 32 heads of 128, 256 sequences, one token each per call, fp32 state carried in the cache.
+        from hdla_hip.layer import HDLA_Custom, RecurrentCache
+        B, H, D = 256, 32, 128
+        d = H * D
+        torch.manual_seed(0)
+        m = HDLA_Custom(d, H, token_mixer_init_type=2, rescale_type=0).to(dev).bfloat16().eval()
+        xs = [torch.randn(B, 1, d, device=dev, dtype=torch.bfloat16) for _ in range(8)]
+        st = {"cache": RecurrentCache(), "i": 0}
+        with torch.no_grad():
+            _, st["cache"] = m(torch.randn(B, 16, d, device=dev, dtype=torch.bfloat16), past_key_values=st["cache"], use_cache=True)
+
+            def step():
+                st["i"] += 1
+                _, st["cache"] = m(xs[st["i"] % 8], past_key_values=st["cache"], use_cache=True)
+            sec = time_steps(step, args.steps, args.warmup)
+        state_bytes = 2 * B * H * D * D * 4
+        print(json.dumps({"metric": "HDLA layer decode tokens/s", "value": B / sec, "unit": "tokens/s", "n_gpus": 1,
+                          "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3, "higher_is_better": True,
+                          "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                          "config": {"workload": "HDLA_Custom layer, embed_dim 4096, 32 heads of 128, 256 sequences, one "
+                                                 "token per call, state carried in the cache", "batch": B},
+                          "roofline": {"bound": "hbm", "kernel": "whole step (recurrent_kernel streams the state; weights 137 MB)",
+                                       "achieved": (state_bytes + 137e6) / sec / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                       "frac": (state_bytes + 137e6) / sec / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                                       "note": "state read + written once and every weight read once, over the step's wall time"}}))
         return
     if wl == "layer":
         # The whole HDLA token mixer (projections, activations, normalisations, the operator, output gate and

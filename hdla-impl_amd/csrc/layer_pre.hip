@@ -223,7 +223,8 @@ static int pre_config(const hdla_pre_dims* d, PreArgs& a, unsigned& nwg) {
     a.nsg = (a.nslot + rpw - 1) / rpw;
     a.norm_q = d->norm_q != 0; a.norm_k = d->norm_k != 0; a.norm_v = d->norm_v != 0;
     a.beta_scale = d->beta_scale; a.eps_d = d->eps * (float)d->D;
-    long long w = (a.nsg + 15) / 16;
+    const long long per_wave = a.nsg >= 16384 ? 4 : 1;          // passes per wavefront; few when the problem is small
+    long long w = (a.nsg + 4 * per_wave - 1) / (4 * per_wave);
     nwg = (unsigned)(w < 1 ? 1 : (w > 8192 ? 8192 : w));
     return HDLA_OK;
 }

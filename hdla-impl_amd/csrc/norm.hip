@@ -344,10 +344,13 @@ static int norm_config(const hdla_norm_dims* d, bool bwd, NormCfg& c) {
     if (pieces > 256 * 8) return HDLA_ERR_SHAPE;                // a group lives in one workgroup's registers
     if (d->rows > (1LL << 40) / d->G) return HDLA_ERR_SHAPE;
     c.nslot = d->rows * d->G;
-    c.wg_row = pieces > 64 * 8;
+    // long groups always, and groups of at least 128 pieces when there are too few of them to fill the chip one
+    // wavefront each (a decode step: a few hundred rows)
+    c.wg_row = pieces > 64 * 8 || (pieces >= 128 && c.nslot <= 2048);
     if (c.wg_row) {
-        // long groups: one per workgroup pass, 256 lanes across it
-        c.nv = pieces <= 256 * 4 ? 4 : 8;
+        // one group per workgroup pass, 256 lanes across it
+        c.nv = 1;
+        while (c.nv * 256 < pieces) c.nv *= 2;
         c.lpr_log2 = 8; c.rpw = 1; c.wg_reduce = 0;
         c.nsg = c.nslot;
     } else {
@@ -362,7 +365,8 @@ static int norm_config(const hdla_norm_dims* d, bool bwd, NormCfg& c) {
     }
     // a few passes per wavefront to amortise the weight loads, enough workgroups to fill the chip, and, backward, a
     // bound on the partial rows of the weight gradient; then a multiple of what keeps a lane on one weight column
-    const long long per_wave = 4, cap = bwd ? 1024 : 8192, owners = c.wg_row ? 1 : 4;
+    const long long cap = bwd ? 1024 : 8192, owners = c.wg_row ? 1 : 4;
+    const long long per_wave = c.nsg >= 4 * owners * 1024 ? 4 : (c.nsg >= 2 * owners * 1024 ? 2 : 1);
     long long nwg = (c.nsg + owners * per_wave - 1) / (owners * per_wave);
     if (nwg < 1) nwg = 1;
     if (nwg > cap) nwg = cap;

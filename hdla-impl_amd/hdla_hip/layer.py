@@ -182,6 +182,21 @@ class HDLA_Custom(nn.Module):
         return (f"embed_dim={self.embed_dim}, num_heads={self.num_heads}, num_blocks={self.num_blocks}, "
                 f"fuse_ab={self.fuse_ab}, dispatch={self.dispatch}")
 
+    def _gathered(self, heads):
+        """Weights (and biases) of the projections of x, concatenated.  With gradients the concatenation is part of
+        the graph; without (evaluation, decoding) it is built once and reused until a parameter changes."""
+        ps = [m.weight for m in heads] + ([m.bias for m in heads] if heads[0].bias is not None else [])
+        if torch.is_grad_enabled() and any(p.requires_grad for p in ps):
+            w = torch.cat([m.weight for m in heads], dim=0)
+            return w, (torch.cat([m.bias for m in heads], dim=0) if heads[0].bias is not None else None)
+        key = tuple((p.data_ptr(), p._version, p.dtype, p.device) for p in ps)
+        if getattr(self, "_gathered_key", None) != key:
+            with torch.no_grad():
+                w = torch.cat([m.weight for m in heads], dim=0)
+                b = torch.cat([m.bias for m in heads], dim=0) if heads[0].bias is not None else None
+            self._gathered_key, self._gathered_val = key, (w, b)
+        return self._gathered_val
+
     def _up(self, lin: nn.Linear, x0: torch.Tensor) -> torch.Tensor:
         """Second half of a low-rank projection (head_dim -> embed_dim)."""
         if self.fuse_pre and lin.bias is None and x0.is_cuda and x0.dtype == torch.bfloat16 == lin.weight.dtype:
@@ -201,8 +216,7 @@ class HDLA_Custom(nn.Module):
         heads.append(self.f_proj[0])
         if self.use_output_gate:
             heads.append(self.output_gate[0])
-        w = torch.cat([m.weight for m in heads], dim=0)
-        bias = torch.cat([m.bias for m in heads], dim=0) if heads[0].bias is not None else None
+        w, bias = self._gathered(heads)
         y = F.linear(x, w, bias)
         ldy, hd = y.shape[-1], self.head_dim
         if (self.fuse_pre and self._all_silu and self.num_blocks == 1 and lower_bound is None and x.is_cuda
