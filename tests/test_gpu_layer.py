@@ -111,3 +111,22 @@ def test_left_padding_mask():
         out, cache = m(x.to(DEV), attention_mask=mask.to(DEV), past_key_values=cache, use_cache=True)
     ro, rS, _ = _oracle(m, x, torch.zeros_like(x), H, attention_mask=mask)
     assert O.rel_l2(out, ro) <= 1e-5 and O.rel_l2(cache[0]["recurrent_state"][0], rS) <= 1e-5
+
+
+def test_autocast_training_step():
+    """fp32 parameters under torch.autocast(bfloat16), the usual mixed-precision set-up: the projections come out in
+    bf16, the kernels run in bf16, gradients arrive in fp32 on the parameters."""
+    d, H, n = 256, 4, 96
+    m = _layer(10, d, H, torch.float32).train()
+    x, do = _x(11, 2, n, d), _x(12, 2, n, d)
+    xd = x.to(DEV).requires_grad_()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out, _ = m(xd)
+    assert out.dtype == torch.bfloat16
+    params = dict(m.named_parameters())
+    g = torch.autograd.grad(out, [xd] + list(params.values()), do.to(DEV).bfloat16())
+    ro, _, rg = _oracle(m, x, do.bfloat16().float(), H)
+    assert O.rel_l2(out, ro) <= 1e-2
+    for name, got in zip(["x"] + list(params), g):
+        assert got.dtype == torch.float32
+        assert O.rel_l2(got, rg[name]) <= 2e-2, name
