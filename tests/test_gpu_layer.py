@@ -130,3 +130,22 @@ def test_autocast_training_step():
     for name, got in zip(["x"] + list(params), g):
         assert got.dtype == torch.float32
         assert O.rel_l2(got, rg[name]) <= 2e-2, name
+
+
+def test_half_precision_module_and_reference_dispatch_decode():
+    """fp16 parameters take the unfused elementwise path and fp32 kernels; with the reference's dispatch rule a cached
+    decode step runs through the chunked operator with one token (hdla_custom.py:295)."""
+    d, H, n, P = 256, 4, 40, 36
+    m = _layer(13, d, H, torch.float16, dispatch="reference").eval()
+    x = _x(14, 2, n, d).half()
+    ro, rS, _ = _oracle(m, x, torch.zeros_like(x), H)
+    cache = RecurrentCache()
+    with torch.no_grad():
+        out, cache = m(x[:, :P].to(DEV), past_key_values=cache, use_cache=True)
+        outs = [out]
+        for t in range(P, n):
+            out, cache = m(x[:, t:t + 1].to(DEV), past_key_values=cache, use_cache=True)
+            outs.append(out)
+    out = torch.cat(outs, 1)
+    assert out.dtype == torch.float16
+    assert O.rel_l2(out, ro) <= 5e-3 and O.rel_l2(cache[0]["recurrent_state"][0], rS) <= 5e-3
