@@ -8,7 +8,7 @@ elementwise stage between projections and operator, and the layer itself (HRDPLR
 from .chunk import ChunkDPLRDeltaRuleFunction, chunk_hrdplr_delta_rule
 from .hdla import ChunkHDLAFunction, chunk_hdla_delta_rule, fused_recurrent_hdla_delta_rule, parameterize_a_b
 from .layer import HDLA_Custom, RecurrentCache, get_activation_fn
-from .layer_pre import layer_pre, logsigmoid, low_rank_up
+from . import layer_pre          # submodule: layer_pre.layer_pre, .logsigmoid, .low_rank_up
 from .normalize import (GroupRMSNorm, GroupRMSNormFusedGate, NormalizeFunction, RMSNorm, RMSNormFusedGate, SRMSNorm,
                         get_norm_fn, l2_norm, normalize_fn)
 from .recurrent import FusedRecurrentDPLRDeltaRuleFunction, fused_recurrent_dplr_delta_rule
@@ -35,6 +35,4 @@ __all__ = [
     "RecurrentCache",
     "get_activation_fn",
     "layer_pre",
-    "logsigmoid",
-    "low_rank_up",
 ]

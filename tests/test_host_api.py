@@ -274,3 +274,11 @@ def test_recurrent_backward_is_not_implemented():
         _dtype = torch.float32
     with pytest.raises(NotImplementedError, match="only for inference"):
         hdla_hip.FusedRecurrentDPLRDeltaRuleFunction.backward(Ctx(), None, None)
+
+
+def test_package_exports_resolve():
+    import types
+    import hdla_hip
+    for name in hdla_hip.__all__:
+        assert hasattr(hdla_hip, name), name
+    assert isinstance(hdla_hip.layer_pre, types.ModuleType) and callable(hdla_hip.layer_pre.layer_pre)
