@@ -70,7 +70,8 @@ def measured_traffic(workload, kernel_key, K, V):
     FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the same counter reads for the streaming kernel of known traffic), or
     None when that summary does not cover the kernel.  The counters cannot be collected from inside this script."""
     try:
-        table = json.load(open(os.path.join(ROOT, "profiles", "hbm_traffic.json"))).get(workload, {})
+        # the forward-only workload runs the forward kernels of the training step on the same shape
+        table = json.load(open(os.path.join(ROOT, "profiles", "hbm_traffic.json"))).get("train" if workload == "fwd" else workload, {})
     except (OSError, ValueError):
         return None
     pass_, name = kernel_key.split(".") if "." in kernel_key else ("", kernel_key)
