@@ -104,6 +104,53 @@ def norm_traffic(rows):
         return None
 
 
+def layer_kernel_times(dev, steps):
+    """Event timing of single C-ABI calls of the layer's elementwise and weight-gradient kernels: the pre kernels
+    (q | k | v | beta column ranges of a [rows, 3216] projection output, 16 heads of 64), logsigmoid over [rows, 1024]
+    and the weight gradient dW [1024, 64] = dY^T X0.  Algorithmic bytes: every input read once, every output written
+    once."""
+    import ctypes
+    from hdla_hip import _lib
+    lib = _lib.load()
+    P, stream = _lib.ptr, _lib.current_stream(dev)
+    H, D, ldy = 16, 64, 3216
+    hd = H * D
+    res = {}
+    for tag, rows in (("config2", 8192), ("hbm", 262144)):
+        bf = lambda *shape: torch.randn(*shape, device=dev, dtype=torch.bfloat16)
+        y, dy = bf(rows, ldy), torch.empty(rows, ldy, device=dev, dtype=torch.bfloat16)
+        q, k, v, beta = bf(rows, hd), bf(rows, hd), bf(rows, hd), bf(rows, H)
+        f, lf = bf(rows, hd), torch.empty(rows, hd, device=dev, dtype=torch.bfloat16)
+        x0, dw = bf(rows, 2 * D)[:, :D], torch.empty(hd, D, device=dev, dtype=torch.bfloat16)
+        dims = _lib.HdlaPreDims(rows, H, D, 0, ldy, 0, hd, 2 * hd, 3 * hd, 0, 1, 0, 2.0, 1e-5)
+        nws = lib.hdla_skinny_wgrad_workspace_bytes(0, rows, D, hd)
+        ws = torch.empty(nws, dtype=torch.uint8, device=dev)
+        cols = (3 * hd + H) * 2
+        calls = {
+            "layer_pre_fwd": (lambda: lib.hdla_layer_pre_fwd(ctypes.byref(dims), P(y), P(q), P(k), P(v), P(beta), stream),
+                              2 * rows * cols),
+            "layer_pre_bwd": (lambda: lib.hdla_layer_pre_bwd(ctypes.byref(dims), P(y), P(q), P(k), P(v), P(beta), P(dy), stream),
+                              3 * rows * cols),
+            "logsigmoid_fwd": (lambda: lib.hdla_logsigmoid_fwd(0, rows * hd, P(f), P(lf), stream), 2 * rows * hd * 2),
+            "logsigmoid_bwd": (lambda: lib.hdla_logsigmoid_bwd(0, rows * hd, P(f), P(q), P(lf), stream), 3 * rows * hd * 2),
+            "skinny_wgrad": (lambda: lib.hdla_skinny_wgrad(0, rows, D, hd, P(f), hd, P(x0), 2 * D, P(dw), P(ws), nws, stream),
+                             rows * (hd + D) * 2 + hd * D * 2),
+        }
+        for name, (fn, nbytes) in calls.items():
+            _lib.check(fn(), name)
+            evs = []
+            for _ in range(steps):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(); _lib.check(fn(), name); e1.record()
+                evs.append((e0, e1))
+            torch.cuda.synchronize()
+            ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+            res.setdefault(name, {})[tag] = {"rows": rows, "ms": ms, "bytes": nbytes, "GB/s": nbytes / ms / 1e6,
+                                             "frac_hbm": nbytes / ms / 1e6 / HBM_PEAK_GBS}
+        del y, dy, q, k, v, f, lf, ws
+    return res
+
+
 def time_steps(fn, steps, warmup):
     for _ in range(warmup):
         fn()
@@ -259,8 +306,9 @@ def main():
     if wl == "layer":
         # The whole HDLA token mixer (projections, activations, normalisations, the operator, output gate and
         # projection) on the layer shape of configuration 2: embed_dim = H*K = 1024, 16 heads, B=4, T=2048, bf16
-        # parameters; forward + backward (gradients of x and of every parameter).  Whole-step rates only: the GEMMs are
-        # the BLAS library's, and the step is partly bound by the host issuing ~90 small launches.
+        # parameters; forward + backward (gradients of x and of every parameter).  `value` is the whole step (its GEMMs
+        # are the BLAS library's); "layer_kernels" times this library's kernels around the operator one by one through
+        # the C ABI, on the step's shape (cache-resident) and on 32x the rows (HBM), like the norm workload.
         from hdla_hip.layer import HDLA_Custom
         B, T, H, D = 4, 2048, 16, 64
         d = H * D
@@ -311,6 +359,7 @@ def main():
                                            "ms_per_step": out["fused_graph"] * 1e3, "value": B * T / out["fused_graph"]},
                           "plain_route": {"what": "same layer with fuse_ab=False: torch parameterize_a_b + the plain operator",
                                           "ms_per_step": out["plain_route"] * 1e3, "value": B * T / out["plain_route"]},
+                          "layer_kernels": layer_kernel_times(dev, args.steps),
                           "roofline": None}))
         return
     if wl == "norm":
