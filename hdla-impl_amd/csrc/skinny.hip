@@ -44,7 +44,7 @@ __global__ __launch_bounds__(256) void skinny_wgrad_kernel(const bf16* __restric
 #pragma unroll
         for (int b = 0; b < 2 * ZP; ++b) acc[a][b] = zero4();
     // the four wavefronts take every fourth 16-row tile of the range
-#pragma unroll 2
+#pragma unroll 4
     for (long long r0 = rbeg + 16 * w; r0 < rend; r0 += 64) {
         const bool ok = r0 + c < rend;
         const long long row = ok ? r0 + c : rbeg;              // a readable row on every lane
@@ -101,14 +101,16 @@ __global__ __launch_bounds__(256) void skinny_wgrad_sum_kernel(const float* __re
     *reinterpret_cast<u32x4*>(dW + i) = o;
 }
 
-// row ranges: enough workgroups for the chip, whole 16-row tiles each
+// row ranges: enough workgroups for the chip (and, when there are many rows, several per CU, about 1024 rows each, so
+// that enough loads are in flight to cover the latency of HBM), whole 16-row tiles each
 static int wgrad_split(long long M, int K, int& rows_per) {
     const int kb = K / 32;
     long long S = (256 + kb - 1) / kb;
+    const long long by_rows = M / 1024, most = (2048 + kb - 1) / kb;
+    if (by_rows > S) S = by_rows < most ? by_rows : most;
     const long long tiles = (M + 15) / 16;
     if (S > tiles) S = tiles;
     if (S < 1) S = 1;
-    if (S > 64) S = 64;
     rows_per = (int)(((tiles + S - 1) / S) * 16);
     return (int)((M + rows_per - 1) / rows_per);
 }
