@@ -12,6 +12,10 @@ CPU oracle timed on this box's host cores on a bounded sample.
 
 Per-kernel durations are measured live with events on the stream the kernels run on, in a second loop of the
 same number of steps that launches the same kernels one at a time through hdla_chunk_stages.
+
+Other workloads: fwd (configuration 1), varlen (3), decode (4); copy (the streaming kernel: counter calibration and
+attainable HBM rates); hdla, hdla_decode (the operators with a, b formed in the kernels, against building a, b in
+torch); norm (gated RMS norm forward + backward); layer, layer_decode (the whole HDLA_Custom layer).
 """
 import argparse
 import ctypes
