@@ -16,8 +16,10 @@ Same constructor arguments, parameter names (so a reference ``state_dict`` loads
 
 Which operator runs: the reference uses the chunked one when training or when ``use_cache`` is set and the token-serial
 one otherwise (hdla_custom.py:295,310); ``dispatch="reference"`` keeps that.  The default ``dispatch="auto"`` uses the
-chunked operator when gradients are needed or the call carries at least 64 tokens and the token-serial one for short
-calls (decode steps), which is where each is the faster; both compute the same function.
+chunked operator when gradients are needed or the call carries more than 8 tokens and the token-serial one for shorter
+calls (decode steps, short bursts), which is where each is the faster (at 8 tokens they take the same time from
+B=1, H=16 to B=256, H=32; at 1 token the token-serial one is 1.5-2.3x faster, at 64 tokens the chunked one 3x); both
+compute the same function.
 
 ``past_key_values`` is duck-typed on the three calls the reference makes (hdla_custom.py:254-257, 332-337):
 ``len(cache)``, ``cache[layer_idx]["recurrent_state"][0]``, ``cache.get_seq_length(layer_idx)`` and
@@ -37,7 +39,7 @@ from .normalize import get_norm_fn, l2_norm
 from .recurrent import fused_recurrent_dplr_delta_rule
 
 EMBED_DIM_BASE = 256                 # HRDPLR/normalizations/normalization_utils.py:14
-RECURRENT_BELOW = 64                 # dispatch="auto": calls shorter than this run token by token
+RECURRENT_BELOW = 9                  # dispatch="auto": calls shorter than this run token by token (measured crossover: 8)
 
 
 def get_activation_fn(activation: str) -> Callable[[torch.Tensor], torch.Tensor]:
