@@ -261,7 +261,7 @@ __global__ __launch_bounds__(256) void normalize_bwd_kernel(NormArgs p) {
         long long prow = L.wave * L.rpw + L.rw;
         if (p.wg_reduce) {
             // lane by lane the four wavefronts hold the same columns: waves 2, 3 hand over to 0, 1, then 1 to 0
-            __shared__ float sred[2 * NV * N * 64];
+            __shared__ float swg[2 * NV * N * 64];
             const int wl = threadIdx.x >> 6, lane = threadIdx.x & 63;
 #pragma unroll
             for (int round = 0; round < 2; ++round) {
@@ -270,14 +270,14 @@ __global__ __launch_bounds__(256) void normalize_bwd_kernel(NormArgs p) {
 #pragma unroll
                     for (int i = 0; i < NV; ++i)
 #pragma unroll
-                        for (int j = 0; j < N; ++j) sred[((wl - half) * NV * N + i * N + j) * 64 + lane] = dw[i][j];
+                        for (int j = 0; j < N; ++j) swg[((wl - half) * NV * N + i * N + j) * 64 + lane] = dw[i][j];
                 }
                 __syncthreads();
                 if (wl < half) {
 #pragma unroll
                     for (int i = 0; i < NV; ++i)
 #pragma unroll
-                        for (int j = 0; j < N; ++j) dw[i][j] += sred[(wl * NV * N + i * N + j) * 64 + lane];
+                        for (int j = 0; j < N; ++j) dw[i][j] += swg[(wl * NV * N + i * N + j) * 64 + lane];
                 }
                 __syncthreads();
             }
