@@ -149,3 +149,29 @@ def test_half_precision_module_and_reference_dispatch_decode():
     out = torch.cat(outs, 1)
     assert out.dtype == torch.float16
     assert O.rel_l2(out, ro) <= 5e-3 and O.rel_l2(cache[0]["recurrent_state"][0], rS) <= 5e-3
+
+
+def test_against_the_committed_fixture():
+    """The module loaded with the fixture's parameters (embed_dim 32, 4 heads of 8: padded head size) against
+    tests/golden/layer0.npz, and the normalisation kernels against the same file."""
+    import os
+    import sys
+    import numpy as np
+    from hdla_hip import normalize as NZ
+    sys.path.insert(0, os.path.join(os.path.dirname(__file__), "golden"))
+    from make_golden import layer_case
+    sd, x, gate, H = layer_case()
+    fix = np.load(os.path.join(os.path.dirname(__file__), "golden", "layer0.npz"))
+    m = HDLA_Custom(32, H, rescale_type=0)
+    m.load_state_dict({k: v.float() for k, v in sd.items()})
+    m = m.to(DEV).eval()
+    cache = RecurrentCache()
+    with torch.no_grad():
+        out, cache = m(x.float().to(DEV), past_key_values=cache, use_cache=True)
+    assert O.rel_l2(out, torch.from_numpy(fix["layer_out"])) <= 1e-5
+    assert O.rel_l2(cache[0]["recurrent_state"][0], torch.from_numpy(fix["layer_state"])) <= 1e-5
+    xf, gf, wf = x.float().to(DEV), gate.float().to(DEV), sd["norm.weight"].float().to(DEV)
+    assert O.rel_l2(NZ.normalize_fn(xf, wf, gate=gf, c=32 ** 0.5, eps=1e-5), torch.from_numpy(fix["rms_gate_pre"])) <= 1e-5
+    assert O.rel_l2(NZ.normalize_fn(xf, wf, gate=gf, gate_pos="post", c=8 ** 0.5, eps=1e-3, num_groups=4),
+                    torch.from_numpy(fix["group_post"])) <= 1e-5
+    assert O.rel_l2(NZ.l2_norm(xf.reshape(2, 10, 4, 8)), torch.from_numpy(fix["l2"])) <= 1e-5

@@ -142,3 +142,22 @@ def test_gathered_projection_weight_is_cached_only_without_gradients():
     assert m._gathered(heads)[0] is b                                            # frozen parameters: cached with grad mode on
     m2 = m.to(torch.bfloat16)
     assert m2._gathered(heads)[0].dtype == torch.bfloat16                        # new storage, new entry
+
+
+def test_golden_fixture_layer0():
+    """Seeded fixture of the normalisation and layer oracles (tests/golden/layer0.npz, written by
+    tests/golden/make_golden.py from this repository's own float64 code): guards the oracles against drift."""
+    import os
+    import sys
+    import numpy as np
+    sys.path.insert(0, os.path.join(os.path.dirname(__file__), "golden"))
+    from make_golden import layer_case
+    sd, x, gate, H = layer_case()
+    fix = np.load(os.path.join(os.path.dirname(__file__), "golden", "layer0.npz"))
+    out, S = LO.hdla_layer(sd, x, H)
+    close = lambda a, name: np.testing.assert_allclose(a.numpy(), fix[name], rtol=1e-12, atol=1e-12)
+    close(out, "layer_out")
+    close(S, "layer_state")
+    close(NO.rms_norm_fused_gate(x, gate, sd["norm.weight"], eps=1e-5), "rms_gate_pre")
+    close(NO.normalize(x, sd["norm.weight"], gate, "sigmoid", "post", c=8 ** 0.5, eps=1e-3, num_groups=4), "group_post")
+    close(NO.l2_norm(x.reshape(2, 10, 4, 8)), "l2")
