@@ -86,6 +86,7 @@ class LayerPreFunction(torch.autograd.Function):
         return (dy,) + (None,) * 13
 
 
+@torch.compiler.disable
 def layer_pre(y, H, D, col_q, col_k, col_v, col_beta, col_tail, tail_widths, norm_q, norm_k, norm_v, beta_scale,
               eps=1e-5):
     """y [rows, ldy] -> q, k, v [rows, H, D], beta [rows, H, 1] (None when col_beta < 0), then one contiguous copy per
@@ -123,6 +124,7 @@ class LogSigmoidFunction(torch.autograd.Function):
         return dx
 
 
+@torch.compiler.disable
 def logsigmoid(x: torch.Tensor) -> torch.Tensor:
     """log(sigmoid(x)) elementwise; the element count must be a multiple of 16 bytes' worth."""
     _require_gpu(x)
@@ -168,6 +170,7 @@ class LowRankUpFunction(torch.autograd.Function):
         return dx0, dw
 
 
+@torch.compiler.disable
 def low_rank_up(x0: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """``x0 [..., head_dim] @ weight[embed_dim, head_dim]^T`` with this library's kernel for the weight gradient."""
     return LowRankUpFunction.apply(x0, weight)

@@ -75,6 +75,7 @@ class NormalizeFunction(torch.autograd.Function):
         return dx, dw, dgate, None, None, None, None
 
 
+@torch.compiler.disable
 def normalize_fn(
     x: torch.Tensor,
     weight: Optional[torch.Tensor] = None,
