@@ -13,6 +13,13 @@
  *   hdla_recurrent_fwd  <-  fused_recurrent_dplr_delta_rule_fwd   HRDPLR/recurrent.py:121-177
  *   hdla_param_*        <-  the same three with parameterize_a_b (HRDPLR/hdla_custom.py:19-43) folded in
  *
+ * and, for the layer around the operator (HRDPLR/hdla_custom.py:45-350):
+ *
+ *   hdla_normalize_*    <-  NormalizeTriton   HRDPLR/normalizations/normalize/normalize/normalize_triton.py:255-449
+ *   hdla_layer_pre_*, hdla_logsigmoid_*   <-  the elementwise steps between projections and operator
+ *                                             HRDPLR/hdla_custom.py:214-251
+ *   hdla_skinny_wgrad   <-  the weight gradient of the low-rank up-projections (a BLAS call inside autograd)
+ *
  * Conventions
  *   - All tensor pointers are DEVICE pointers to contiguous, 16-byte aligned buffers owned by the caller.
  *     Layouts are the reference's (head_first = False): q,k,gk [B,T,H,K]; v,o,do [B,T,H,V];
