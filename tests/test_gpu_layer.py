@@ -23,6 +23,9 @@ def _layer(seed, d, H, dtype, **kw):
             p.mul_(4.0)                                   # spread decays and gates away from 1/2
         for p in (m.q_proj.weight, m.k_proj.weight, m.v_proj.weight):
             p.mul_(3.0)
+        for name, p in m.named_parameters():
+            if name.endswith(".bias"):
+                p.normal_(0.0, 0.2)
     return m.to(DEV).to(dtype)
 
 
@@ -43,6 +46,8 @@ def _oracle(m, x, do, H, **kw):
     (torch.float32, 256, 4, 80, {}),
     (torch.float32, 256, 2, 37, {"num_blocks": 2, "norm_q": True, "norm_v": True}),
     (torch.float32, 192, 3, 50, {"use_beta": False, "use_output_gate": False, "use_offset": True}),
+    (torch.float32, 256, 4, 40, {"bias": True}),
+    (torch.bfloat16, 256, 4, 64, {"bias": True}),
     (torch.bfloat16, 512, 8, 128, {}),
     (torch.bfloat16, 512, 8, 128, {"fuse_pre": False}),
     (torch.float32, 256, 4, 80, {"fuse_pre": False, "fuse_ab": False}),
@@ -64,7 +69,10 @@ def test_training_step_against_the_oracle(dtype, d, H, n, kw):
     print(dtype, d, H, n, kw, {k: f"{v:.1e}" for k, v in errs.items()}, flush=True)
     assert errs.pop("out") <= tol_o
     for k_, e in errs.items():
-        assert e <= tol_g, (k_, e)
+        # the bias of beta's projection has one entry per head, each the sum over all tokens of per-token gradients
+        # that largely cancel: in bf16 the relative error of such a sum is several times the per-token error (5e-2 here,
+        # and the same with torch's elementwise operators and the plain operator in place of this library's kernels)
+        assert e <= (5 * tol_g if k_ == "bet_proj.bias" and dtype == torch.bfloat16 else tol_g), (k_, e)
 
 
 @pytest.mark.parametrize("dispatch,fuse_ab", [("auto", True), ("reference", True), ("auto", False), ("reference", False)])
