@@ -183,3 +183,27 @@ def test_against_the_committed_fixture():
     assert O.rel_l2(NZ.normalize_fn(xf, wf, gate=gf, gate_pos="post", c=8 ** 0.5, eps=1e-3, num_groups=4),
                     torch.from_numpy(fix["group_post"])) <= 1e-5
     assert O.rel_l2(NZ.l2_norm(xf.reshape(2, 10, 4, 8)), torch.from_numpy(fix["l2"])) <= 1e-5
+
+
+def test_full_size_split_run_equals_one_pass():
+    """Configuration 2's layer shape (B=4, T=2048, embed_dim 1024, 16 heads, bf16), where the oracle's token loop is
+    too slow: a run split at an odd position that carries the state through the cache, followed by eight single-token
+    steps, must reproduce one pass over the whole sequence (state hand-over and both operators at full size)."""
+    d, H, B, T, P = 1024, 16, 4, 2048, 1037
+    m = _layer(15, d, H, torch.bfloat16).eval()
+    x = _x(16, B, T, d).bfloat16().to(DEV)
+    with torch.no_grad():
+        ref, c0 = m(x, past_key_values=RecurrentCache(), use_cache=True)
+        cache = RecurrentCache()
+        o1, cache = m(x[:, :P], past_key_values=cache, use_cache=True)
+        o2, cache = m(x[:, P:T - 8], past_key_values=cache, use_cache=True)
+        outs = [o1, o2]
+        for t in range(T - 8, T):
+            o, cache = m(x[:, t:t + 1], past_key_values=cache, use_cache=True)
+            outs.append(o)
+    out = torch.cat(outs, 1)
+    assert cache.get_seq_length(0) == T
+    e_o = O.rel_l2(out, ref.double().cpu())
+    e_s = O.rel_l2(cache[0]["recurrent_state"][0], c0[0]["recurrent_state"][0].double().cpu())
+    print(f"full-size split run: out {e_o:.2e} state {e_s:.2e}", flush=True)
+    assert e_o <= 5e-3 and e_s <= 5e-3
