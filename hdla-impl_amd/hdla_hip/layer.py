@@ -185,10 +185,13 @@ class HDLA_Custom(nn.Module):
                 f"fuse_ab={self.fuse_ab}, dispatch={self.dispatch}")
 
     def _gathered(self, heads):
-        """Weights (and biases) of the projections of x, concatenated.  With gradients the concatenation is part of
-        the graph; without (evaluation, decoding) it is built once and reused until a parameter changes."""
+        """Weights (and biases) of the projections of x, concatenated.  With gradients, or in training mode, the
+        concatenation is rebuilt per call (and is part of the graph).  In evaluation mode without gradients it is built
+        once and reused: it is rebuilt when a parameter is replaced or modified in place (tracked by its version
+        counter), on ``.train()`` / ``.eval()``, ``.to()`` and ``load_state_dict``, and by ``reset_cache()`` -- which
+        is what code that writes through ``param.data`` (untracked) has to call."""
         ps = [m.weight for m in heads] + ([m.bias for m in heads] if heads[0].bias is not None else [])
-        if torch.is_grad_enabled() and any(p.requires_grad for p in ps):
+        if self.training or (torch.is_grad_enabled() and any(p.requires_grad for p in ps)):
             w = torch.cat([m.weight for m in heads], dim=0)
             return w, (torch.cat([m.bias for m in heads], dim=0) if heads[0].bias is not None else None)
         key = tuple((p.data_ptr(), p._version, p.dtype, p.device) for p in ps)
@@ -198,6 +201,22 @@ class HDLA_Custom(nn.Module):
                 b = torch.cat([m.bias for m in heads], dim=0) if heads[0].bias is not None else None
             self._gathered_key, self._gathered_val = key, (w, b)
         return self._gathered_val
+
+    def reset_cache(self):
+        """Forget the concatenated projection weight of evaluation mode."""
+        self._gathered_key = self._gathered_val = None
+
+    def train(self, mode: bool = True):
+        self.reset_cache()
+        return super().train(mode)
+
+    def _apply(self, fn, *args, **kwargs):
+        self.reset_cache()
+        return super()._apply(fn, *args, **kwargs)
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        self.reset_cache()
+        return super()._load_from_state_dict(*args, **kwargs)
 
     def _up(self, lin: nn.Linear, x0: torch.Tensor) -> torch.Tensor:
         """Second half of a low-rank projection (head_dim -> embed_dim)."""

@@ -126,20 +126,34 @@ def test_recurrent_cache_contract():
     assert len(c) == 2 and c[0]["recurrent_state"][0] == "S0b" and c.get_seq_length(0) == 6 and c.get_seq_length(1) == 5
 
 
-def test_gathered_projection_weight_is_cached_only_without_gradients():
+def test_gathered_projection_weight_is_cached_only_in_evaluation_mode_without_gradients():
     m = HDLA_Custom(64, 4)
     heads = [m.q_proj, m.k_proj, m.v_proj, m.bet_proj, m.f_proj[0], m.output_gate[0]]
     w1, _ = m._gathered(heads)
     assert w1.requires_grad and w1.shape == (3 * 64 + 4 + 16 + 16, 64)          # part of the graph: rebuilt per call
     assert m._gathered(heads)[0] is not w1
     with torch.no_grad():
+        assert m._gathered(heads)[0] is not m._gathered(heads)[0]                # training mode: never cached
+        m.eval()
         a, _ = m._gathered(heads)
         assert m._gathered(heads)[0] is a and not a.requires_grad                # reused
         m.k_proj.weight.mul_(2.0)                                                # a parameter changes in place
         b, _ = m._gathered(heads)
         assert b is not a and torch.equal(b[64:128], m.k_proj.weight)
+        m.k_proj.weight.data.mul_(0.5)                                           # untracked write: needs reset_cache()
+        assert m._gathered(heads)[0] is b
+        m.reset_cache()
+        c, _ = m._gathered(heads)
+        assert c is not b and torch.equal(c[64:128], m.k_proj.weight)
+        m.train()
+        m.eval()                                                                 # mode switches drop it too
+        assert m._gathered(heads)[0] is not c
+        d = m._gathered(heads)[0]
+        m.load_state_dict({k: v.clone() for k, v in m.state_dict().items()})
+        assert m._gathered(heads)[0] is not d
     m.requires_grad_(False)
-    assert m._gathered(heads)[0] is b                                            # frozen parameters: cached with grad mode on
+    e = m._gathered(heads)[0]
+    assert m._gathered(heads)[0] is e                                            # frozen parameters: cached with grad mode on
     m2 = m.to(torch.bfloat16)
     assert m2._gathered(heads)[0].dtype == torch.bfloat16                        # new storage, new entry
 
