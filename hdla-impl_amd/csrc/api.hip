@@ -3,6 +3,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "hdla_launch.h"
 #include "hdla_ws.h"
 
@@ -154,6 +156,30 @@ int run_chunk(const hdla_dims* d, int pass, const void* q, const void* k, const 
 
 }  // namespace
 
+// ---- scratch memory of the entry point that allocates nothing ------------------------------------------------
+// One array per GPU, part of the loaded code object, held until the process ends.  In host code the array's name is
+// only a handle for hipGetSymbolAddress; the address kernels can use is looked up once per device and kept here.
+// (No `used` attribute on the array: with it the compiler keeps the symbol local to the code object, where the runtime's
+// lookup by name fails; the host-side reference below is what keeps the array and makes its symbol visible.)
+static __device__ __align__(256) unsigned char scratch[HDLA_STATIC_WORKSPACE_BYTES];
+static constexpr int MAX_DEVICES = 64;
+static std::atomic<void*> g_scratch_ptr[MAX_DEVICES];
+
+// Device address of `scratch` on the current device (looked up on the first call per device); nullptr and *err set
+// on failure.  Two threads racing on the first call both obtain the same address.
+static void* static_scratch(int* err) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { *err = (int)e; return nullptr; }
+    if (dev < 0 || dev >= MAX_DEVICES) { *err = HDLA_ERR_SHAPE; return nullptr; }
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p) return p;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) { *err = e != hipSuccess ? (int)e : HDLA_ERR_WORKSPACE; return nullptr; }
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+    return p;
+}
+
 extern "C" {
 
 int hdla_version(void) { return HDLA_VERSION; }
@@ -168,6 +194,7 @@ const char* hdla_strerror(int code) {
         case HDLA_ERR_WORKSPACE: return "workspace is NULL, not 256-byte aligned, or smaller than hdla_workspace_bytes()";
         case HDLA_ERR_ALIGN: return "tensor pointers must be 16-byte aligned";
         case HDLA_ERR_SEQ: return "cu_seqlens needs B == 1; without it N must equal B";
+        case HDLA_ERR_STATIC_LIMIT: return "the call needs more scratch memory than the built-in HDLA_STATIC_WORKSPACE_BYTES; use hdla_chunk_fwd with a caller-owned workspace";
         default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error code";
     }
 }
@@ -212,6 +239,19 @@ int hdla_chunk_fwd(const hdla_dims* dims, const void* q, const void* k, const vo
                                nullptr, nullptr, nullptr, nullptr, workspace, workspace_bytes, s);
     return run_chunk<float>(dims, 0, q, k, v, a, b, gk, h0, o, ht, nullptr, nullptr, nullptr, nullptr, nullptr,
                             nullptr, nullptr, nullptr, nullptr, workspace, workspace_bytes, s);
+}
+
+int hdla_chunk_fwd_static(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
+                          const void* b, const void* gk, const float* h0, void* o, float* ht, void* stream) {
+    const size_t need = hdla_workspace_bytes(dims, 0);
+    if (need == 0) { const int rc = check_dims(dims); return rc ? rc : HDLA_ERR_SHAPE; }
+    if (need > (size_t)HDLA_STATIC_WORKSPACE_BYTES) return HDLA_ERR_STATIC_LIMIT;
+    int err = 0;
+    void* ws = static_scratch(&err);
+    if (!ws) return err;
+    // every byte of the workspace that a kernel of the forward pass reads has been written by an earlier kernel of
+    // the same call, so nothing has to be cleared between calls
+    return hdla_chunk_fwd(dims, q, k, v, a, b, gk, h0, o, ht, ws, (size_t)HDLA_STATIC_WORKSPACE_BYTES, stream);
 }
 
 int hdla_chunk_bwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,

@@ -73,6 +73,8 @@ def load():
     lib.hdla_workspace_layout.argtypes = [F, ctypes.c_int, ctypes.POINTER(HdlaWsLayout)]
     lib.hdla_chunk_fwd.restype = ctypes.c_int
     lib.hdla_chunk_fwd.argtypes = [F] + [P] * 9 + [P, ctypes.c_size_t, P]
+    lib.hdla_chunk_fwd_static.restype = ctypes.c_int
+    lib.hdla_chunk_fwd_static.argtypes = [F] + [P] * 9 + [P]
     lib.hdla_chunk_bwd.restype = ctypes.c_int
     lib.hdla_chunk_bwd.argtypes = [F] + [P] * 16 + [P, ctypes.c_size_t, P]
     lib.hdla_param_chunk_fwd.restype = ctypes.c_int

@@ -56,7 +56,8 @@ enum {
     HDLA_ERR_DTYPE = -4,       /* unknown dtype code or unsupported combination */
     HDLA_ERR_WORKSPACE = -5,   /* workspace NULL, misaligned or too small */
     HDLA_ERR_ALIGN = -6,       /* a tensor pointer is not 16-byte aligned */
-    HDLA_ERR_SEQ = -7          /* cu_seqlens given with B != 1, or N inconsistent with B */
+    HDLA_ERR_SEQ = -7,         /* cu_seqlens given with B != 1, or N inconsistent with B */
+    HDLA_ERR_STATIC_LIMIT = -8 /* hdla_chunk_fwd_static: the shape needs more than HDLA_STATIC_WORKSPACE_BYTES */
 };
 
 typedef struct hdla_dims {
@@ -95,6 +96,20 @@ int hdla_workspace_layout(const hdla_dims* dims, int pass, hdla_ws_layout* out);
 int hdla_chunk_fwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
                    const void* b, const void* gk, const float* h0, void* o, float* ht,
                    void* workspace, size_t workspace_bytes, void* stream);
+
+/* hdla_chunk_fwd for callers that cannot allocate device memory and have no workspace to pass: code under HIP graph
+ * capture, tight serving loops (a prefill or a burst of a few tokens per sequence), harnesses that forbid
+ * hipMalloc.  It has no counterpart in the reference.  Same arguments and results as hdla_chunk_fwd without the
+ * workspace: the kernels use an array of HDLA_STATIC_WORKSPACE_BYTES bytes that is part of the library's device
+ * code (every GPU the library runs on holds it until the process ends); the call allocates and frees nothing.
+ * A shape whose hdla_workspace_bytes(dims, 0) exceeds that size is refused with HDLA_ERR_STATIC_LIMIT (K = V = 64,
+ * bf16: up to 3276 (16-token chunk, head) pairs, e.g. one sequence of 3276 tokens with 16 heads).  All calls on
+ * one GPU share the array: calls that may overlap on one GPU (different streams, different threads) race; calls
+ * on one stream are safe.  The array's device address is looked up on the first call on each device; make that
+ * call outside graph capture. */
+#define HDLA_STATIC_WORKSPACE_BYTES (64u << 20)
+int hdla_chunk_fwd_static(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
+                          const void* b, const void* gk, const float* h0, void* o, float* ht, void* stream);
 
 /* Chunked backward (HRDPLR/hrdplr.py:149-284): recomputes the forward intermediates from the inputs, then
  * writes dq,dk,dv,da,db (in_dtype), dgk (gk_dtype) and, if dh0 != NULL, dh0 (fp32).  dht may be NULL. */
