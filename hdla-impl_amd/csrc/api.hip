@@ -68,6 +68,7 @@ int make_layout(const hdla_dims* d, int pass, WsLayout& L, int& nch) {
         L.HC = take(chw * K * V * es);
         L.DHC = take(chw * K * V * es);
         L.DVN = take(chw * 2 * 16 * V * es);
+        L.STRONG = take(chw * 4);
     }
     if (d->cu_seqlens) {
         L.CHUNK_OFF = take((size_t)(d->N + 1) * 4);
@@ -87,6 +88,7 @@ void bind_ws(ChunkArgs<T>& a, const hdla_dims* d, const WsLayout& L, int nch, vo
     a.ws.HC = at(L.HC); a.ws.DHC = at(L.DHC); a.ws.DVN = at(L.DVN);
     a.ws.EGL = reinterpret_cast<float*>(base + L.EGL);
     a.ws.TM = reinterpret_cast<T*>(base + L.TM);
+    a.ws.STRONG = reinterpret_cast<int32_t*>(base + L.STRONG);
     a.st.cu = d->cu_seqlens;
     a.st.chunk_off = d->cu_seqlens ? reinterpret_cast<const int32_t*>(base + L.CHUNK_OFF) : nullptr;
     a.st.chunk_seq = d->cu_seqlens ? reinterpret_cast<const int32_t*>(base + L.CHUNK_SEQ) : nullptr;
@@ -124,7 +126,7 @@ int run_chunk(const hdla_dims* d, int pass, const void* q, const void* k, const 
     hipError_t e;
     if (d->cu_seqlens && (stages & HDLA_STAGE_PREP)) {
         char* base = static_cast<char*>(workspace);
-        e = launch_chunk_table(d->cu_seqlens, d->N, nch, reinterpret_cast<int32_t*>(base + L.CHUNK_OFF),
+        e = launch_chunk_table(d->cu_seqlens, d->N, d->T, nch, reinterpret_cast<int32_t*>(base + L.CHUNK_OFF),
                                reinterpret_cast<int32_t*>(base + L.CHUNK_SEQ), stream);
         if (e != hipSuccess) return (int)e;
     }
@@ -219,7 +221,7 @@ int hdla_workspace_layout(const hdla_dims* dims, int pass, hdla_ws_layout* out) 
     out->QG = L.QG; out->AQK = L.AQK; out->AQB = L.AQB;
     out->AQBT = L.AQBT; out->QGT = L.QGT; out->TM = L.TM;
     out->SA_STRIDE = L.SA_STRIDE; out->SB_STRIDE = L.SB_STRIDE;
-    out->HC = L.HC; out->DHC = L.DHC; out->DVN = L.DVN;
+    out->HC = L.HC; out->DHC = L.DHC; out->DVN = L.DVN; out->STRONG = L.STRONG;
     out->CHUNK_OFF = L.CHUNK_OFF; out->CHUNK_SEQ = L.CHUNK_SEQ;
     out->total = L.total;
     return HDLA_OK;

@@ -76,6 +76,12 @@ __device__ __forceinline__ f32x4 to_f32(Frag<bf16> a) {
 }
 __device__ __forceinline__ f32x4 to_f32(Frag<float> a) { return a.v; }
 
+// Tells the optimiser that x may have changed (it has not, and no instruction is emitted): what is computed from x
+// after this point stays after it, in particular inside a loop in which x does not change, instead of being hoisted
+// out of the loop and kept in registers across it.
+__device__ __forceinline__ void pin(Frag<bf16>& x) { asm volatile("" : "+v"(x.v)); }
+__device__ __forceinline__ void pin(Frag<float>&) {}     // fp32 operands are used as they are: nothing to hoist
+
 __device__ __forceinline__ f32x4 zero4() { f32x4 z = {0.f, 0.f, 0.f, 0.f}; return z; }
 
 // ---- the tile product --------------------------------------------------------------------------------------
@@ -219,6 +225,13 @@ struct ChunkPos {
     int n;         // sequence
 };
 
+// Token rows [bos, eos) of packed sequence n, forced into 0 <= bos <= eos <= total: the table comes from the caller
+// and is not validated on the device, and no value in it may take an access outside the tensors.
+__device__ __forceinline__ void packed_bounds(const int64_t* cu, int n, int64_t total, int64_t& bos, int64_t& eos) {
+    bos = min(max(cu[n], (int64_t)0), total);
+    eos = min(max(cu[n + 1], bos), total);
+}
+
 __device__ __forceinline__ bool locate_chunk(const SeqTab& st, int cid, ChunkPos& cp) {
     if (st.cu == nullptr) {
         if (cid >= st.N * st.NT) return false;
@@ -231,10 +244,11 @@ __device__ __forceinline__ bool locate_chunk(const SeqTab& st, int cid, ChunkPos
     if (cid >= st.chunk_off[st.N]) return false;
     cp.n = st.chunk_seq[cid];
     const int ic = cid - st.chunk_off[cp.n];
-    const int64_t bos = st.cu[cp.n], eos = st.cu[cp.n + 1];
+    int64_t bos, eos;
+    packed_bounds(st.cu, cp.n, st.T, bos, eos);
     cp.tok0 = bos + (int64_t)ic * CH;
     cp.len = (int)min((int64_t)CH, eos - cp.tok0);
-    return true;
+    return cp.len > 0;
 }
 
 // chunk range [c0, c1) of sequence n
@@ -246,7 +260,7 @@ __device__ __forceinline__ void seq_chunks(const SeqTab& st, int n, int& c0, int
 // token rows [bos, eos) of sequence n on the flattened axis
 __device__ __forceinline__ void seq_bounds(const SeqTab& st, int n, int64_t& bos, int64_t& eos) {
     if (st.cu == nullptr) { bos = (int64_t)n * st.T; eos = bos + st.T; }
-    else { bos = st.cu[n]; eos = st.cu[n + 1]; }
+    else packed_bounds(st.cu, n, st.T, bos, eos);
 }
 
 // ---- per-chunk decay quantities in fragment layout ---------------------------------------------------------
@@ -286,6 +300,14 @@ __device__ __forceinline__ f32x4 bcast16(f32x4 x, int src) {  // value of lane `
     for (int i = 0; i < 4; ++i) r[i] = __shfl(x[i], src, 16);
     return r;
 }
+// the same with a compile-time source lane: one DPP move per register (row_newbcast), no LDS round trip
+template <int SRC> __device__ __forceinline__ f32x4 bcast16(f32x4 x) {
+    f32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        r[i] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x[i]), 0x150 + SRC, 0xf, 0xf, false));
+    return r;
+}
 // value held by the lane 32 positions away (v_permlane32_swap exchanges the two halves of the wave)
 __device__ __forceinline__ float xor32(float x) {
     const int xi = __float_as_int(x);
@@ -306,5 +328,66 @@ __device__ __forceinline__ float sum_groups(float x) {
     x += xor32(x);
     return x;
 }
+
+
+// ---- decay factors of the factorised score products --------------------------------------------------------------
+// A score sums q_i[ch] k_j[ch] exp(gi_i[ch] - gi_j[ch]) over channels (j <= i; likewise with a, ge on the row side and b
+// on the inner side).  To be a matrix product the decay must factorise: exp(gi_i - m) exp(m - gi_j) with a centre m per
+// channel.  One centre (gi of token MID) serves the whole 16 x 16 tile as long as no exponent gi_i - m, ge_i - m exceeds
+// SAFE_RANGE in magnitude: the factors then stay within e^+-70, inside the range of the element types with room for
+// the operands themselves.  Beyond that (a channel that loses more than e^-70 over eight tokens) exp(gi_i - m) would
+// overflow for pairs on one side of the centre, so the tile is assembled from three products whose exponents are all
+// <= 0 or bounded:
+//   pass 0: rows 8..15 x inner 0..7, centre token 7: gi_i - m <= 0 and m - gi_j <= 0, exact;
+//   pass 1: rows 0..7 x inner 0..7, centre token 3;      pass 2: rows 8..15 x inner 8..15, centre token 11:
+//           inside a half the per-token log-decay is clamped at -PASS_CLAMP first, so no exponent exceeds 4 tokens x
+//           PASS_CLAMP = 80.  A pair (i, j) whose span holds a clamped token has weight < e^-20 = 2e-9 either way, and
+//           every other pair is exact, so each weight is within 2e-9 (absolute) of its true value.
+// Tokens outside a pass's rows / inner range get the factor 0, and what the passes leave above the diagonal is removed
+// by the causal masks as before.
+constexpr float SAFE_RANGE = 70.f;
+constexpr float PASS_CLAMP = 20.f;
+
+template <int N> __device__ __forceinline__ bool strong_decay(const f32x4 (&gi)[N], const f32x4 (&ge)[N]) {
+    float big = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < N; ++kt) {
+        const f32x4 m = bcast16<MID>(gi[kt]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) big = fmaxf(big, fmaxf(fabsf(gi[kt][i] - m[i]), fabsf(ge[kt][i] - m[i])));
+    }
+    return __any(big > SAFE_RANGE) != 0;                 // the same answer on every lane of the wave
+}
+
+struct DecayPass {
+    static constexpr int COUNT = 3;
+    int centre;          // token whose cumulative decay centres the pass
+    bool rows, cols;     // does this lane's token take part on the row side (q, a) / on the inner side (k, b)
+    bool clamp;
+    __device__ __forceinline__ DecayPass(int ps, int c) {
+        centre = ps == 0 ? MID : ps == 1 ? MID / 2 : MID + (CH - MID) / 2;
+        rows = ps == 1 ? c <= MID : c > MID;
+        cols = ps == 2 ? c > MID : c <= MID;
+        clamp = ps != 0;
+    }
+    // gi, ge: inclusive / exclusive cumulative log-decay of the lane's token (four channels)
+    template <typename T> __device__ __forceinline__ void factors(f32x4 gi, f32x4 ge, f32x4& eq, f32x4& ek, f32x4& ea) const {
+        if (clamp) {                                      // uniform over the wave
+            f32x4 g = gi - ge;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) g[i] = fmaxf(g[i], -PASS_CLAMP);
+            gi = scan16_incl(g);
+            ge = gi - g;
+        }
+        const f32x4 m = bcast16(gi, centre);
+        const f32x4 z = zero4();
+        f32x4 dq = gi - m, dk = m - gi, da = ge - m;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { dq[i] = fminf(dq[i], 80.f); dk[i] = fminf(dk[i], 80.f); da[i] = fminf(da[i], 80.f); }
+        eq = rows ? exp4<T>(dq) : z;
+        ek = cols ? exp4<T>(dk) : z;
+        ea = rows ? exp4<T>(da) : z;
+    }
+};
 
 }  // namespace hdla

@@ -6,7 +6,7 @@
 
 namespace hdla {
 
-hipError_t launch_chunk_table(const int64_t* cu, int N, int nch, int32_t* chunk_off, int32_t* chunk_seq, hipStream_t stream);
+hipError_t launch_chunk_table(const int64_t* cu, int N, int T, int nch, int32_t* chunk_off, int32_t* chunk_seq, hipStream_t stream);
 
 // K, V in {64, 128}; returns hipErrorInvalidValue for any other pair.
 template <typename T> hipError_t launch_prep(const ChunkArgs<T>& a, int K, int V, bool bwd, hipStream_t stream);

@@ -86,6 +86,7 @@ struct WsLayout {
     size_t HC;     // tiles  [K/32][V/16] pairs  F(S^T), state entering the chunk: rows value, inner channel
     size_t DHC;    // tiles  [K/32][V/16] pairs  the same for the gradient of the state leaving the chunk
     size_t DVN;    // tiles  [V/16] pairs        F(dv_new_s^T), the two ranks paired: rows value, inner token
+    size_t STRONG; // int32  [1]         nonzero: a channel of this (chunk, head) decays beyond SAFE_RANGE within the chunk
     // chunk table (only with cu_seqlens)
     size_t CHUNK_OFF;  // int32 [N+1]
     size_t CHUNK_SEQ;  // int32 [nch]
@@ -97,6 +98,7 @@ struct Ws {
     T *W, *UT, *KGT, *BGT, *VTT, *QG, *AQK, *AQB, *AQBT, *QGT, *HC, *DHC, *DVN;
     float *EGL;
     T* TM;
+    int32_t* STRONG;
 };
 
 template <typename T>

@@ -27,6 +27,7 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
     __shared__ __attribute__((aligned(16))) float sTw[NWP][32 * LDP];   // (I - A_ab)^-1
     constexpr int NPART = BWD ? 8 : 9;                                    // score tiles that are summed over the waves
     __shared__ __attribute__((aligned(16))) float sPart[NWP > 1 ? NWP * NPART * 256 : 4];
+    __shared__ int sStrong[NWP];
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     float* const sN = sNw[w];
     float* const sT = sTw[w];
@@ -103,7 +104,10 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
         }
         gi[kt] = scan16_incl(g4);
         ge[kt] = gi[kt] - g4;
-        const f32x4 m = bcast16(gi[kt], MID);
+        // Every score is a dense product of operands decayed relative to the middle of the chunk: exp(gi_i - gi_j) =
+        // exp(gi_i - m) exp(m - gi_j) with m = gi of token MID.  That is done here for every chunk, tile by tile as the
+        // inputs arrive; it is only valid while the exponents stay within +-SAFE_RANGE, which is checked afterwards.
+        const f32x4 m = bcast16<MID>(gi[kt]);
         const f32x4 eq = exp4<T>(gi[kt] - m), ek = exp4<T>(m - gi[kt]), ea = exp4<T>(ge[kt] - m);
         const f32x4 q4 = to_f32(rq[kt]), k4 = to_f32(rk[kt]);
         const f32x4 a0 = to_f32(ra[0][kt]), a1 = to_f32(ra[1][kt]), b0 = to_f32(rb[0][kt]), b1 = to_f32(rb[1][kt]);
@@ -124,6 +128,57 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
             for (int r = 0; r < 2; ++r) aab[r][s] = mm3(ah[r], bh[s], aab[r][s]);
         }
     }
+    // Each wave decides for its own channels (the parts of the score tiles add up whichever way they were formed); the
+    // backward pass records the decision per (chunk, head) for the chunk_grad kernels.  Where a channel decays too
+    // strongly for the single centre, what was accumulated above may hold infinities: it is thrown away and the tiles
+    // are formed again by passes whose exponents cannot overflow (see DecayPass).
+    const bool strong = strong_decay(gi, ge);
+    if (BWD && l == 0) {
+        if (NWP == 1) p.ws.STRONG[chw] = strong;
+        else sStrong[w] = strong;
+    }
+    if (strong) {
+        aqk = zero4();
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            aqb[s] = zero4(); aak[s] = zero4(); aqbT[s] = zero4(); aab[0][s] = zero4(); aab[1][s] = zero4();
+        }
+#pragma unroll 1
+        for (int ps = 0; ps < DecayPass::COUNT; ++ps) {
+            const DecayPass dp(ps, c);
+#pragma unroll
+            for (int kt = 0; kt < KTW; ++kt) {
+                f32x4 eq, ek, ea;
+                dp.factors<T>(gi[kt], ge[kt], eq, ek, ea);
+                // the same products as above, one operand at a time with the scheduler kept from interleaving them: this
+                // path is rare and must not cost the common one registers
+                // (pin(): the conversions of the inputs do not depend on the pass, and hoisted out of the pass loop they
+                // would all be live across it)
+                pin(rk[kt]); pin(rq[kt]); pin(ra[0][kt]); pin(ra[1][kt]); pin(rb[0][kt]); pin(rb[1][kt]);
+                Split<T> qh, kh, bh[2];
+                split(to_f32(rk[kt]) * ek, kh);
+                split(to_f32(rq[kt]) * eq * scale, qh);
+                aqk = mm3(qh, kh, aqk);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    split(to_f32(rb[s][kt]) * ek, bh[s]);
+                    aqb[s] = mm3(qh, bh[s], aqb[s]);
+                    if (BWD) aqbT[s] = mm3(bh[s], qh, aqbT[s]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int r = 0; r < 2; ++r) {
+                    Split<T> ah;
+                    split(to_f32(ra[r][kt]) * ea, ah);
+                    aak[r] = mm3(ah, kh, aak[r]);
+                    aab[r][0] = mm3(ah, bh[0], aab[r][0]);
+                    aab[r][1] = mm3(ah, bh[1], aab[r][1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+    }
     if (NWP > 1) {
         // sums over all channels: every wave leaves its parts in LDS and adds the others'
         f32x4* const tiles[9] = {&aak[0], &aak[1], &aab[0][0], &aab[0][1], &aab[1][0], &aab[1][1],
@@ -136,6 +191,12 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
 #pragma unroll
             for (int i = 0; i < NPART; ++i)
                 *tiles[i] += *reinterpret_cast<const f32x4*>(&sPart[((((w + ww) % NWP) * NPART + i) * 64 + l) * 4]);
+        if (BWD && w == 0 && l == 0) {
+            int any = 0;
+#pragma unroll
+            for (int ww = 0; ww < NWP; ++ww) any |= sStrong[ww];
+            p.ws.STRONG[chw] = any;
+        }
     }
     // causal masks: lane (g,c) reg i is entry (row c, inner 4g+i)
 #pragma unroll
@@ -213,7 +274,7 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const int kt = 2 * kpl + e;
-            const f32x4 gl = bcast16(gi[kt], CH - 1);
+            const f32x4 gl = bcast16<CH - 1>(gi[kt]);
             const f32x4 egi = exp4<T>(gi[kt]), ege = exp4<T>(ge[kt]), edn = exp4<T>(gl - gi[kt]);
             const Frag<T> agT[2] = {transpose(to_frag<T>(to_f32(ra[0][kt]) * ege), ident),
                                     transpose(to_frag<T>(to_f32(ra[1][kt]) * ege), ident)};
@@ -266,19 +327,20 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
 }
 
 // ---- chunk table for packed variable-length batches ----------------------------------------------------------
-__global__ void build_chunk_table_kernel(const int64_t* cu, int N, int nch, int32_t* chunk_off, int32_t* chunk_seq) {
+__global__ void build_chunk_table_kernel(const int64_t* cu, int N, int T, int nch, int32_t* chunk_off, int32_t* chunk_seq) {
     // one workgroup; N is small (number of packed sequences)
     __shared__ int total;
     if (threadIdx.x == 0) {
-        int acc = 0;
+        int64_t acc = 0;
         for (int n = 0; n < N; ++n) {
-            chunk_off[n] = acc;
-            const int64_t len = cu[n + 1] - cu[n];
-            acc += (int)((len + CH - 1) / CH);
+            // never beyond the slots the workspace has (cannot happen for a non-decreasing table that ends at T)
+            chunk_off[n] = (int)min(acc, (int64_t)nch);
+            int64_t bos, eos;
+            packed_bounds(cu, n, T, bos, eos);
+            acc += (eos - bos + CH - 1) / CH;
         }
-        if (acc > nch) acc = nch;   // cannot happen for a monotone cu_seqlens ending at T; guards the table writes
-        chunk_off[N] = acc;
-        total = acc;
+        total = (int)min(acc, (int64_t)nch);
+        chunk_off[N] = total;
     }
     __syncthreads();
     for (int cid = threadIdx.x; cid < total; cid += blockDim.x) {
@@ -321,8 +383,8 @@ hipError_t launch_prep(const ChunkArgs<T>& a, int K, int V, bool bwd, hipStream_
 template hipError_t launch_prep<bf16>(const ChunkArgs<bf16>&, int, int, bool, hipStream_t);
 template hipError_t launch_prep<float>(const ChunkArgs<float>&, int, int, bool, hipStream_t);
 
-hipError_t launch_chunk_table(const int64_t* cu, int N, int nch, int32_t* chunk_off, int32_t* chunk_seq, hipStream_t stream) {
-    hipLaunchKernelGGL(build_chunk_table_kernel, dim3(1), dim3(256), 0, stream, cu, N, nch, chunk_off, chunk_seq);
+hipError_t launch_chunk_table(const int64_t* cu, int N, int T, int nch, int32_t* chunk_off, int32_t* chunk_seq, hipStream_t stream) {
+    hipLaunchKernelGGL(build_chunk_table_kernel, dim3(1), dim3(256), 0, stream, cu, N, T, nch, chunk_off, chunk_seq);
     return hipGetLastError();
 }
 

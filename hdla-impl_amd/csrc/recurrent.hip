@@ -42,7 +42,7 @@ __global__ __launch_bounds__(256) void recurrent_kernel(RecurrentArgs<T> p) {
     const int H = p.H;
     const int tid = threadIdx.x, cg = tid % CG, rg = tid / CG, wave = tid >> 6, lane = tid & 63;
     int64_t bos, eos;
-    if (p.cu) { bos = p.cu[n]; eos = p.cu[n + 1]; }
+    if (p.cu) packed_bounds(p.cu, n, p.T_, bos, eos);
     else { bos = (int64_t)n * p.T_; eos = bos + p.T_; }
     const int len = (int)(eos - bos);
 

@@ -25,7 +25,7 @@ class HdlaDims(ctypes.Structure):
 
 class HdlaWsLayout(ctypes.Structure):
     _names = ["nch", "W", "UT", "KGT", "BGT", "VTT", "EGL", "QG", "AQK", "AQB", "AQBT", "QGT", "TM",
-              "HC", "DHC", "DVN", "SA_STRIDE", "SB_STRIDE", "CHUNK_OFF", "CHUNK_SEQ", "total"]
+              "HC", "DHC", "DVN", "STRONG", "SA_STRIDE", "SB_STRIDE", "CHUNK_OFF", "CHUNK_SEQ", "total"]
     _fields_ = [(n, ctypes.c_int64) for n in _names]
 
 
@@ -135,6 +135,21 @@ def dtype_code(dt: torch.dtype) -> int:
 def make_dims(B, T, H, K, V, R, N, in_dtype, gk_dtype, scale, cu_seqlens: Optional[torch.Tensor]) -> HdlaDims:
     return HdlaDims(B, T, H, K, V, R, N, dtype_code(in_dtype), dtype_code(gk_dtype), float(scale),
                     None if cu_seqlens is None else cu_seqlens.data_ptr())
+
+
+def check_cu_seqlens(cu_seqlens: torch.Tensor, T: int) -> None:
+    """Validate a packed-sequence table that is still on the CPU (free: no device synchronisation): it must start at
+    0, end at T and never decrease.  A table that already lives on the GPU is not read back; the kernels force its
+    entries into [0, T], so a bad one cannot cause an access outside the tensors, but rows that belong to no sequence
+    are then left unwritten in the outputs."""
+    if cu_seqlens.dim() != 1 or cu_seqlens.numel() < 2:
+        raise ValueError(f"cu_seqlens must be a 1-d tensor of N+1 >= 2 entries, got shape {tuple(cu_seqlens.shape)}")
+    if cu_seqlens.is_cuda:
+        return
+    cu = cu_seqlens.to(torch.int64)
+    if int(cu[0]) != 0 or int(cu[-1]) != T or bool((cu[1:] < cu[:-1]).any()):
+        raise ValueError(f"cu_seqlens must start at 0, end at the number of tokens ({T}) and never decrease, "
+                         f"got {cu.tolist()}")
 
 
 def current_stream(device) -> ctypes.c_void_p:

@@ -139,6 +139,7 @@ def chunk_hdla_delta_rule(
         if initial_state is not None and initial_state.shape[0] != len(cu_seqlens) - 1:
             raise ValueError(f"The number of initial states is expected to be equal to the number of input sequences, "
                              f"i.e., {len(cu_seqlens) - 1} rather than {initial_state.shape[0]}.")
+        _lib.check_cu_seqlens(cu_seqlens, q.shape[1])
         cu_seqlens = cu_seqlens.to(device=q.device, dtype=torch.int64).contiguous()
     elif initial_state is not None and initial_state.shape[0] != B:
         raise ValueError(f"initial_state must hold one state per sequence ({B}), got {initial_state.shape[0]}")
@@ -199,6 +200,7 @@ def fused_recurrent_hdla_delta_rule(
         if initial_state is not None and initial_state.shape[0] != len(cu_seqlens) - 1:
             raise ValueError(f"The number of initial states is expected to be equal to the number of input sequences, "
                              f"i.e., {len(cu_seqlens) - 1} rather than {initial_state.shape[0]}.")
+        _lib.check_cu_seqlens(cu_seqlens, q.shape[1])
         cu_seqlens = cu_seqlens.to(device=q.device, dtype=torch.int64).contiguous()
     elif initial_state is not None and initial_state.shape[0] != B:
         raise ValueError(f"initial_state must hold one state per sequence ({B}), got {initial_state.shape[0]}")

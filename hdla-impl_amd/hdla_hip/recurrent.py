@@ -110,6 +110,7 @@ def fused_recurrent_dplr_delta_rule(
         raise NotImplementedError(f"rank_ab = {rank_ab} is not supported (1 or 2)")
     _require_gpu(q, k, v, a, b, gk, initial_state)
     if cu_seqlens is not None:
+        _lib.check_cu_seqlens(cu_seqlens, q.shape[1])
         cu_seqlens = cu_seqlens.to(device=q.device, dtype=torch.int64).contiguous()
 
     K, V = q.shape[-1], v.shape[-1]

@@ -79,6 +79,7 @@ typedef struct hdla_dims {
 typedef struct hdla_ws_layout {
     int64_t nch;               /* chunk slots per head */
     int64_t W, UT, KGT, BGT, VTT, EGL, QG, AQK, AQB, AQBT, QGT, TM, HC, DHC, DVN;
+    int64_t STRONG;            /* int32 per (head, chunk) slot: nonzero where the chunk takes the strong-decay route */
     int64_t SA_STRIDE, SB_STRIDE;
     int64_t CHUNK_OFF, CHUNK_SEQ;
     int64_t total;

@@ -14,13 +14,18 @@ TOL = {torch.bfloat16: (5e-3, 1e-2), torch.float32: (1e-5, 1e-5)}
 GRADS = ["dq", "dk", "dv", "da", "db", "dgk", "dh0"]
 
 
-def _oracle(inp, dtype, scale, heads=None, use_h0=True, use_dht=True, cu=None, R=2):
-    """float64 recurrence + autograd on the dtype-rounded inputs (optionally on a subset of heads)."""
+def _oracle(inp, dtype, scale, heads=None, use_h0=True, use_dht=True, cu=None, R=2, chunk=None):
+    """float64 recurrence + autograd on the dtype-rounded inputs (optionally on a subset of heads); with `chunk` the
+    float64 chunk form of that size instead (the same function, tests/test_oracle.py; much faster on long sequences)."""
     sl = (lambda x: x) if heads is None else (lambda x: x[:, :, heads])
     slh = (lambda x: x) if heads is None else (lambda x: x[:, heads])
     leaves = [sl(t.to(dtype)).double().requires_grad_() for t in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
     h0 = slh(inp.h0).double().requires_grad_() if use_h0 else None
-    o, ht = O.recurrence(*leaves, scale, h0, cu_seqlens=cu, rank_ab=R)
+    if chunk is None:
+        o, ht = O.recurrence(*leaves, scale, h0, cu_seqlens=cu, rank_ab=R)
+    else:
+        assert cu is None
+        o, ht = O.chunk_naive(*leaves, scale, h0, rank_ab=R, chunk_size=chunk, dtype=torch.float64)
     do = sl(inp.do.to(dtype)).double()
     outs, gos = [o], [do]
     if use_dht:
@@ -33,7 +38,7 @@ def _gpu(inp, dtype, scale, use_h0=True, use_dht=True, cu=None, R=2, chunk_size=
     leaves = [t.to(dtype).to(DEV).requires_grad_() for t in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
     h0 = inp.h0.to(DEV).requires_grad_() if use_h0 else None
     o, ht = chunk_hrdplr_delta_rule(*leaves, R, scale=scale, initial_state=h0, output_final_state=True,
-                                    chunk_size=chunk_size, cu_seqlens=None if cu is None else cu.to(DEV))
+                                    chunk_size=chunk_size, cu_seqlens=cu)
     assert o.dtype == dtype and ht.dtype == torch.float32
     outs, gos = [o], [inp.do.to(dtype).to(DEV)]
     if use_dht:
@@ -116,6 +121,39 @@ def test_log_decay_gradient_under_strong_decay(B, T, H, K, V):
     assert O.rel_l2(got[2]["dgk"], ref[2]["dgk"]) <= 6e-3
 
 
+def _strong_decay_gk(gk, seed):
+    """Log-decays the reference's input domain holds (hdla_custom.py:219: log_f = logsigmoid(f), unbounded below) but a
+    factorisation of the scores around one token of the chunk cannot: on some channels every token decays by e^-12 ..
+    e^-20 (8 tokens sum to -96 .. -160, beyond the fp32 exponent range), on others only some tokens do, and some sit right
+    at the boundary between the two routes of the kernels (8 tokens summing to about -70)."""
+    g = torch.Generator().manual_seed(seed)
+    gk = gk.clone()
+    B, T, H, K = gk.shape
+    gk[..., 3] = -20.0 * (0.6 + 0.4 * torch.rand(B, T, H, generator=g))
+    gk[..., 17] = -12.0
+    hit = torch.rand(B, T, H, generator=g) < 0.3
+    gk[..., 5] = torch.where(hit, torch.full((B, T, H), -20.0), gk[..., 5])
+    gk[..., K - 1] = torch.where(hit, gk[..., K - 1], torch.full((B, T, H), -35.0))
+    gk[..., 9] = -8.75 + 0.3 * torch.randn(B, T, H, generator=g)
+    gk[:, :, 0, 40] = -6.0                                    # one head only: the other heads of this channel stay mild
+    return gk
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("B,T,H,K,V", [(1, 83, 2, 64, 64), (2, 48, 2, 128, 128), (1, 40, 3, 64, 128)])
+def test_strong_decay_stays_finite_and_within_tolerance(dtype, B, T, H, K, V):
+    inp = make_inputs(1200 + T, B, T, H, K, V, gk_div=1.0)
+    inp.gk = _strong_decay_gk(inp.gk, T)
+    got = _gpu(inp, dtype, 0.8)
+    for x in [got[0], got[1]] + list(got[2].values()):
+        assert torch.isfinite(x.float()).all()
+    _compare(got, _oracle(inp, dtype, 0.8), dtype, what=f"strong decay {dtype} T{T} K{K} V{V}")
+    cu = torch.tensor([0, 5, T - 20, T])
+    inp2 = make_inputs(1300 + T, 1, T, H, K, V, gk_div=1.0, n_states=3)
+    inp2.gk = _strong_decay_gk(inp2.gk, T + 1)
+    _compare(_gpu(inp2, dtype, 1.0, cu=cu), _oracle(inp2, dtype, 1.0, cu=cu), dtype, what=f"strong decay, packed {dtype}")
+
+
 def test_reference_integrated_test_shape_fp32():
     """Shape and distributions of the reference's end-to-end test (test_integrated.py:9-42): B2 H4 T256 K128 V64
     fp32, scale 1, gk = logsigmoid(randn), random initial state, random do / dht."""
@@ -163,10 +201,52 @@ def test_varlen_config3_reduced(dtype):
     _compare(_gpu(inp, dtype, 1.0, cu=cu), _oracle(inp, dtype, 1.0, cu=cu), dtype, what=f"varlen {dtype}")
 
 
+def test_varlen_config3_full_size_sequence_and_head_subset():
+    """Configuration 3 at full size (B1 T16384 H16 K=V=128 bf16, four packed sequences of 2048, 4096, 4096 and 6144
+    tokens, initial states, gradient into the final states), forward + backward on the GPU; the CPU oracle runs one
+    head of the longest sequence and one head of the shortest one (sequences and heads are independent)."""
+    inp = make_config(3)
+    cu = inp.cu_seqlens
+    dtype = torch.bfloat16
+    o, ht, g = _gpu(inp, dtype, 1.0, cu=cu)
+    for x in [o, ht] + list(g.values()):
+        assert torch.isfinite(x.float()).all()
+    for n, h in ((3, 5), (0, 14)):
+        s, e = int(cu[n]), int(cu[n + 1])
+        sub = type(inp)(inp.q[:, s:e, h:h + 1], inp.k[:, s:e, h:h + 1], inp.v[:, s:e, h:h + 1], inp.a[:, 2 * s:2 * e, h:h + 1],
+                        inp.b[:, 2 * s:2 * e, h:h + 1], inp.gk[:, s:e, h:h + 1], inp.h0[n:n + 1, h:h + 1],
+                        inp.do[:, s:e, h:h + 1], inp.dht[n:n + 1, h:h + 1])
+        ref = _oracle(sub, dtype, 1.0, chunk=32)
+        got_g = {m: (x[n:n + 1, h:h + 1] if m == "dh0" else x[:, 2 * s:2 * e, h:h + 1] if m in ("da", "db") else x[:, s:e, h:h + 1])
+                 for m, x in g.items()}
+        _compare((o[:, s:e, h:h + 1], ht[n:n + 1, h:h + 1], got_g), ref, dtype, what=f"cfg3 full size, sequence {n} ({e - s} tokens) head {h}")
+
+
 def test_varlen_ragged_and_empty_sequences():
     inp = make_inputs(9, 1, 100, 2, 64, 64, n_states=5)
     cu = torch.tensor([0, 3, 3, 36, 83, 100])
     _compare(_gpu(inp, torch.float32, 1.0, cu=cu), _oracle(inp, torch.float32, 1.0, cu=cu), torch.float32)
+
+
+def test_device_side_sequence_table_is_forced_into_the_token_range():
+    """A table that is already on the GPU is not validated on the host; the kernels force its entries into [0, T], so
+    one that runs past the end gives what the table cut at T gives (and rows outside every sequence stay unwritten)."""
+    inp = make_inputs(18, 1, 100, 2, 64, 64, n_states=2)
+    dtype = torch.bfloat16
+    good = torch.tensor([0, 40, 100])
+    ref = _gpu(inp, dtype, 1.0, cu=good)
+    got = _gpu(inp, dtype, 1.0, cu=torch.tensor([0, 40, 250]).to(DEV))
+    assert torch.equal(got[0], ref[0]) and torch.equal(got[1], ref[1])
+    for n in GRADS:
+        assert torch.equal(got[2][n], ref[2][n]), n
+    t = [x.to(dtype).to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    o1, h1 = fused_recurrent_dplr_delta_rule(*t, 2, scale=1.0, initial_state=inp.h0.to(DEV), output_final_state=True,
+                                             cu_seqlens=good.to(DEV))
+    o2, h2 = fused_recurrent_dplr_delta_rule(*t, 2, scale=1.0, initial_state=inp.h0.to(DEV), output_final_state=True,
+                                             cu_seqlens=torch.tensor([-5, 40, 250]).to(DEV))
+    assert torch.equal(o1, o2) and torch.equal(h1, h2)
+    with pytest.raises(ValueError):
+        _gpu(inp, dtype, 1.0, cu=torch.tensor([0, 40, 250]))          # the same table on the CPU is refused
 
 
 def test_varlen_equals_per_sequence_calls_bitwise():

@@ -71,6 +71,24 @@ def _check(got, ref, tol_o, tol_g, what):
         assert errs[n] <= tol_g, (n, errs)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("K,V", [(64, 64), (128, 128)])
+def test_strong_decay_stays_finite_and_within_tolerance(dtype, K, V):
+    """log_f = logsigmoid(f) has no lower bound (hdla_custom.py:219): channels on which every token, or every third
+    token, decays by e^-12 .. e^-20, forward and backward."""
+    q, k, v, beta, log_f, h0, do, dht = _inputs(77, 1, 70, 2, K, V, gk_div=1.0)
+    g = torch.Generator().manual_seed(5)
+    log_f[..., 2] = -20.0 * (0.6 + 0.4 * torch.rand(log_f.shape[:3], generator=g))
+    log_f[..., 11] = -12.0
+    log_f[:, ::3, :, 30] = -16.0
+    log_f[..., K - 2] = -4.0
+    inp = (q, k, v, beta, log_f, h0, do, dht)
+    got = _fused(inp, dtype, 1.0)
+    for x in [got[0], got[1]] + list(got[2].values()):
+        assert torch.isfinite(x.float()).all()
+    _check(got, _oracle(inp, dtype, 1.0), *TOL[dtype], f"strong decay {dtype} K{K} V{V}")
+
+
 CASES = [
     (torch.float32, 2, 40, 2, 64, 64, 4.0, 1.0),
     (torch.float32, 1, 50, 2, 128, 128, 1.0, 0.5),

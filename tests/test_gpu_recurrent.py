@@ -71,6 +71,29 @@ def test_decode_steps_config4_reduced():
     assert O.rel_l2(o, o_r) <= 5e-3 and O.rel_l2(S, S_r) <= 1e-5
 
 
+def test_decode_steps_config4_full_size_batch_subset():
+    """Configuration 4 at full size (B256 H32 K=V=128 bf16 inputs, fp32 state of 512 MiB): 64 single-token calls
+    carrying the state; the CPU oracle runs the same 64 tokens for three of the 256 sequences."""
+    steps = 64
+    inp = make_config(4, shape=(256, steps, 32, 128, 128))
+    t = [x.bfloat16().to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    q, k, v, a, b, gk = t
+    S = inp.h0.to(DEV)
+    outs = []
+    for i in range(steps):
+        o, S = fused_recurrent_dplr_delta_rule(q[:, i:i + 1], k[:, i:i + 1], v[:, i:i + 1], a[:, 2 * i:2 * i + 2],
+                                               b[:, 2 * i:2 * i + 2], gk[:, i:i + 1], 2, scale=1.0, initial_state=S,
+                                               output_final_state=True)
+        outs.append(o)
+    o = torch.cat(outs, 1)
+    assert torch.isfinite(o.float()).all() and torch.isfinite(S).all()
+    sel = [0, 101, 255]
+    o_r, S_r = O.recurrence(*[x[sel].bfloat16() for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)], 1.0, inp.h0[sel])
+    e_o, e_s = O.rel_l2(o[sel], o_r), O.rel_l2(S[sel], S_r)
+    print(f"cfg4 full size, 64 carried steps: o {e_o:.2e} state {e_s:.2e}", flush=True)
+    assert e_o <= 5e-3 and e_s <= 1e-5
+
+
 def test_rank_one_and_padded_dims():
     inp = make_inputs(33, 2, 12, 2, 96, 48, R=1)
     t = [x.float().to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]

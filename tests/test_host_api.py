@@ -282,3 +282,16 @@ def test_package_exports_resolve():
     for name in hdla_hip.__all__:
         assert hasattr(hdla_hip, name), name
     assert isinstance(hdla_hip.layer_pre, types.ModuleType) and callable(hdla_hip.layer_pre.layer_pre)
+
+
+def test_cu_seqlens_on_the_cpu_is_validated_before_any_launch():
+    import torch
+    from hdla_hip import _lib
+    _lib.check_cu_seqlens(torch.tensor([0, 3, 3, 10]), 10)
+    for bad in ([1, 5, 10], [0, 5, 9], [0, 7, 5, 10], [0, 5, 12], [-2, 10]):
+        with pytest.raises(ValueError):
+            _lib.check_cu_seqlens(torch.tensor(bad), 10)
+    with pytest.raises(ValueError):
+        _lib.check_cu_seqlens(torch.tensor([[0, 10]]), 10)
+    with pytest.raises(ValueError):
+        _lib.check_cu_seqlens(torch.tensor([0]), 0)
