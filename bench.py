@@ -69,6 +69,50 @@ def interface_bytes(kernel, pass_, K, V, es, gs):
     raise ValueError(kernel)
 
 
+def algorithmic_bytes(kernel, pass_, K, V, es, gs):
+    """Compulsory HBM bytes per (16-token chunk, head) that the roofline fraction is priced on: what the ALGORITHM has
+    to move, whatever this implementation's split into kernels writes in between.
+      prep, chunk_grad (the kernels that touch the operator's inputs and outputs): the compulsory bytes of their pass --
+        forward: q, k, gk, a, b (2 ranks each), v read, o written = (7K + 2V) elements per token and head (9 D at K = V = D);
+        backward: the same inputs and do read, dq, dk, dgk, da, db, dv written = (14K + 3V) elements (17 D);
+      state scans: per chunk kg (C K), v (C V), w and bg (2 ranks: 4 C K), u (2 C V) read, v_new (2 C V) and the state
+        checkpoint (K V) written = C (5K + 5V) elements + K V; the reverse scan likewise (qg, do, w, bg, dv in; dv2, dh out);
+        the forward pass's scan writes the output rows instead of a checkpoint and reads qg: C (6K + 4V) elements."""
+    C = 16
+    if kernel in ("prep", "chunk_grad"):
+        if pass_ == 0:
+            return C * ((6 * K + 2 * V) * es + K * gs)
+        return C * ((12 * K + 3 * V) * es + 2 * K * gs)
+    if kernel == "scan_fwd":
+        return C * (6 * K + 4 * V) * es if pass_ == 0 else C * (5 * K + 5 * V) * es + K * V * es
+    if kernel == "scan_bwd":
+        return C * (5 * K + 5 * V) * es + K * V * es
+    if kernel == "scan_pair":
+        return 2 * (C * (5 * K + 5 * V) * es + K * V * es)
+    raise ValueError(kernel)
+
+
+def kernel_sources_digest():
+    """Digest of the HIP sources: the counter summaries under profiles/ record the one they were taken with."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    for f in sorted(glob.glob(os.path.join(ROOT, "hdla-impl_amd", "csrc", "*.*"))):
+        if f.endswith((".hip", ".cuh", ".h", ".inc")):
+            h.update(open(f, "rb").read())
+    return h.hexdigest()[:16]
+
+
+def traffic_is_current():
+    """True when profiles/hbm_traffic.json was collected from the kernels as they are now, False when the sources
+    changed since, None when the file does not say."""
+    try:
+        rec = json.load(open(os.path.join(ROOT, "profiles", "hbm_traffic.json"))).get("kernel_sources_digest")
+    except (OSError, ValueError):
+        return None
+    return None if rec is None else rec == kernel_sources_digest()
+
+
 def measured_traffic(workload, kernel_key, K, V):
     """HBM bytes per launch of one kernel from the committed rocprofv3 counter summary (profiles/hbm_traffic.json:
     FETCH_SIZE and WRITE_SIZE per dispatch, each scaled by what the same counter reads for the streaming kernel of known traffic), or
@@ -463,46 +507,14 @@ def main():
         return
     cfg = {"train": 2, "fwd": 1, "varlen": 3, "decode": 4, "hdla": 2, "hdla_decode": 4}[wl]
     B, T, H, K, V = CONFIG_SHAPES[cfg]
-    inp = make_config(cfg)
+    inp = make_config(cfg) if wl in ("hdla", "hdla_decode") else None
     dt = torch.bfloat16
     res = {"metric": METRIC if wl == "train" else f"{wl} tokens/s", "unit": "tokens/s", "n_gpus": 1,
            "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
            "vs_baseline": None, "dtype": "bf16", "data": "synthetic"}
 
     if wl == "decode":
-        from hdla_hip.recurrent import fused_recurrent_dplr_delta_rule_fwd
-        from hdla_hip.synthetic import make_inputs
-        ncycle = 8                                             # distinct per-step inputs, cycled
-        gen = [inp] + [make_inputs(2000 + i, B, 1, H, K, V, h0_std=0.1) for i in range(1, ncycle)]
-        steps_in = [[x.to(dt).to(dev) for x in (g.q, g.k, g.v, g.a, g.b, g.gk)] for g in gen]
-        state = {"S": inp.h0.to(dev), "i": 0}
-
-        def step():
-            t = steps_in[state["i"] % ncycle]
-            state["i"] += 1
-            _, state["S"] = fused_recurrent_dplr_delta_rule(*t, 2, scale=1.0, initial_state=state["S"],
-                                                            output_final_state=True)
-        sec = time_steps(step, args.steps, args.warmup)
-        # kernel-only duration with events on the launch stream
-        evs = []
-        for _ in range(args.steps):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            t = steps_in[state["i"] % ncycle]
-            state["i"] += 1
-            q, k, v, a, b, gk = t
-            e0.record()
-            _, state["S"] = fused_recurrent_dplr_delta_rule_fwd(q, k, v, a, b, gk, 2, 1.0, state["S"], True)
-            e1.record()
-            evs.append((e0, e1))
-        torch.cuda.synchronize()
-        kms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
-        nbytes = 2 * B * H * K * V * 4 + B * H * (4 * K + 4 * K + V + V) * 2
-        res.update(value=B / sec, ms_per_step=sec * 1e3,
-                   config={"workload": "config 4: fused recurrent decode, B=256 H=32 K=V=128, one token per call, "
-                                       "persistent fp32 state", "batch": B, "heads": H, "K": K, "V": V},
-                   roofline={"bound": "hbm", "kernel": "recurrent_kernel", "achieved": nbytes / (kms * 1e-3) / 1e9,
-                             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                             "traffic": measured_traffic("decode", "recurrent", K, V), "bytes_per_launch": nbytes, "ms_per_launch": kms})
+        res.update(run_decode_workload(args.steps, args.warmup, dev))
         if not args.no_cpu_baseline:
             res["cpu_baseline"] = cpu_baseline_decode()
         print(json.dumps(res))
@@ -580,6 +592,38 @@ def main():
                    roofline=None)
         print(json.dumps(res))
         return
+    res.update(run_chunk_workload(wl, cfg, args.steps, args.warmup, dev))
+    if wl == "train":
+        # the other configurations, measured in this process after the headline (fewer steps: they are reported, the
+        # headline is what the step count is about)
+        n_other = max(5, args.steps // 3)
+        others = {}
+        for name, owl, ocfg in (("config1_fwd", "fwd", 1), ("config3_varlen", "varlen", 3)):
+            r = run_chunk_workload(owl, ocfg, n_other, 3, dev)
+            others[name] = {"workload": r["config"]["workload"], "tokens/s": r["value"], "ms_per_step": r["ms_per_step"],
+                            "dominant_kernel": r["roofline"]["kernel"], "frac": r["roofline"]["frac"],
+                            "achieved_GB/s": r["roofline"]["achieved"], "traffic": r["roofline"]["traffic"],
+                            "whole_step_frac_hbm": r["whole_step"]["frac_hbm"],
+                            "kernels": [{k: x[k] for k in ("kernel", "ms", "frac_hbm", "frac_interface")} for x in r["kernels"]]}
+        r = run_decode_workload(4 * n_other, 5, dev)
+        others["config4_decode"] = {"workload": r["config"]["workload"], "tokens/s": r["value"], "ms_per_step": r["ms_per_step"],
+                                    "dominant_kernel": "recurrent_kernel", "frac": r["roofline"]["frac"],
+                                    "achieved_GB/s": r["roofline"]["achieved"], "traffic": r["roofline"]["traffic"],
+                                    "ms_per_launch": r["roofline"]["ms_per_launch"]}
+        res["other_configs"] = others
+    if not args.no_cpu_baseline and wl == "train":
+        res["cpu_baseline"] = cpu_baseline_train()
+    print(json.dumps(res))
+
+
+def run_chunk_workload(wl, cfg, steps, warmup, dev):
+    """One of the chunked configurations (train = 2, fwd = 1, varlen = 3): whole-step time through the public operator,
+    then every kernel by itself."""
+    from hdla_hip import chunk_hrdplr_delta_rule
+    from hdla_hip.synthetic import CONFIG_SHAPES, make_config
+    B, T, H, K, V = CONFIG_SHAPES[cfg]
+    inp = make_config(cfg)
+    dt = torch.bfloat16
     cu = None if inp.cu_seqlens is None else inp.cu_seqlens.to(dev)
     N = B if cu is None else cu.numel() - 1
     leaves = [x.to(dt).to(dev).requires_grad_(wl != "fwd") for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
@@ -593,12 +637,11 @@ def main():
         if wl != "fwd":
             torch.autograd.grad([o, ht], leaves + [h0], [do, dht])
 
-    sec = time_steps(step, args.steps, args.warmup)
+    sec = time_steps(step, steps, warmup)
     tokens = B * T
     # per-kernel durations
     raw = [x.detach() for x in leaves] + [None if h0 is None else h0.detach(), do, dht]
     dims_kw = dict(B=B, T=T, H=H, K=K, V=V, R=2, N=N, in_dtype=dt, gk_dtype=dt, scale=1.0, cu_seqlens=cu)
-    q = raw[0]
     o = torch.empty_like(raw[2])
     ht = torch.empty(N, H, K, V, dtype=torch.float32, device=dev)
     grads = [torch.empty_like(x) for x in (raw[0], raw[1], raw[2], raw[3], raw[4], raw[5])]
@@ -606,33 +649,81 @@ def main():
     outs = (o, ht, *grads, dh0)
     kern = {}
     for pass_ in ([0] if wl == "fwd" else [0, 1]):
-        for name, ms in stage_times(raw, dims_kw, pass_, args.steps, outs).items():
+        for name, ms in stage_times(raw, dims_kw, pass_, steps, outs).items():
             kern[f"{'fwd' if pass_ == 0 else 'bwd'}.{name}"] = ms
     nchunk_heads = H * sum(-(-int(l) // 16) for l in ([T] * B if cu is None else (cu[1:] - cu[:-1]).tolist()))
     klist = []
     for name, ms in kern.items():
         p_, kn = name.split(".")
-        by = interface_bytes(kn, 0 if p_ == "fwd" else 1, K, V, 2, 2) * nchunk_heads
-        klist.append({"kernel": name, "ms": ms, "bytes": by, "GB/s": by / (ms * 1e-3) / 1e9,
-                      "frac_hbm": by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
+        alg = algorithmic_bytes(kn, 0 if p_ == "fwd" else 1, K, V, 2, 2) * nchunk_heads
+        itf = interface_bytes(kn, 0 if p_ == "fwd" else 1, K, V, 2, 2) * nchunk_heads
+        klist.append({"kernel": name, "ms": ms, "bytes": alg, "GB/s": alg / (ms * 1e-3) / 1e9,
+                      "frac_hbm": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                      "interface_bytes": itf, "frac_interface": itf / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
     dom = max(klist, key=lambda x: x["ms"])
-    per_tok_head = (9 * K * 2) if wl == "fwd" else (26 * K * 2)            # compulsory bytes per (token, head), K = V
+    per_tok_head = ((7 * K + 2 * V) * 2) if wl == "fwd" else ((21 * K + 5 * V) * 2)   # compulsory bytes per (token, head)
     whole = per_tok_head * H * tokens
-    res.update(value=tokens / sec, ms_per_step=sec * 1e3,
-               config={"workload": {"train": "config 2: chunked fwd+bwd, B=4 T=2048 H=16 K=V=64, bf16 in, fp32 state, h0/do/dht",
-                                    "fwd": "config 1: chunked fwd, B=4 T=2048 H=16 K=V=64, bf16 in, fp32 state",
-                                    "varlen": "config 3: chunked fwd+bwd, packed 2048/4096/4096/6144, H=16 K=V=128"}[wl],
-                       "global_batch": B, "seq_len": T, "heads": H, "K": K, "V": V, "chunk": 16},
-               roofline={"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS,
-                         "unit": "GB/s", "frac": dom["frac_hbm"],
-                         "traffic": measured_traffic(wl, dom["kernel"], K, V),
-                         "bytes_per_launch": dom["bytes"], "ms_per_launch": dom["ms"]},
-               kernels=klist,
-               whole_step={"compulsory_bytes": whole, "GB/s": whole / sec / 1e9, "frac_hbm": whole / sec / 1e9 / HBM_PEAK_GBS,
-                           "sum_kernel_ms": sum(x["ms"] for x in klist)})
-    if not args.no_cpu_baseline and wl == "train":
-        res["cpu_baseline"] = cpu_baseline_train()
-    print(json.dumps(res))
+    return dict(
+        value=tokens / sec, ms_per_step=sec * 1e3,
+        config={"workload": {"train": "config 2: chunked fwd+bwd, B=4 T=2048 H=16 K=V=64, bf16 in, fp32 state, h0/do/dht",
+                             "fwd": "config 1: chunked fwd, B=4 T=2048 H=16 K=V=64, bf16 in, fp32 state",
+                             "varlen": "config 3: chunked fwd+bwd, packed 2048/4096/4096/6144, H=16 K=V=128"}[wl],
+                "global_batch": B, "seq_len": T, "heads": H, "K": K, "V": V, "chunk": 16},
+        roofline={"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["GB/s"], "peak": HBM_PEAK_GBS,
+                  "unit": "GB/s", "frac": dom["frac_hbm"],
+                  "traffic": measured_traffic(wl, dom["kernel"], K, V),
+                  "traffic_from_current_kernels": traffic_is_current(),
+                  "bytes_per_launch": dom["bytes"], "ms_per_launch": dom["ms"],
+                  "note": "achieved = compulsory bytes of the kernel's pass (every input of the operator read once, every "
+                          "output written once; for the scans their operands and one state checkpoint per chunk) over the "
+                          "kernel's time; frac_interface in `kernels` counts what this implementation's kernels hand each "
+                          "other as well; traffic = HBM bytes per launch from the committed counter summary"},
+        kernels=klist,
+        whole_step={"compulsory_bytes": whole, "GB/s": whole / sec / 1e9, "frac_hbm": whole / sec / 1e9 / HBM_PEAK_GBS,
+                    "sum_kernel_ms": sum(x["ms"] for x in klist)})
+
+
+def run_decode_workload(steps, warmup, dev):
+    """Configuration 4: one token per call for 256 sequences, the fp32 state carried from call to call."""
+    from hdla_hip import fused_recurrent_dplr_delta_rule
+    from hdla_hip.recurrent import fused_recurrent_dplr_delta_rule_fwd
+    from hdla_hip.synthetic import CONFIG_SHAPES, make_config, make_inputs
+    B, T, H, K, V = CONFIG_SHAPES[4]
+    inp = make_config(4)
+    dt = torch.bfloat16
+    ncycle = 8                                             # distinct per-step inputs, cycled
+    gen = [inp] + [make_inputs(2000 + i, B, 1, H, K, V, h0_std=0.1) for i in range(1, ncycle)]
+    steps_in = [[x.to(dt).to(dev) for x in (g.q, g.k, g.v, g.a, g.b, g.gk)] for g in gen]
+    state = {"S": inp.h0.to(dev), "i": 0}
+
+    def step():
+        t = steps_in[state["i"] % ncycle]
+        state["i"] += 1
+        _, state["S"] = fused_recurrent_dplr_delta_rule(*t, 2, scale=1.0, initial_state=state["S"],
+                                                        output_final_state=True)
+    sec = time_steps(step, steps, warmup)
+    # kernel-only duration with events on the launch stream
+    evs = []
+    for _ in range(steps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t = steps_in[state["i"] % ncycle]
+        state["i"] += 1
+        q, k, v, a, b, gk = t
+        e0.record()
+        _, state["S"] = fused_recurrent_dplr_delta_rule_fwd(q, k, v, a, b, gk, 2, 1.0, state["S"], True)
+        e1.record()
+        evs.append((e0, e1))
+    torch.cuda.synchronize()
+    kms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    nbytes = 2 * B * H * K * V * 4 + B * H * (4 * K + 4 * K + V + V) * 2
+    return dict(value=B / sec, ms_per_step=sec * 1e3,
+                config={"workload": "config 4: fused recurrent decode, B=256 H=32 K=V=128, one token per call, "
+                                    "persistent fp32 state", "batch": B, "heads": H, "K": K, "V": V},
+                roofline={"bound": "hbm", "kernel": "recurrent_kernel", "achieved": nbytes / (kms * 1e-3) / 1e9,
+                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                          "traffic": measured_traffic("decode", "recurrent", K, V),
+                          "traffic_from_current_kernels": traffic_is_current(),
+                          "bytes_per_launch": nbytes, "ms_per_launch": kms})
 
 
 if __name__ == "__main__":
