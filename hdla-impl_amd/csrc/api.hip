@@ -10,11 +10,6 @@
 
 using namespace hdla;
 
-#ifdef HDLA_PHASE_TIMING
-static long long* g_phase_clk = nullptr;
-extern "C" void hdla_debug_set_phase_buffer(long long* p) { g_phase_clk = p; }
-#endif
-
 namespace {
 
 constexpr int CHUNK = 16;
@@ -120,9 +115,6 @@ int run_chunk(const hdla_dims* d, int pass, const void* q, const void* k, const 
     a.da = static_cast<T*>(da); a.db = static_cast<T*>(db); a.dgk = dgk;
     a.beta = static_cast<const T*>(beta); a.dbeta = static_cast<T*>(dbeta);
     bind_ws(a, d, L, nch, workspace);
-#ifdef HDLA_PHASE_TIMING
-    a.phase_clk = g_phase_clk;
-#endif
     hipError_t e;
     if (d->cu_seqlens && (stages & HDLA_STAGE_PREP)) {
         char* base = static_cast<char*>(workspace);

@@ -23,14 +23,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
-// Developer profiling: with -DHDLA_PHASE_TIMING every 128th workgroup (up to 64 of them) records the shader clock at
-// marked points into ChunkArgs::phase_clk[block][16]; in normal builds the macro expands to nothing.
-#ifdef HDLA_PHASE_TIMING
-#define PHASE_CLOCK(p, blk, i) do { if ((p).phase_clk && ((blk) & 127) == 0 && ((blk) >> 7) < 64 && lane_id() == 0) (p).phase_clk[((blk) >> 7) * 16 + (i)] = clock64(); } while (0)
-#else
-#define PHASE_CLOCK(p, blk, i) do { } while (0)
-#endif
-
 constexpr int CH = 16;       // tokens per chunk
 constexpr int MID = 7;       // token whose cumulative log-decay centres the factorised scores
 constexpr int RANK = 2;      // rank of the a/b update

@@ -124,7 +124,6 @@ struct ChunkArgs {            // inputs of the chunked operator + workspace
     float* dh0;               // nullable
     T *dq, *dk, *dv, *da, *db;
     void* dgk;
-    long long* phase_clk;     // developer profiling only (builds with -DHDLA_PHASE_TIMING); otherwise unused
 };
 
 template <typename T>

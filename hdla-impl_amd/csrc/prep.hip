@@ -53,8 +53,6 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
     const int64_t voff = (tok * H + h) * V + 4 * g;
     const int64_t chw = (int64_t)h * p.st.nch + cid;                // chunk-head slot in the workspace
     const float scale = p.scale;
-    const int blk = blockIdx.x;
-    PHASE_CLOCK(p, blk, 0);
 
     // ---- phase A: cumulative decays and the score tiles (rows i, inner j) -----------------------------------
     f32x4 gi[KTW], ge[KTW];
@@ -221,7 +219,6 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
         for (int s = 0; s < 2; ++s)
             *reinterpret_cast<f32x4*>(&sN[(16 * r + c) * LDP + 16 * s + 4 * g]) = aab[r][s];
     __syncthreads();
-    PHASE_CLOCK(p, blk, 1);
 
     // ---- phase B: (I - A_ab)^-1 by forward substitution over tokens, in registers -----------------------------
     // Lane (r, col) builds column `col` of the rows (r, i), i = 0..15, one token per step; the entries of the
@@ -251,7 +248,6 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
         for (int i = 0; i < 16; ++i) sT[(16 * r + i) * LDP + col] = x[i];
         __syncthreads();
     }
-    PHASE_CLOCK(p, blk, 2);
     Frag<T> tm[2][2];   // F(Tm^{s s'}): rows i, inner j
 #pragma unroll
     for (int s = 0; s < 2; ++s)
@@ -305,7 +301,6 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
         else st_pair2(p.ws.QGT + chw * SBS + kp * PAIR, fqgT[0], fqgT[1]);
     }
 
-    PHASE_CLOCK(p, blk, 3);
     // ---- phase D: u = Tm (A_ak v), kept transposed (rows value, inner token) ---------------------------------
     const Frag<T> aakf[2] = {to_frag<T>(aak[0]), to_frag<T>(aak[1])};
 #pragma unroll
@@ -323,7 +318,6 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
         }
         st_pair2(p.ws.UT + (chw * VT + vt) * PAIR, fu[0], fu[1]);
     }
-    PHASE_CLOCK(p, blk, 4);
 }
 
 // ---- chunk table for packed variable-length batches ----------------------------------------------------------

@@ -31,8 +31,9 @@
  *   - Return value: 0 = success, < 0 = argument error detected on the host before any launch (see
  *     hdla_strerror), > 0 = a hipError_t from a kernel launch.
  *   - Supported: R = 2; K, V in {64, 128}; in_dtype bf16 or fp32; gk fp32, or bf16 when in_dtype is bf16.
- *     Scores are factorised around the middle of each 16-token chunk, which is exact as long as the summed
- *     log-decay of any 8 consecutive tokens of one channel stays above about -80.
+ *     gk (log-space decay, <= 0) may be arbitrarily strong: where a channel loses more than e^-70 within eight
+ *     tokens the chunk's scores are formed by passes whose exponents cannot overflow, as the reference's
+ *     re-centred sub-chunks are (HRDPLR/fwd_triton.py:420-463).
  */
 #ifndef HDLA_HIP_H
 #define HDLA_HIP_H

@@ -156,6 +156,18 @@ def chunk_naive(
     return o, (S if output_final_state else None)
 
 
+def hrdplr_naive(q, k, v, a, b, gk, scale, initial_state, output_final_state, RANK_AB, head_first, chunk_size):
+    """The reference's oracle under its own name and positional signature (HRDPLR/naive.py:76-90, exported at
+    HRDPLR/__init__.py:3), so that its test call pattern ``hrdplr_naive(q, k, v, a, b, gk, 1.0, initial_state, True,
+    RANK_AB, False, chunk_size=BT)`` (test_integrated.py:72-74) can be replayed.  Like the reference it never reads
+    ``scale`` (naive.py:83: the output is ``(q * exp(gi)) @ S`` without it, :240), works in the dtype of ``q``, needs
+    ``T % chunk_size == 0`` (:98-105) and returns ``(o, final_state or None)`` (:263)."""
+    assert not head_first, "only head_first=False is supported (naive.py:98-105 rearranges [B, T, H, D])"
+    del scale
+    return chunk_naive(q, k, v, a, b, gk, 1.0, initial_state, output_final_state, rank_ab=RANK_AB,
+                       chunk_size=chunk_size, dtype=q.dtype)
+
+
 def parameterize_a_b(beta: torch.Tensor, k: torch.Tensor, log_f: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """HRDPLR/hdla_custom.py:19-43: beta [B,T,H,1] (or [B,T,H]), k and log_f [B,T,H,K] -> a, b [B,2T,H,K]."""
     if beta.dim() == 3:

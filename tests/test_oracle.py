@@ -187,3 +187,20 @@ def test_parameterize_a_b_gives_the_two_sided_householder_decay():
     a3, b3 = O.parameterize_a_b(beta[..., 0], k, log_f)
     assert torch.equal(a3, a) and torch.equal(b3, b)
     assert not torch.allclose(a[:, 0], a[:, 1]) and torch.equal(b[:, 1], k[:, 0])
+
+
+def test_hrdplr_naive_shim_has_the_reference_signature_and_ignores_scale():
+    """hrdplr_naive(q, k, v, a, b, gk, scale, initial_state, output_final_state, RANK_AB, head_first, chunk_size)
+    (naive.py:76-90): equals the recurrence at scale 1 whatever `scale` is passed (naive.py:83 is never read)."""
+    import inspect
+    from hdla_hip.synthetic import make_inputs
+    assert list(inspect.signature(O.hrdplr_naive).parameters) == [
+        "q", "k", "v", "a", "b", "gk", "scale", "initial_state", "output_final_state", "RANK_AB", "head_first", "chunk_size"]
+    inp = make_inputs(41, 2, 64, 2, 32, 16, gk_div=1.0)
+    t = [x.double() for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    o_r, s_r = O.recurrence(*t, 1.0, inp.h0.double())
+    for scale in (1.0, 0.25):
+        o, s = O.hrdplr_naive(*t, scale, inp.h0.double(), True, 2, False, chunk_size=16)
+        assert o.dtype == torch.float64 and O.rel_l2(o, o_r) < 1e-12 and O.rel_l2(s, s_r) < 1e-12
+    o, s = O.hrdplr_naive(*t, 1.0, None, False, 2, False, 32)
+    assert s is None and o.shape == inp.v.shape
