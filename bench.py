@@ -604,6 +604,7 @@ def main():
                             "dominant_kernel": r["roofline"]["kernel"], "frac": r["roofline"]["frac"],
                             "achieved_GB/s": r["roofline"]["achieved"], "traffic": r["roofline"]["traffic"],
                             "whole_step_frac_hbm": r["whole_step"]["frac_hbm"],
+                            **({"keep_forward": r["keep_forward"]} if "keep_forward" in r else {}),
                             "kernels": [{k: x[k] for k in ("kernel", "ms", "frac_hbm", "frac_interface")} for x in r["kernels"]]}
         r = run_decode_workload(4 * n_other, 5, dev)
         others["config4_decode"] = {"workload": r["config"]["workload"], "tokens/s": r["value"], "ms_per_step": r["ms_per_step"],
@@ -631,13 +632,16 @@ def run_chunk_workload(wl, cfg, steps, warmup, dev):
     h0 = inp.h0.to(dev).requires_grad_(True) if use_h0 else None
     do, dht = inp.do.to(dt).to(dev), inp.dht.to(dev)
 
-    def step():
+    def step(keep=False):
         o, ht = chunk_hrdplr_delta_rule(*leaves, 2, scale=1.0, initial_state=h0, output_final_state=True,
-                                        chunk_size=16, cu_seqlens=cu)
+                                        chunk_size=16, cu_seqlens=cu, keep_forward=keep)
         if wl != "fwd":
             torch.autograd.grad([o, ht], leaves + [h0], [do, dht])
 
     sec = time_steps(step, steps, warmup)
+    # the same step with keep_forward=True (an option, off by default: the forward pass's per-chunk intermediates stay
+    # alive until the backward pass, which then does not recompute them); `value` is the default route
+    sec_keep = time_steps(lambda: step(True), steps, warmup) if wl != "fwd" else None
     tokens = B * T
     # per-kernel durations
     raw = [x.detach() for x in leaves] + [None if h0 is None else h0.detach(), do, dht]
@@ -663,7 +667,13 @@ def run_chunk_workload(wl, cfg, steps, warmup, dev):
     dom = max(klist, key=lambda x: x["ms"])
     per_tok_head = ((7 * K + 2 * V) * 2) if wl == "fwd" else ((21 * K + 5 * V) * 2)   # compulsory bytes per (token, head)
     whole = per_tok_head * H * tokens
+    keep = {} if sec_keep is None else {"keep_forward": {
+        "what": "the same step with keep_forward=True: the backward pass reads the forward pass's per-chunk intermediates "
+                "instead of recomputing them (more memory held between the passes than the reference's inputs-only contract)",
+        "ms_per_step": sec_keep * 1e3, "value": tokens / sec_keep,
+        "whole_step_frac_hbm": ((21 * K + 5 * V) * 2) * H * tokens / sec_keep / 1e9 / HBM_PEAK_GBS}}
     return dict(
+        **keep,
         value=tokens / sec, ms_per_step=sec * 1e3,
         config={"workload": {"train": "config 2: chunked fwd+bwd, B=4 T=2048 H=16 K=V=64, bf16 in, fp32 state, h0/do/dht",
                              "fwd": "config 1: chunked fwd, B=4 T=2048 H=16 K=V=64, bf16 in, fp32 state",

@@ -31,7 +31,8 @@ int check_dims(const hdla_dims* d) {
     return HDLA_OK;
 }
 
-// pass 0 = forward, 1 = backward
+// pass: HDLA_PASS_FWD, _BWD, _FWD_KEEP (a forward pass that leaves what the backward pass needs of it), _BWD_KEPT (the
+// scratch of a backward pass that runs on such a workspace: only what its own scans write)
 int make_layout(const hdla_dims* d, int pass, WsLayout& L, int& nch) {
     const int rc = check_dims(d);
     if (rc) return rc;
@@ -46,26 +47,33 @@ int make_layout(const hdla_dims* d, int pass, WsLayout& L, int& nch) {
     size_t off = 0;
     auto take = [&](size_t bytes) { const size_t o = off; off += up256(bytes); return o; };
     L = WsLayout{};
-    const BlkF bf = blk_fwd(d->K, (int)es, pass == 0);
-    const size_t sa = take(chw * (size_t)bf.SIZE);
-    L.SA_STRIDE = bf.SIZE;
-    L.W = sa + bf.W; L.BGT = sa + bf.BGT; L.KGT = sa + bf.KGT; L.EGL = sa + bf.EGL;
-    L.UT = take(chw * 2 * V * 16 * es);
-    L.VTT = take(chw * V * 16 * es);
-    if (pass == 0) {
-        L.QG = sa + bf.QG; L.AQB = sa + bf.AQB; L.AQK = sa + bf.AQK;
-    } else {
+    const bool prep_out = pass != HDLA_PASS_BWD_KEPT;             // what the prep kernel writes
+    const bool with_o = pass == HDLA_PASS_FWD || pass == HDLA_PASS_FWD_KEEP;
+    const bool bwd_parts = pass == HDLA_PASS_BWD || pass == HDLA_PASS_FWD_KEEP;
+    const bool scan_out = pass == HDLA_PASS_BWD || pass == HDLA_PASS_BWD_KEPT;
+    if (prep_out) {
+        const BlkF bf = blk_fwd(d->K, (int)es, with_o);
+        const size_t sa = take(chw * (size_t)bf.SIZE);
+        L.SA_STRIDE = bf.SIZE;
+        L.W = sa + bf.W; L.BGT = sa + bf.BGT; L.KGT = sa + bf.KGT; L.EGL = sa + bf.EGL;
+        if (with_o) { L.QG = sa + bf.QG; L.AQB = sa + bf.AQB; L.AQK = sa + bf.AQK; }
+        L.UT = take(chw * 2 * V * 16 * es);
+        L.VTT = take(chw * V * 16 * es);
+    }
+    if (bwd_parts) {
         const BlkB bb = blk_bwd(d->K, (int)es);
         const size_t sb = take(chw * (size_t)bb.SIZE);
         L.SB_STRIDE = bb.SIZE;
         L.QGT = sb + bb.QGT; L.AQBT = sb + bb.AQBT;
         L.TM = take(chw * 1024 * es);
+        L.STRONG = take(chw * 4);
+    }
+    if (scan_out) {
         L.HC = take(chw * K * V * es);
         L.DHC = take(chw * K * V * es);
         L.DVN = take(chw * 2 * 16 * V * es);
-        L.STRONG = take(chw * 4);
     }
-    if (d->cu_seqlens) {
+    if (d->cu_seqlens && prep_out) {
         L.CHUNK_OFF = take((size_t)(d->N + 1) * 4);
         L.CHUNK_SEQ = take((size_t)(nch > 0 ? nch : 1) * 4);
     }
@@ -73,69 +81,91 @@ int make_layout(const hdla_dims* d, int pass, WsLayout& L, int& nch) {
     return HDLA_OK;
 }
 
+// what the prep kernel writes (and the sequence tables) lives in `prep_ws`, laid out by LP; what the scans of the
+// backward pass write lives in `scan_ws`, laid out by LS (the same buffer and layout unless the backward pass runs on a
+// kept forward workspace)
 template <typename T>
-void bind_ws(ChunkArgs<T>& a, const hdla_dims* d, const WsLayout& L, int nch, void* workspace) {
-    char* base = static_cast<char*>(workspace);
+void bind_ws(ChunkArgs<T>& a, const hdla_dims* d, const WsLayout& LP, void* prep_ws, const WsLayout& LS, void* scan_ws, int nch) {
+    char* base = static_cast<char*>(prep_ws);
     auto at = [&](size_t o) { return reinterpret_cast<T*>(base + o); };
-    a.ws.W = at(L.W); a.ws.UT = at(L.UT); a.ws.KGT = at(L.KGT); a.ws.BGT = at(L.BGT); a.ws.VTT = at(L.VTT);
-    a.ws.QG = at(L.QG); a.ws.AQK = at(L.AQK); a.ws.AQB = at(L.AQB);
-    a.ws.AQBT = at(L.AQBT); a.ws.QGT = at(L.QGT);
-    a.ws.HC = at(L.HC); a.ws.DHC = at(L.DHC); a.ws.DVN = at(L.DVN);
-    a.ws.EGL = reinterpret_cast<float*>(base + L.EGL);
-    a.ws.TM = reinterpret_cast<T*>(base + L.TM);
-    a.ws.STRONG = reinterpret_cast<int32_t*>(base + L.STRONG);
+    a.ws.W = at(LP.W); a.ws.UT = at(LP.UT); a.ws.KGT = at(LP.KGT); a.ws.BGT = at(LP.BGT); a.ws.VTT = at(LP.VTT);
+    a.ws.QG = at(LP.QG); a.ws.AQK = at(LP.AQK); a.ws.AQB = at(LP.AQB);
+    a.ws.AQBT = at(LP.AQBT); a.ws.QGT = at(LP.QGT);
+    a.ws.EGL = reinterpret_cast<float*>(base + LP.EGL);
+    a.ws.TM = at(LP.TM);
+    a.ws.STRONG = reinterpret_cast<int32_t*>(base + LP.STRONG);
+    a.ws.sa_stride = (int)LP.SA_STRIDE;
+    char* sbase = static_cast<char*>(scan_ws);
+    a.ws.HC = reinterpret_cast<T*>(sbase + LS.HC); a.ws.DHC = reinterpret_cast<T*>(sbase + LS.DHC);
+    a.ws.DVN = reinterpret_cast<T*>(sbase + LS.DVN);
     a.st.cu = d->cu_seqlens;
-    a.st.chunk_off = d->cu_seqlens ? reinterpret_cast<const int32_t*>(base + L.CHUNK_OFF) : nullptr;
-    a.st.chunk_seq = d->cu_seqlens ? reinterpret_cast<const int32_t*>(base + L.CHUNK_SEQ) : nullptr;
+    a.st.chunk_off = d->cu_seqlens ? reinterpret_cast<const int32_t*>(base + LP.CHUNK_OFF) : nullptr;
+    a.st.chunk_seq = d->cu_seqlens ? reinterpret_cast<const int32_t*>(base + LP.CHUNK_SEQ) : nullptr;
     a.st.T = d->T;
     a.st.NT = (d->T + CHUNK - 1) / CHUNK;
     a.st.N = d->N;
     a.st.nch = nch;
 }
 
+inline bool bad_ws(const void* p, size_t have, size_t need) {
+    return !p || (reinterpret_cast<uintptr_t>(p) & 255) || have < need;
+}
+
+// pass: HDLA_PASS_FWD / _BWD on `workspace`; HDLA_PASS_FWD_KEEP on `kept`; HDLA_PASS_BWD_KEPT on `kept` (read) and
+// `workspace` (what the scans write)
 template <typename T>
 int run_chunk(const hdla_dims* d, int pass, const void* q, const void* k, const void* v, const void* a_,
               const void* b, const void* gk, const float* h0, void* o, float* ht, const void* d_o,
               const float* dht, void* dq, void* dk, void* dv, void* da, void* db, void* dgk, float* dh0,
               void* workspace, size_t workspace_bytes, hipStream_t stream, int stages = HDLA_STAGE_ALL,
-              const void* beta = nullptr, void* dbeta = nullptr) {
-    WsLayout L;
+              const void* beta = nullptr, void* dbeta = nullptr, void* kept = nullptr, size_t kept_bytes = 0) {
+    WsLayout LP, LS;
     int nch = 0;
-    int rc = make_layout(d, pass, L, nch);
+    const bool fwd = pass == HDLA_PASS_FWD || pass == HDLA_PASS_FWD_KEEP;
+    const bool on_kept = pass == HDLA_PASS_FWD_KEEP || pass == HDLA_PASS_BWD_KEPT;
+    int rc = make_layout(d, on_kept ? HDLA_PASS_FWD_KEEP : pass, LP, nch);
     if (rc) return rc;
-    if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255) || workspace_bytes < L.total) return HDLA_ERR_WORKSPACE;
+    void* prep_ws = on_kept ? kept : workspace;
+    if (bad_ws(prep_ws, on_kept ? kept_bytes : workspace_bytes, LP.total)) return HDLA_ERR_WORKSPACE;
+    LS = LP;
+    if (pass == HDLA_PASS_BWD_KEPT) {
+        rc = make_layout(d, pass, LS, nch);
+        if (rc) return rc;
+        if (bad_ws(workspace, workspace_bytes, LS.total)) return HDLA_ERR_WORKSPACE;
+    }
     ChunkArgs<T> a{};
     a.q = static_cast<const T*>(q); a.k = static_cast<const T*>(k); a.v = static_cast<const T*>(v);
     a.a = static_cast<const T*>(a_); a.b = static_cast<const T*>(b);
     a.gk = gk; a.gk_f32 = d->gk_dtype == HDLA_FP32;
     a.H = d->H; a.scale = d->scale;
-    a.h0 = h0; a.ht = pass == 0 ? ht : nullptr; a.o = static_cast<T*>(o);
+    a.h0 = h0; a.ht = fwd ? ht : nullptr; a.o = static_cast<T*>(o);
     a.dout = static_cast<const T*>(d_o); a.dht = dht; a.dh0 = dh0;
     a.dq = static_cast<T*>(dq); a.dk = static_cast<T*>(dk); a.dv = static_cast<T*>(dv);
     a.da = static_cast<T*>(da); a.db = static_cast<T*>(db); a.dgk = dgk;
     a.beta = static_cast<const T*>(beta); a.dbeta = static_cast<T*>(dbeta);
-    bind_ws(a, d, L, nch, workspace);
+    bind_ws(a, d, LP, prep_ws, LS, pass == HDLA_PASS_BWD_KEPT ? workspace : prep_ws, nch);
     hipError_t e;
+    if (pass == HDLA_PASS_BWD_KEPT) stages &= ~HDLA_STAGE_PREP;    // the forward pass has run it
     if (d->cu_seqlens && (stages & HDLA_STAGE_PREP)) {
-        char* base = static_cast<char*>(workspace);
-        e = launch_chunk_table(d->cu_seqlens, d->N, d->T, nch, reinterpret_cast<int32_t*>(base + L.CHUNK_OFF),
-                               reinterpret_cast<int32_t*>(base + L.CHUNK_SEQ), stream);
+        char* base = static_cast<char*>(prep_ws);
+        e = launch_chunk_table(d->cu_seqlens, d->N, d->T, nch, reinterpret_cast<int32_t*>(base + LP.CHUNK_OFF),
+                               reinterpret_cast<int32_t*>(base + LP.CHUNK_SEQ), stream);
         if (e != hipSuccess) return (int)e;
     }
     if (nch > 0 && (stages & HDLA_STAGE_PREP)) {
-        e = launch_prep<T>(a, d->K, d->V, pass == 1, stream);
+        e = launch_prep<T>(a, d->K, d->V, pass == HDLA_PASS_FWD ? 0 : pass == HDLA_PASS_BWD ? 1 : 2, stream);
         if (e != hipSuccess) return (int)e;
     }
     // the two scans of the backward pass are independent of each other: one launch when both are asked for
-    const bool pair = pass == 1 && (stages & HDLA_STAGE_SCAN_FWD) && (stages & HDLA_STAGE_SCAN_BWD);
+    const bool pair = !fwd && (stages & HDLA_STAGE_SCAN_FWD) && (stages & HDLA_STAGE_SCAN_BWD);
     if (pair) {
         e = launch_scan_pair<T>(a, d->K, d->V, stream);
         if (e != hipSuccess) return (int)e;
     } else if (stages & HDLA_STAGE_SCAN_FWD) {
-        e = launch_scan_fwd<T>(a, d->K, d->V, pass == 0, stream);
+        e = launch_scan_fwd<T>(a, d->K, d->V, fwd, stream);
         if (e != hipSuccess) return (int)e;
     }
-    if (pass == 1) {
+    if (!fwd) {
         if (!pair && (stages & HDLA_STAGE_SCAN_BWD)) {
             e = launch_scan_bwd<T>(a, d->K, d->V, stream);
             if (e != hipSuccess) return (int)e;
@@ -196,14 +226,14 @@ const char* hdla_strerror(int code) {
 size_t hdla_workspace_bytes(const hdla_dims* dims, int pass) {
     WsLayout L;
     int nch;
-    if (pass != 0 && pass != 1) return 0;
+    if (pass < HDLA_PASS_FWD || pass > HDLA_PASS_BWD_KEPT) return 0;
     if (make_layout(dims, pass, L, nch)) return 0;
     return L.total;
 }
 
 int hdla_workspace_layout(const hdla_dims* dims, int pass, hdla_ws_layout* out) {
     if (!out) return HDLA_ERR_NULL;
-    if (pass != 0 && pass != 1) return HDLA_ERR_SHAPE;
+    if (pass < HDLA_PASS_FWD || pass > HDLA_PASS_BWD_KEPT) return HDLA_ERR_SHAPE;
     WsLayout L;
     int nch;
     const int rc = make_layout(dims, pass, L, nch);
@@ -302,6 +332,46 @@ int hdla_param_chunk_bwd(const hdla_dims* dims, const void* q, const void* k, co
                                nullptr, nullptr, dgk, dh0, workspace, workspace_bytes, s, HDLA_STAGE_ALL, beta, dbeta);
     return run_chunk<float>(dims, 1, q, k, v, nullptr, nullptr, gk, h0, nullptr, nullptr, d_o, dht, dq, dk, dv,
                             nullptr, nullptr, dgk, dh0, workspace, workspace_bytes, s, HDLA_STAGE_ALL, beta, dbeta);
+}
+
+int hdla_chunk_fwd_keep(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
+                        const void* b, const void* beta, const void* gk, const float* h0, void* o, float* ht,
+                        void* kept, size_t kept_bytes, void* stream) {
+    const int rc = check_dims(dims);
+    if (rc) return rc;
+    if (dims->T > 0 && (!q || !k || !v || !gk || !o || (!beta && (!a || !b)))) return HDLA_ERR_NULL;
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(a) || !aligned16(b) || !aligned16(gk) ||
+        !aligned16(o) || !aligned16(h0) || !aligned16(ht)) return HDLA_ERR_ALIGN;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (beta) { a = nullptr; b = nullptr; }
+    if (dims->in_dtype == HDLA_BF16)
+        return run_chunk<bf16>(dims, HDLA_PASS_FWD_KEEP, q, k, v, a, b, gk, h0, o, ht, nullptr, nullptr, nullptr, nullptr,
+                               nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, s, HDLA_STAGE_ALL, beta, nullptr,
+                               kept, kept_bytes);
+    return run_chunk<float>(dims, HDLA_PASS_FWD_KEEP, q, k, v, a, b, gk, h0, o, ht, nullptr, nullptr, nullptr, nullptr,
+                            nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, s, HDLA_STAGE_ALL, beta, nullptr,
+                            kept, kept_bytes);
+}
+
+int hdla_chunk_bwd_kept(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
+                        const void* b, const void* beta, const void* gk, const float* h0, const void* d_o,
+                        const float* dht, void* dq, void* dk, void* dv, void* da, void* db, void* dbeta, void* dgk,
+                        float* dh0, void* kept, size_t kept_bytes, void* workspace, size_t workspace_bytes,
+                        void* stream) {
+    const int rc = check_dims(dims);
+    if (rc) return rc;
+    if (dims->T > 0 && (!q || !k || !v || !gk || !d_o || !dq || !dk || !dv || !dgk)) return HDLA_ERR_NULL;
+    if (dims->T > 0 && (beta ? !dbeta : (!a || !b || !da || !db))) return HDLA_ERR_NULL;
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(a) || !aligned16(b) || !aligned16(gk) ||
+        !aligned16(d_o) || !aligned16(dq) || !aligned16(dk) || !aligned16(dv) || !aligned16(da) || !aligned16(db) ||
+        !aligned16(dgk) || !aligned16(h0) || !aligned16(dht) || !aligned16(dh0)) return HDLA_ERR_ALIGN;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (beta) { a = nullptr; b = nullptr; da = nullptr; db = nullptr; }
+    if (dims->in_dtype == HDLA_BF16)
+        return run_chunk<bf16>(dims, HDLA_PASS_BWD_KEPT, q, k, v, a, b, gk, h0, nullptr, nullptr, d_o, dht, dq, dk, dv, da,
+                               db, dgk, dh0, workspace, workspace_bytes, s, HDLA_STAGE_ALL, beta, dbeta, kept, kept_bytes);
+    return run_chunk<float>(dims, HDLA_PASS_BWD_KEPT, q, k, v, a, b, gk, h0, nullptr, nullptr, d_o, dht, dq, dk, dv, da,
+                            db, dgk, dh0, workspace, workspace_bytes, s, HDLA_STAGE_ALL, beta, dbeta, kept, kept_bytes);
 }
 
 int hdla_chunk_stages(const hdla_dims* dims, int pass, int stages, const void* q, const void* k, const void* v,

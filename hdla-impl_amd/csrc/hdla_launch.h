@@ -9,7 +9,8 @@ namespace hdla {
 hipError_t launch_chunk_table(const int64_t* cu, int N, int T, int nch, int32_t* chunk_off, int32_t* chunk_seq, hipStream_t stream);
 
 // K, V in {64, 128}; returns hipErrorInvalidValue for any other pair.
-template <typename T> hipError_t launch_prep(const ChunkArgs<T>& a, int K, int V, bool bwd, hipStream_t stream);
+// mode: 0 = for the forward pass, 1 = for the backward pass, 2 = forward pass whose workspace the backward pass will use
+template <typename T> hipError_t launch_prep(const ChunkArgs<T>& a, int K, int V, int mode, hipStream_t stream);
 template <typename T> hipError_t launch_scan_fwd(const ChunkArgs<T>& a, int K, int V, bool write_o, hipStream_t stream);
 template <typename T> hipError_t launch_scan_bwd(const ChunkArgs<T>& a, int K, int V, hipStream_t stream);
 // both scans of the backward pass (scan_fwd without the output, scan_bwd) in one launch

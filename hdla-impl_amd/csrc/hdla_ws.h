@@ -26,20 +26,29 @@ struct SeqTab {
 // Operands of the state scans that all value-column blocks of a (chunk, head) share are kept in ONE contiguous
 // block per (chunk, head), so that a workgroup can copy a block into LDS with a few whole-kilobyte loads.
 // Byte offsets inside a block, by head size K, element size es and pass:
-//   forward-scan block:  W [2][K/16] | BGT [2][K/16] | KGT [K/16] | (QG [K/16] | AQB [2] | AQK [1]) | EGL fp32[K]
+//   forward-scan block:  W [2][K/16] | BGT [2][K/16] | KGT [K/16] | EGL fp32[K] (one 1-KiB piece) | (QG [K/16] | AQB [2])
+//                        with AQK [1] in the second half of the EGL piece (2-byte elements) or in a piece of its own
 //   reverse-scan block:  QGT [K/16] | AQBT [2]       (the reverse scan also reads W, BGT and EGL of the forward-scan
 //                        block and turns the tiles of W and BGT itself)
-// (tiles of 256 elements in fragment order, consecutive tile pairs interleaved; the part in parentheses only in
-// the forward pass, where the scan also produces the output)
+// (tiles of 256 elements in fragment order, consecutive tile pairs interleaved; the part in parentheses and AQK only
+// where the scan also produces the output.  The block without that part is a prefix of the block with it, so the
+// kernels of the backward pass can work on blocks a forward pass left behind: only the distance between blocks differs.)
 struct BlkF { int W, BGT, KGT, QG, AQB, AQK, EGL, SIZE; };
 struct BlkB { int QGT, AQBT, SIZE; };
 constexpr BlkF blk_fwd(int K, int es, bool with_o) {
     const int tb = 256 * es, KT = K / 16;
     BlkF b{};
-    b.W = 0; b.BGT = 2 * KT * tb; b.KGT = 4 * KT * tb;
-    if (with_o) { b.QG = 5 * KT * tb; b.AQB = 6 * KT * tb; b.AQK = (6 * KT + 2) * tb; b.EGL = (6 * KT + 3) * tb; }
-    else { b.QG = 0; b.AQB = 0; b.AQK = 0; b.EGL = 5 * KT * tb; }
-    b.SIZE = (b.EGL + 4 * K + 1023) & ~1023;
+    b.W = 0; b.BGT = 2 * KT * tb; b.KGT = 4 * KT * tb; b.EGL = 5 * KT * tb;
+    const int egl_end = b.EGL + 1024;                    // 4 K <= 512 bytes of decay factors, rounded to a piece
+    if (with_o) {
+        b.AQK = es == 2 ? b.EGL + 512 : egl_end;
+        b.QG = es == 2 ? egl_end : egl_end + tb;
+        b.AQB = b.QG + KT * tb;
+        b.SIZE = (b.AQB + 2 * tb + 1023) & ~1023;
+    } else {
+        b.QG = 0; b.AQB = 0; b.AQK = 0;
+        b.SIZE = egl_end;
+    }
     return b;
 }
 constexpr BlkB blk_bwd(int K, int es) {
@@ -99,6 +108,7 @@ struct Ws {
     float *EGL;
     T* TM;
     int32_t* STRONG;
+    int sa_stride;            // bytes between the forward-scan blocks of consecutive (chunk, head) slots
 };
 
 template <typename T>

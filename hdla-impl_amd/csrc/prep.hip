@@ -17,8 +17,14 @@ namespace hdla {
 
 constexpr int LDP = 36;   // padded row length of the 32x32 LDS matrices (keeps 16-byte row alignment)
 
-template <typename T, bool GKF32, int K, int V, bool BWD, bool HD>
+// MODE: what the kernel leaves in the workspace -- PREP_FWD: what the forward pass's scan reads (which also forms the
+// output); PREP_BWD: what the two scans of the backward pass and the chunk_grad kernels read; PREP_KEEP: both, for a
+// forward pass whose workspace the backward pass will use instead of running this kernel again.
+enum PrepMode { PREP_FWD = 0, PREP_BWD = 1, PREP_KEEP = 2 };
+template <typename T, bool GKF32, int K, int V, int MODE, bool HD>
 __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void prep_kernel(ChunkArgs<T> p) {
+    constexpr bool BWD = MODE == PREP_BWD;                // neither the output's score tiles nor qg are needed
+    constexpr bool WB = MODE != PREP_FWD;                 // the backward pass's extras are
     constexpr int NWP = K / 64;                       // waves per (chunk, head)
     constexpr int KTW = 4, VT = V / 16, VTW = VT / NWP, KT2 = K / 32;
     constexpr int SAS = blk_fwd(K, sizeof(T), !BWD).SIZE / (int)sizeof(T);   // elements between (chunk, head) slots
@@ -131,7 +137,7 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
     // strongly for the single centre, what was accumulated above may hold infinities: it is thrown away and the tiles
     // are formed again by passes whose exponents cannot overflow (see DecayPass).
     const bool strong = strong_decay(gi, ge);
-    if (BWD && l == 0) {
+    if (WB && l == 0) {
         if (NWP == 1) p.ws.STRONG[chw] = strong;
         else sStrong[w] = strong;
     }
@@ -189,7 +195,7 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
 #pragma unroll
             for (int i = 0; i < NPART; ++i)
                 *tiles[i] += *reinterpret_cast<const f32x4*>(&sPart[((((w + ww) % NWP) * NPART + i) * 64 + l) * 4]);
-        if (BWD && w == 0 && l == 0) {
+        if (WB && w == 0 && l == 0) {
             int any = 0;
 #pragma unroll
             for (int ww = 0; ww < NWP; ++ww) any |= sStrong[ww];
@@ -209,8 +215,12 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
         if (!BWD) {
             st_tile(p.ws.AQK + chw * SAS, to_frag<T>(aqk));
             st_pair2(p.ws.AQB + chw * SAS, to_frag<T>(aqb[0]), to_frag<T>(aqb[1]));
-        } else {
-            st_pair2(p.ws.AQBT + chw * SBS, to_frag<T>(aqbT[0]), to_frag<T>(aqbT[1]));
+        }
+        if (BWD) st_pair2(p.ws.AQBT + chw * SBS, to_frag<T>(aqbT[0]), to_frag<T>(aqbT[1]));
+        else if (WB) {
+            // both orientations wanted: the second is the first turned (a product with the identity: exact)
+            const Frag<T> id = ident_frag<T>();
+            st_pair2(p.ws.AQBT + chw * SBS, transpose(to_frag<T>(aqb[0]), id), transpose(to_frag<T>(aqb[1]), id));
         }
     }
 #pragma unroll
@@ -255,7 +265,7 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
         for (int s2 = 0; s2 < 2; ++s2)
             tm[s][s2] = to_frag<T>(*reinterpret_cast<const f32x4*>(&sT[(16 * s + c) * LDP + 16 * s2 + 4 * g]));
     const Frag<T> ident = ident_frag<T>();
-    if (BWD && w == NWP - 1) {
+    if (WB && w == NWP - 1) {
         // for the chunk_grad kernel: the four blocks transposed, as fragments (two tile pairs), ready to load
         T* tmw = p.ws.TM + chw * 1024;
 #pragma unroll
@@ -285,7 +295,7 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
             fkgT[e] = transpose(kg, ident);
             fbgT[0][e] = transpose(to_frag<T>(to_f32(rb[0][kt]) * edn), ident);
             fbgT[1][e] = transpose(to_frag<T>(to_f32(rb[1][kt]) * edn), ident);
-            if (BWD) fqgT[e] = transpose(fqg[e], ident);
+            if (WB) fqgT[e] = transpose(fqg[e], ident);
             if (c == 0) {
                 const f32x4 egl = exp4<T>(gl);
                 *reinterpret_cast<f32x4*>(p.ws.EGL + chw * (SAS * (int)sizeof(T) / 4) + 16 * (kt0 + kt) + 4 * g) = egl;
@@ -298,7 +308,7 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
         }
         st_pair2(p.ws.KGT + chw * SAS + kp * PAIR, fkgT[0], fkgT[1]);
         if (!BWD) st_pair2(p.ws.QG + chw * SAS + kp * PAIR, fqg[0], fqg[1]);
-        else st_pair2(p.ws.QGT + chw * SBS + kp * PAIR, fqgT[0], fqgT[1]);
+        if (WB) st_pair2(p.ws.QGT + chw * SBS + kp * PAIR, fqgT[0], fqgT[1]);
     }
 
     // ---- phase D: u = Tm (A_ak v), kept transposed (rows value, inner token) ---------------------------------
@@ -348,34 +358,39 @@ __global__ void build_chunk_table_kernel(const int64_t* cu, int N, int T, int nc
 }
 
 template <typename T, int K, int V, bool HD>
-static hipError_t launch_prep_kv(const ChunkArgs<T>& a, bool bwd, hipStream_t stream) {
+static hipError_t launch_prep_kv(const ChunkArgs<T>& a, int mode, hipStream_t stream) {
     dim3 grid(a.st.nch * a.H), block(K);
     constexpr bool kAlwaysF32 = sizeof(T) == 4;
-    if (kAlwaysF32 || a.gk_f32) {
-        if (bwd) hipLaunchKernelGGL((prep_kernel<T, true, K, V, true, HD>), grid, block, 0, stream, a);
-        else hipLaunchKernelGGL((prep_kernel<T, true, K, V, false, HD>), grid, block, 0, stream, a);
+    const bool gkf32 = kAlwaysF32 || a.gk_f32;
+#define HDLA_PREP_LAUNCH(GK, MODE) hipLaunchKernelGGL((prep_kernel<T, GK, K, V, MODE, HD>), grid, block, 0, stream, a)
+    if (gkf32) {
+        if (mode == PREP_FWD) HDLA_PREP_LAUNCH(true, PREP_FWD);
+        else if (mode == PREP_BWD) HDLA_PREP_LAUNCH(true, PREP_BWD);
+        else HDLA_PREP_LAUNCH(true, PREP_KEEP);
     } else {
-        if (bwd) hipLaunchKernelGGL((prep_kernel<T, kAlwaysF32, K, V, true, HD>), grid, block, 0, stream, a);
-        else hipLaunchKernelGGL((prep_kernel<T, kAlwaysF32, K, V, false, HD>), grid, block, 0, stream, a);
+        if (mode == PREP_FWD) HDLA_PREP_LAUNCH(kAlwaysF32, PREP_FWD);
+        else if (mode == PREP_BWD) HDLA_PREP_LAUNCH(kAlwaysF32, PREP_BWD);
+        else HDLA_PREP_LAUNCH(kAlwaysF32, PREP_KEEP);
     }
+#undef HDLA_PREP_LAUNCH
     return hipGetLastError();
 }
 
 template <typename T, bool HD>
-static hipError_t launch_prep_hd(const ChunkArgs<T>& a, int K, int V, bool bwd, hipStream_t stream) {
-    if (K == 64 && V == 64) return launch_prep_kv<T, 64, 64, HD>(a, bwd, stream);
-    if (K == 128 && V == 128) return launch_prep_kv<T, 128, 128, HD>(a, bwd, stream);
-    if (K == 64 && V == 128) return launch_prep_kv<T, 64, 128, HD>(a, bwd, stream);
-    if (K == 128 && V == 64) return launch_prep_kv<T, 128, 64, HD>(a, bwd, stream);
+static hipError_t launch_prep_hd(const ChunkArgs<T>& a, int K, int V, int mode, hipStream_t stream) {
+    if (K == 64 && V == 64) return launch_prep_kv<T, 64, 64, HD>(a, mode, stream);
+    if (K == 128 && V == 128) return launch_prep_kv<T, 128, 128, HD>(a, mode, stream);
+    if (K == 64 && V == 128) return launch_prep_kv<T, 64, 128, HD>(a, mode, stream);
+    if (K == 128 && V == 64) return launch_prep_kv<T, 128, 64, HD>(a, mode, stream);
     return hipErrorInvalidValue;
 }
 
 template <typename T>
-hipError_t launch_prep(const ChunkArgs<T>& a, int K, int V, bool bwd, hipStream_t stream) {
-    return a.beta ? launch_prep_hd<T, true>(a, K, V, bwd, stream) : launch_prep_hd<T, false>(a, K, V, bwd, stream);
+hipError_t launch_prep(const ChunkArgs<T>& a, int K, int V, int mode, hipStream_t stream) {
+    return a.beta ? launch_prep_hd<T, true>(a, K, V, mode, stream) : launch_prep_hd<T, false>(a, K, V, mode, stream);
 }
-template hipError_t launch_prep<bf16>(const ChunkArgs<bf16>&, int, int, bool, hipStream_t);
-template hipError_t launch_prep<float>(const ChunkArgs<float>&, int, int, bool, hipStream_t);
+template hipError_t launch_prep<bf16>(const ChunkArgs<bf16>&, int, int, int, hipStream_t);
+template hipError_t launch_prep<float>(const ChunkArgs<float>&, int, int, int, hipStream_t);
 
 hipError_t launch_chunk_table(const int64_t* cu, int N, int T, int nch, int32_t* chunk_off, int32_t* chunk_seq, hipStream_t stream) {
     hipLaunchKernelGGL(build_chunk_table_kernel, dim3(1), dim3(256), 0, stream, cu, N, T, nch, chunk_off, chunk_seq);

@@ -234,7 +234,8 @@ __device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem,
     // that may or may not have been issued would make the compiler wait for all outstanding loads)
     auto blk = [&](int t) __attribute__((always_inline)) {
         const int64_t chw = chw0 + min(c0 + t, last);
-        const char* b = reinterpret_cast<const char*>(p.ws.W) + chw * B.SIZE;
+        // (the forward pass's blocks are B.SIZE apart; those the backward pass reads may be a forward pass's, further apart)
+        const char* b = reinterpret_cast<const char*>(p.ws.W) + chw * (WRITE_O ? B.SIZE : p.ws.sa_stride);
         if constexpr (OWN_LDS)
             return BlockFwd<NIB, C::OWN_UT, C::OWN_VTT>{b, reinterpret_cast<const char*>(p.ws.UT + (chw * VT + vt0) * PAIR),
                                                         reinterpret_cast<const char*>(p.ws.VTT + (chw * VT + vt0) * TILE)};
@@ -488,7 +489,8 @@ __device__ __forceinline__ void scan_bwd_body(const ChunkArgs<T>& p, char* smem,
     constexpr int KT = K / 16, KT2 = KT / 2, VT = V / 16, NM = C::NM, ES = sizeof(T);
     // LDS slot: [BG | WT] (BGT and W of the forward-scan block, transposed on their way in) | EGL | QGT | AQBT
     constexpr SlotB B = slot_bwd(K, sizeof(T));
-    constexpr int SFWD = blk_fwd(K, sizeof(T), false).SIZE, SBWD = blk_bwd(K, sizeof(T)).SIZE, NT = B.NIF;
+    constexpr int SBWD = blk_bwd(K, sizeof(T)).SIZE, NT = B.NIF;
+    const int SFWD = p.ws.sa_stride;
     constexpr bool PIPE = C::pipelined(false);
     constexpr bool PIPE_UPD = PIPE && C::early_update_reads(false);
     constexpr int NI = B.SIZE / 1024, SLOT = B.SIZE;

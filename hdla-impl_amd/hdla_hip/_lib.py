@@ -81,6 +81,10 @@ def load():
     lib.hdla_param_chunk_fwd.argtypes = [F] + [P] * 8 + [P, ctypes.c_size_t, P]
     lib.hdla_param_chunk_bwd.restype = ctypes.c_int
     lib.hdla_param_chunk_bwd.argtypes = [F] + [P] * 14 + [P, ctypes.c_size_t, P]
+    lib.hdla_chunk_fwd_keep.restype = ctypes.c_int
+    lib.hdla_chunk_fwd_keep.argtypes = [F] + [P] * 10 + [P, ctypes.c_size_t, P]
+    lib.hdla_chunk_bwd_kept.restype = ctypes.c_int
+    lib.hdla_chunk_bwd_kept.argtypes = [F] + [P] * 18 + [P, ctypes.c_size_t, P, ctypes.c_size_t, P]
     lib.hdla_chunk_stages.restype = ctypes.c_int
     lib.hdla_chunk_stages.argtypes = [F, ctypes.c_int, ctypes.c_int] + [P] * 18 + [P, ctypes.c_size_t, P]
     lib.hdla_calib_stream.restype = ctypes.c_int
@@ -150,6 +154,16 @@ def check_cu_seqlens(cu_seqlens: torch.Tensor, T: int) -> None:
     if int(cu[0]) != 0 or int(cu[-1]) != T or bool((cu[1:] < cu[:-1]).any()):
         raise ValueError(f"cu_seqlens must start at 0, end at the number of tokens ({T}) and never decrease, "
                          f"got {cu.tolist()}")
+
+
+PASS_FWD, PASS_BWD, PASS_FWD_KEEP, PASS_BWD_KEPT = 0, 1, 2, 3
+
+
+def keep_forward_default() -> bool:
+    """Whether the chunked operators keep the forward pass's per-chunk intermediates for the backward pass when the
+    caller does not say (``keep_forward=None``): environment variable HDLA_HIP_KEEP_FORWARD=1.  Off by default: the
+    reference keeps only the inputs between the passes (HRDPLR/hrdplr.py:137) and so does this library unless asked."""
+    return os.environ.get("HDLA_HIP_KEEP_FORWARD", "0") not in ("", "0", "false", "False")
 
 
 def current_stream(device) -> ctypes.c_void_p:

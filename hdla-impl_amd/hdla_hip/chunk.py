@@ -63,22 +63,63 @@ def _dims(q, v, gk, scale, cu_seqlens, n_seq):
     return _lib.make_dims(B, T, H, K, v.shape[-1], 2, n_seq, q.dtype, gk.dtype, scale, cu_seqlens)
 
 
-def chunk_hrdplr_fwd(q, k, v, a, b, gk, scale, initial_state, output_final_state, cu_seqlens=None):
-    """Forward launch sequence (HRDPLR/hrdplr.py:25-99) on native shapes: returns (o, final_state)."""
+def chunk_hrdplr_fwd(q, k, v, a, b, gk, scale, initial_state, output_final_state, cu_seqlens=None, keep=False,
+                     beta=None):
+    """Forward launch sequence (HRDPLR/hrdplr.py:25-99) on native shapes: returns (o, final_state), and with ``keep``
+    also the workspace the backward pass can run on instead of recomputing it (``hdla_chunk_fwd_keep``).  With ``beta``
+    a and b are formed in the kernels (they may be None)."""
     lib = _lib.load()
     B, T, H, K = q.shape
     V = v.shape[-1]
     N = B if cu_seqlens is None else cu_seqlens.numel() - 1
     with torch.cuda.device(q.device):
         dims = _dims(q, v, gk, scale, cu_seqlens, N)
-        ws = _lib.workspace(dims, 0, q.device)
         o = torch.empty_like(v)
         ht = torch.empty(N, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
+        if keep:
+            ws = _lib.workspace(dims, _lib.PASS_FWD_KEEP, q.device)
+            rc = lib.hdla_chunk_fwd_keep(ctypes.byref(dims), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(a),
+                                         _lib.ptr(b), _lib.ptr(beta), _lib.ptr(gk), _lib.ptr(initial_state), _lib.ptr(o),
+                                         _lib.ptr(ht), _lib.ptr(ws), ws.numel(), _lib.current_stream(q.device))
+            _lib.check(rc, "hdla_chunk_fwd_keep")
+            return o, ht, ws
+        assert beta is None
+        ws = _lib.workspace(dims, _lib.PASS_FWD, q.device)
         rc = lib.hdla_chunk_fwd(ctypes.byref(dims), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(a), _lib.ptr(b),
                                 _lib.ptr(gk), _lib.ptr(initial_state), _lib.ptr(o), _lib.ptr(ht),
                                 _lib.ptr(ws), ws.numel(), _lib.current_stream(q.device))
         _lib.check(rc, "hdla_chunk_fwd")
     return o, ht
+
+
+def chunk_hrdplr_bwd_kept(q, k, v, a, b, gk, scale, initial_state, do, dht, kept, cu_seqlens=None, want_dh0=True,
+                          beta=None):
+    """Backward launch sequence on the workspace a forward pass kept (``hdla_chunk_bwd_kept``): the per-chunk
+    intermediates are read there, not recomputed.  Returns (dq, dk, dv, da, db, dgk, dh0), or with ``beta``
+    (dq, dk, dv, dbeta, dgk, dh0)."""
+    lib = _lib.load()
+    B, T, H, K = q.shape
+    V = v.shape[-1]
+    N = B if cu_seqlens is None else cu_seqlens.numel() - 1
+    with torch.cuda.device(q.device):
+        dims = _dims(q, v, gk, scale, cu_seqlens, N)
+        ws = _lib.workspace(dims, _lib.PASS_BWD_KEPT, q.device)
+        dq, dk, dv, dgk = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.empty_like(gk)
+        da = db = dbeta = None
+        if beta is None:
+            da, db = torch.empty_like(a), torch.empty_like(b)
+        else:
+            dbeta = torch.empty_like(beta)
+        dh0 = torch.empty(N, H, K, V, dtype=torch.float32, device=q.device) if want_dh0 else None
+        rc = lib.hdla_chunk_bwd_kept(ctypes.byref(dims), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(a), _lib.ptr(b),
+                                     _lib.ptr(beta), _lib.ptr(gk), _lib.ptr(initial_state), _lib.ptr(do), _lib.ptr(dht),
+                                     _lib.ptr(dq), _lib.ptr(dk), _lib.ptr(dv), _lib.ptr(da), _lib.ptr(db), _lib.ptr(dbeta),
+                                     _lib.ptr(dgk), _lib.ptr(dh0), _lib.ptr(kept), kept.numel(), _lib.ptr(ws), ws.numel(),
+                                     _lib.current_stream(q.device))
+        _lib.check(rc, "hdla_chunk_bwd_kept")
+    if beta is None:
+        return dq, dk, dv, da, db, dgk, dh0
+    return dq, dk, dv, dbeta, dgk, dh0
 
 
 def chunk_hrdplr_bwd(q, k, v, a, b, gk, scale, initial_state, do, dht, cu_seqlens=None, want_dh0=True,
@@ -111,9 +152,15 @@ class ChunkDPLRDeltaRuleFunction(torch.autograd.Function):
     @contiguous
     @autocast_custom_fwd
     def forward(ctx, q, k, v, a, b, gk, scale, initial_state, output_final_state, RANK_AB, head_first, chunk_size,
-                cu_seqlens=None):
+                cu_seqlens=None, keep_forward=False):
         h0 = None if initial_state is None else initial_state.to(torch.float32).contiguous()
-        o, final_state = chunk_hrdplr_fwd(q, k, v, a, b, gk, scale, h0, output_final_state, cu_seqlens)
+        # keep_forward (off unless asked for): the per-chunk intermediates of this pass stay alive on ctx until the
+        # backward pass, which then does not recompute them; only when a gradient can be asked for at all
+        ctx.kept = None
+        if keep_forward and any(ctx.needs_input_grad):
+            o, final_state, ctx.kept = chunk_hrdplr_fwd(q, k, v, a, b, gk, scale, h0, output_final_state, cu_seqlens, keep=True)
+        else:
+            o, final_state = chunk_hrdplr_fwd(q, k, v, a, b, gk, scale, h0, output_final_state, cu_seqlens)
         ctx.save_for_backward(q, k, v, a, b, gk, initial_state, cu_seqlens)     # inputs only (hrdplr.py:137)
         ctx.scale = scale
         ctx.chunk_size = chunk_size
@@ -133,12 +180,16 @@ class ChunkDPLRDeltaRuleFunction(torch.autograd.Function):
         if dht is not None:
             dht = dht.to(torch.float32).contiguous()
         h0 = None if initial_state is None else initial_state.to(torch.float32).contiguous()
-        dq, dk, dv, da, db, dgk, dh0 = chunk_hrdplr_bwd(q, k, v, a, b, gk, ctx.scale, h0, do, dht, cu_seqlens,
-                                                        want_dh0=initial_state is not None)
+        if ctx.kept is not None:
+            dq, dk, dv, da, db, dgk, dh0 = chunk_hrdplr_bwd_kept(q, k, v, a, b, gk, ctx.scale, h0, do, dht, ctx.kept,
+                                                                 cu_seqlens, want_dh0=initial_state is not None)
+        else:
+            dq, dk, dv, da, db, dgk, dh0 = chunk_hrdplr_bwd(q, k, v, a, b, gk, ctx.scale, h0, do, dht, cu_seqlens,
+                                                            want_dh0=initial_state is not None)
         if dh0 is not None:
             dh0 = dh0.to(initial_state.dtype)
-        # one slot per forward argument (hrdplr.py:284), plus one for cu_seqlens
-        return dq.to(q), dk.to(k), dv.to(v), da.to(a), db.to(b), dgk.to(gk), None, dh0, None, None, None, None, None
+        # one slot per forward argument (hrdplr.py:284), plus one each for cu_seqlens and keep_forward
+        return dq.to(q), dk.to(k), dv.to(v), da.to(a), db.to(b), dgk.to(gk), None, dh0, None, None, None, None, None, None
 
 
 @torch.compiler.disable
@@ -157,11 +208,17 @@ def chunk_hrdplr_delta_rule(
     chunk_size: int = 32,
     *,
     cu_seqlens: Optional[torch.Tensor] = None,
+    keep_forward: Optional[bool] = None,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """S_t = Diag(exp(gk_t)) S_{t-1} + sum_r b_t^r (a_t^r . S_{t-1}) + k_t v_t^T,  o_t = scale * S_t^T q_t.
 
     Signature and semantics of HRDPLR/hrdplr.py:286-318; returns ``(o [B,T,H,V] in q.dtype, final_state
     [N,H,K,V] fp32 or None)``.
+
+    ``keep_forward`` (keyword-only, not in the reference): True keeps the forward pass's per-chunk intermediates alive
+    until the backward pass (about 1.6 times the bytes of q, k, v, a, b, gk together), which then skips recomputing
+    them; False (and None without HDLA_HIP_KEEP_FORWARD=1 in the environment) is the reference's behaviour: only the
+    inputs are kept (hrdplr.py:137) and the backward pass recomputes (:161-198).  Results agree to rounding.
     """
     assert head_first is False or head_first == 0, "only head_first=False is supported (HRDPLR/fwd_func.py:28)"
     assert q.dtype == k.dtype == v.dtype                                                   # hrdplr.py:301
@@ -207,7 +264,8 @@ def chunk_hrdplr_delta_rule(
         h0 = F.pad(h0, (0, Vn - V, 0, Kn - K))
     o, final_state = ChunkDPLRDeltaRuleFunction.apply(
         _pad_last(q, Kn), _pad_last(k, Kn), _pad_last(v, Vn), _pad_last(a2, Kn), _pad_last(b2, Kn), _pad_last(gk, Kn),
-        scale, h0, output_final_state, 2, head_first, chunk_size, cu_seqlens)
+        scale, h0, output_final_state, 2, head_first, chunk_size, cu_seqlens,
+        _lib.keep_forward_default() if keep_forward is None else bool(keep_forward))
     if Vn != V:
         o = o[..., :V]
     if final_state is not None and (Kn != K or Vn != V):

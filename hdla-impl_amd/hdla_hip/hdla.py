@@ -21,7 +21,7 @@ import torch
 import torch.nn.functional as F
 
 from . import _lib
-from .chunk import _dims, _native_dim, _pad_last, _require_gpu
+from .chunk import _dims, _native_dim, _pad_last, _require_gpu, chunk_hrdplr_bwd_kept, chunk_hrdplr_fwd
 from .utils import autocast_custom_bwd, autocast_custom_fwd, contiguous
 
 
@@ -82,9 +82,14 @@ class ChunkHDLAFunction(torch.autograd.Function):
     @staticmethod
     @contiguous
     @autocast_custom_fwd
-    def forward(ctx, q, k, v, beta, gk, scale, initial_state, output_final_state, cu_seqlens=None):
+    def forward(ctx, q, k, v, beta, gk, scale, initial_state, output_final_state, cu_seqlens=None, keep_forward=False):
         h0 = None if initial_state is None else initial_state.to(torch.float32).contiguous()
-        o, final_state = _fwd(q, k, v, beta, gk, scale, h0, output_final_state, cu_seqlens)
+        ctx.kept = None
+        if keep_forward and any(ctx.needs_input_grad):     # see ChunkDPLRDeltaRuleFunction.forward
+            o, final_state, ctx.kept = chunk_hrdplr_fwd(q, k, v, None, None, gk, scale, h0, output_final_state, cu_seqlens,
+                                                        keep=True, beta=beta)
+        else:
+            o, final_state = _fwd(q, k, v, beta, gk, scale, h0, output_final_state, cu_seqlens)
         ctx.save_for_backward(q, k, v, beta, gk, initial_state, cu_seqlens)
         ctx.scale = scale
         return o.to(q.dtype), final_state
@@ -100,11 +105,15 @@ class ChunkHDLAFunction(torch.autograd.Function):
         if dht is not None:
             dht = dht.to(torch.float32).contiguous()
         h0 = None if initial_state is None else initial_state.to(torch.float32).contiguous()
-        dq, dk, dv, dbeta, dgk, dh0 = _bwd(q, k, v, beta, gk, ctx.scale, h0, do, dht, cu_seqlens,
-                                           want_dh0=initial_state is not None)
+        if ctx.kept is not None:
+            dq, dk, dv, dbeta, dgk, dh0 = chunk_hrdplr_bwd_kept(q, k, v, None, None, gk, ctx.scale, h0, do, dht, ctx.kept,
+                                                                cu_seqlens, want_dh0=initial_state is not None, beta=beta)
+        else:
+            dq, dk, dv, dbeta, dgk, dh0 = _bwd(q, k, v, beta, gk, ctx.scale, h0, do, dht, cu_seqlens,
+                                               want_dh0=initial_state is not None)
         if dh0 is not None:
             dh0 = dh0.to(initial_state.dtype)
-        return dq.to(q), dk.to(k), dv.to(v), dbeta.to(beta), dgk.to(gk), None, dh0, None, None
+        return dq.to(q), dk.to(k), dv.to(v), dbeta.to(beta), dgk.to(gk), None, dh0, None, None, None
 
 
 @torch.compiler.disable
@@ -119,10 +128,12 @@ def chunk_hdla_delta_rule(
     output_final_state: bool = False,
     *,
     cu_seqlens: Optional[torch.Tensor] = None,
+    keep_forward: Optional[bool] = None,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """``chunk_hrdplr_delta_rule(q, k, v, *parameterize_a_b(beta, k, log_f), gk=log_f, RANK_AB=2, ...)`` with a and
     b (rounded to q's dtype, as ``hdla_custom.py:301-304`` does) formed inside the kernels.  Returns ``(o, final_state)``
-    like the plain operator; gradients flow to q, k, v, beta, log_f and initial_state."""
+    like the plain operator; gradients flow to q, k, v, beta, log_f and initial_state.  ``keep_forward``: as for
+    ``chunk_hrdplr_delta_rule``."""
     assert q.dtype == k.dtype == v.dtype
     if q.dim() != 4 or v.dim() != 4:
         raise ValueError("q, k, v must be 4-dimensional [B, T, H, D]")
@@ -160,7 +171,8 @@ def chunk_hdla_delta_rule(
     if h0 is not None and (Kn != K or Vn != V):
         h0 = F.pad(h0, (0, Vn - V, 0, Kn - K))
     o, final_state = ChunkHDLAFunction.apply(_pad_last(q, Kn), _pad_last(k, Kn), _pad_last(v, Vn), beta,
-                                             _pad_last(gk, Kn), scale, h0, output_final_state, cu_seqlens)
+                                             _pad_last(gk, Kn), scale, h0, output_final_state, cu_seqlens,
+                                             _lib.keep_forward_default() if keep_forward is None else bool(keep_forward))
     if Vn != V:
         o = o[..., :V]
     if final_state is not None and (Kn != K or Vn != V):

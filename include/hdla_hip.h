@@ -89,7 +89,11 @@ typedef struct hdla_ws_layout {
 int hdla_version(void);
 const char* hdla_strerror(int code);
 
-/* pass: 0 = forward, 1 = backward.  Returns 0 for invalid dims. */
+/* Workspaces by pass.  HDLA_PASS_FWD and HDLA_PASS_BWD are the scratch of hdla_chunk_fwd / hdla_chunk_bwd (contents
+ * disposable after the call).  HDLA_PASS_FWD_KEEP is the buffer hdla_chunk_fwd_keep fills and hdla_chunk_bwd_kept
+ * reads (it must survive from the one to the other), HDLA_PASS_BWD_KEPT the scratch of hdla_chunk_bwd_kept.
+ * hdla_workspace_bytes returns 0 for invalid dims or pass. */
+enum { HDLA_PASS_FWD = 0, HDLA_PASS_BWD = 1, HDLA_PASS_FWD_KEEP = 2, HDLA_PASS_BWD_KEPT = 3 };
 size_t hdla_workspace_bytes(const hdla_dims* dims, int pass);
 int hdla_workspace_layout(const hdla_dims* dims, int pass, hdla_ws_layout* out);
 
@@ -134,6 +138,25 @@ int hdla_param_chunk_bwd(const hdla_dims* dims, const void* q, const void* k, co
                          const void* gk, const float* h0, const void* d_o, const float* dht,
                          void* dq, void* dk, void* dv, void* dbeta, void* dgk, float* dh0,
                          void* workspace, size_t workspace_bytes, void* stream);
+
+/* The pair for callers that would rather spend memory than time: hdla_chunk_fwd_keep is hdla_chunk_fwd (or, with beta
+ * given, hdla_param_chunk_fwd: a and b are then ignored and may be NULL) whose per-chunk intermediates -- the operands
+ * of the state scans, (I - A_ab)^-1, the strong-decay flags -- are written into a buffer `kept` of
+ * hdla_workspace_bytes(dims, HDLA_PASS_FWD_KEEP) bytes that the caller holds until the backward pass;
+ * hdla_chunk_bwd_kept is hdla_chunk_bwd (hdla_param_chunk_bwd with beta: dbeta is written, da and db are not) that reads
+ * them there instead of recomputing them from the inputs, which saves the backward pass its first kernel.  The reference
+ * keeps only the inputs between the passes and recomputes (ctx.save_for_backward at HRDPLR/hrdplr.py:137, recompute at
+ * :161-198); these two trade that for about 1.2x the inputs' bytes of extra memory held between the passes.  `kept` is
+ * only read by the backward call (it can be used again); `workspace` is scratch of
+ * hdla_workspace_bytes(dims, HDLA_PASS_BWD_KEPT) bytes.  Same dims, inputs and stream ordering as the forward call. */
+int hdla_chunk_fwd_keep(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
+                        const void* b, const void* beta, const void* gk, const float* h0, void* o, float* ht,
+                        void* kept, size_t kept_bytes, void* stream);
+int hdla_chunk_bwd_kept(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
+                        const void* b, const void* beta, const void* gk, const float* h0, const void* d_o,
+                        const float* dht, void* dq, void* dk, void* dv, void* da, void* db, void* dbeta, void* dgk,
+                        float* dh0, void* kept, size_t kept_bytes, void* workspace, size_t workspace_bytes,
+                        void* stream);
 
 /* Profiling / debugging aid with no counterpart in the reference: runs only the kernels selected by `stages`
  * (a bit mask) of the forward (pass 0) or backward (pass 1) launch sequence, in order, on the same workspace, so

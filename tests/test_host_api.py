@@ -55,11 +55,20 @@ def test_workspace_size_and_layout():
     assert L["SB_STRIDE"] % 1024 == 0 and L["SB_STRIDE"] >= (K // 16 + 2) * 512
     assert L["UT"] - L["W"] >= d.H * L["nch"] * L["SA_STRIDE"] and L["TM"] - L["QGT"] >= d.H * L["nch"] * L["SB_STRIDE"]
     Lf = _lib.workspace_layout(d, 0)
-    assert Lf["W"] < Lf["QG"] < Lf["AQB"] < Lf["AQK"] < Lf["EGL"] < Lf["W"] + Lf["SA_STRIDE"] and Lf["SB_STRIDE"] == 0
+    # the forward block: the backward pass's block as a prefix (same offsets of W, BGT, KGT, EGL), then the output's parts
+    assert all(Lf[k] - Lf["W"] == L[k] - L["W"] for k in ("BGT", "KGT", "EGL"))
+    assert Lf["EGL"] < Lf["AQK"] < Lf["QG"] < Lf["AQB"] < Lf["W"] + Lf["SA_STRIDE"] and Lf["SB_STRIDE"] == 0
+    assert Lf["SA_STRIDE"] > L["SA_STRIDE"]
     # ragged T and packed sequences reserve one extra chunk per sequence
     assert _lib.workspace_layout(_dims(T=65), 0)["nch"] == 2 * 5
     assert _lib.workspace_layout(_dims(B=1, N=3, T=64, cu_seqlens=256), 0)["nch"] == 4 + 3
-    assert lib.hdla_workspace_bytes(ctypes.byref(d), 2) == 0
+    # a forward pass that keeps its intermediates for the backward pass, and the scratch of that backward pass
+    keep, kept = lib.hdla_workspace_bytes(ctypes.byref(d), 2), lib.hdla_workspace_bytes(ctypes.byref(d), 3)
+    assert fwd < keep and 0 < kept < bwd and keep + kept > bwd
+    Lk, Ls = _lib.workspace_layout(d, 2), _lib.workspace_layout(d, 3)
+    assert Lk["SA_STRIDE"] == Lf["SA_STRIDE"] and Lk["TM"] > Lk["AQBT"] > Lk["QGT"] > Lk["VTT"] and Lk["STRONG"] > Lk["TM"]
+    assert Ls["HC"] == 0 and Ls["HC"] < Ls["DHC"] < Ls["DVN"] < Ls["total"] == kept
+    assert lib.hdla_workspace_bytes(ctypes.byref(d), 4) == 0 and lib.hdla_workspace_bytes(ctypes.byref(d), -1) == 0
 
 
 @pytest.mark.parametrize("kw,code", [
