@@ -17,11 +17,13 @@ constexpr int CHUNK = 16;
 inline size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-int check_dims(const hdla_dims* d) {
+// max_dim: 128 for the chunked entry points, 256 for the token-serial ones
+int check_dims(const hdla_dims* d, int max_dim = 128) {
     if (!d) return HDLA_ERR_NULL;
     if (d->R != 2) return HDLA_ERR_RANK;
     if (d->B < 1 || d->T < 0 || d->H < 1 || d->N < 1) return HDLA_ERR_SHAPE;
-    if (!((d->K == 64 || d->K == 128) && (d->V == 64 || d->V == 128))) return HDLA_ERR_SHAPE;
+    auto ok = [&](int x) { return x == 64 || x == 128 || (x == 256 && max_dim >= 256); };
+    if (!ok(d->K) || !ok(d->V)) return HDLA_ERR_SHAPE;
     if (d->H > 65535) return HDLA_ERR_SHAPE;
     if (d->in_dtype != HDLA_BF16 && d->in_dtype != HDLA_FP32) return HDLA_ERR_DTYPE;
     if (d->gk_dtype != HDLA_BF16 && d->gk_dtype != HDLA_FP32) return HDLA_ERR_DTYPE;
@@ -212,7 +214,7 @@ const char* hdla_strerror(int code) {
     switch (code) {
         case HDLA_OK: return "success";
         case HDLA_ERR_NULL: return "a required pointer is NULL";
-        case HDLA_ERR_SHAPE: return "unsupported shape (need K,V in {64,128}, B,H,N >= 1, T >= 0, H,N <= 65535, chunks x heads < 2^31)";
+        case HDLA_ERR_SHAPE: return "unsupported shape (need K,V in {64,128}, or 256 as well for the token-serial entry points; B,H,N >= 1, T >= 0, H,N <= 65535, chunks x heads < 2^31)";
         case HDLA_ERR_RANK: return "only rank R = 2 is supported";
         case HDLA_ERR_DTYPE: return "unsupported dtype (in_dtype bf16|fp32; gk fp32, or bf16 with bf16 inputs)";
         case HDLA_ERR_WORKSPACE: return "workspace is NULL, not 256-byte aligned, or smaller than hdla_workspace_bytes()";
@@ -421,7 +423,7 @@ static int run_recurrent(const hdla_dims* dims, const void* q, const void* k, co
 int hdla_recurrent_fwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
                        const void* b, const void* gk, int reverse, const float* h0, void* o, float* ht,
                        void* stream) {
-    const int rc = check_dims(dims);
+    const int rc = check_dims(dims, 256);
     if (rc) return rc;
     if (dims->T > 0 && (!q || !k || !v || !a || !b || !gk || !o)) return HDLA_ERR_NULL;
     if (!aligned16(h0) || !aligned16(ht)) return HDLA_ERR_ALIGN;
@@ -430,7 +432,7 @@ int hdla_recurrent_fwd(const hdla_dims* dims, const void* q, const void* k, cons
 
 int hdla_param_recurrent_fwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* beta,
                              const void* gk, int reverse, const float* h0, void* o, float* ht, void* stream) {
-    const int rc = check_dims(dims);
+    const int rc = check_dims(dims, 256);
     if (rc) return rc;
     if (!beta) return HDLA_ERR_NULL;
     if (dims->T > 0 && (!q || !k || !v || !gk || !o)) return HDLA_ERR_NULL;

@@ -160,6 +160,13 @@ hipError_t launch_recurrent(const RecurrentArgs<T>& a, int K, int V, hipStream_t
     if (K == 128 && V == 128) return launch_recurrent_kv<T, 128, 128>(a, stream);
     if (K == 64 && V == 128) return launch_recurrent_kv<T, 64, 128>(a, stream);
     if (K == 128 && V == 64) return launch_recurrent_kv<T, 128, 64>(a, stream);
+    // head sizes up to 256 (the reference's token-serial kernel takes any K, HRDPLR/recurrent.py:155-176): the state
+    // block of a workgroup is K x 64 values in registers, 64 per lane at K = 256
+    if (K == 256 && V == 256) return launch_recurrent_kv<T, 256, 256>(a, stream);
+    if (K == 256 && V == 128) return launch_recurrent_kv<T, 256, 128>(a, stream);
+    if (K == 128 && V == 256) return launch_recurrent_kv<T, 128, 256>(a, stream);
+    if (K == 256 && V == 64) return launch_recurrent_kv<T, 256, 64>(a, stream);
+    if (K == 64 && V == 256) return launch_recurrent_kv<T, 64, 256>(a, stream);
     return hipErrorInvalidValue;
 }
 template hipError_t launch_recurrent<bf16>(const RecurrentArgs<bf16>&, int, int, hipStream_t);

@@ -35,11 +35,11 @@ def _require_gpu(*ts):
                                  f"{t.device}); there is no CPU fallback")
 
 
-def _native_dim(d: int) -> int:
-    for n in _NATIVE_D:
+def _native_dim(d: int, sizes=_NATIVE_D) -> int:
+    for n in sizes:
         if d <= n:
             return n
-    raise ValueError(f"head dimension {d} is not supported (maximum {_NATIVE_D[-1]})")
+    raise ValueError(f"head dimension {d} is not supported (maximum {sizes[-1]})")
 
 
 def _pad_last(x: Optional[torch.Tensor], d: int) -> Optional[torch.Tensor]:

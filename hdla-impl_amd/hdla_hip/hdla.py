@@ -231,7 +231,7 @@ def fused_recurrent_hdla_delta_rule(
     gk = log_f
     if gk.dtype != torch.float32 and gk.dtype != q.dtype:
         gk = gk.float()
-    Kn, Vn = _native_dim(K), _native_dim(V)
+    Kn, Vn = _native_dim(K, (64, 128, 256)), _native_dim(V, (64, 128, 256))
     h0 = None if initial_state is None else initial_state.to(torch.float32)
     if h0 is not None and (Kn != K or Vn != V):
         h0 = F.pad(h0, (0, Vn - V, 0, Kn - K))

@@ -14,6 +14,8 @@ from . import _lib
 from .chunk import _native_dim, _pad_last, _rank2, _require_gpu
 from .utils import autocast_custom_bwd, autocast_custom_fwd, contiguous
 
+_RECURRENT_D = (64, 128, 256)     # head sizes the token-serial kernel is built for (smaller ones are zero-padded)
+
 
 def fused_recurrent_dplr_delta_rule_fwd(q, k, v, a, b, gk, rank_ab, scale=1.0, initial_state=None,
                                         output_final_state=False, reverse=False, cu_seqlens=None):
@@ -122,7 +124,7 @@ def fused_recurrent_dplr_delta_rule(
     k, v, a, b = k.to(q.dtype), v.to(q.dtype), a.to(q.dtype), b.to(q.dtype)
     if gk.dtype != torch.float32 and gk.dtype != q.dtype:
         gk = gk.float()
-    Kn, Vn = _native_dim(K), _native_dim(V)
+    Kn, Vn = _native_dim(K, _RECURRENT_D), _native_dim(V, _RECURRENT_D)
     h0 = initial_state
     if h0 is not None and (Kn != K or Vn != V):
         h0 = F.pad(h0, (0, Vn - V, 0, Kn - K))

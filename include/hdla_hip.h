@@ -30,7 +30,8 @@
  *     synchronise, keep no global mutable state and are reentrant as long as workspaces are distinct.
  *   - Return value: 0 = success, < 0 = argument error detected on the host before any launch (see
  *     hdla_strerror), > 0 = a hipError_t from a kernel launch.
- *   - Supported: R = 2; K, V in {64, 128}; in_dtype bf16 or fp32; gk fp32, or bf16 when in_dtype is bf16.
+ *   - Supported: R = 2; K, V in {64, 128} (the token-serial entry points also 256); in_dtype bf16 or fp32; gk fp32,
+ *     or bf16 when in_dtype is bf16.
  *     gk (log-space decay, <= 0) may be arbitrarily strong: where a channel loses more than e^-70 within eight
  *     tokens the chunk's scores are formed by passes whose exponents cannot overflow, as the reference's
  *     re-centred sub-chunks are (HRDPLR/fwd_triton.py:420-463).

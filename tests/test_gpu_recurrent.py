@@ -103,6 +103,28 @@ def test_rank_one_and_padded_dims():
     assert O.rel_l2(o, o_r) <= 1e-5 and O.rel_l2(ht, ht_r) <= 1e-5
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 5e-3)])
+@pytest.mark.parametrize("K,V", [(256, 256), (200, 72), (64, 256), (256, 128)])
+def test_head_sizes_up_to_256(dtype, tol, K, V):
+    """The reference's token-serial kernel takes any K (BK = next_pow2(K), recurrent.py:155-176); here up to 256, both
+    operators (a, b given; a, b formed in the kernel), with a packed batch."""
+    from hdla_hip import fused_recurrent_hdla_delta_rule
+    inp = make_inputs(700 + K + V, 1, 23, 2, K, V, gk_div=2.0, n_states=2)
+    cu = torch.tensor([0, 9, 23])
+    o, ht = _run(inp, dtype, scale=0.5, initial_state=inp.h0.to(DEV), output_final_state=True, cu_seqlens=cu.to(DEV))
+    o_r, ht_r = _ref(inp, dtype, scale=0.5, initial_state=inp.h0, cu_seqlens=cu)
+    assert o.shape == inp.v.shape and ht.shape == inp.h0.shape
+    assert O.rel_l2(o, o_r) <= tol and O.rel_l2(ht, ht_r) <= min(tol, 1e-5)
+    g = torch.Generator().manual_seed(1)
+    beta = 2 * torch.rand(1, 23, 2, 1, generator=g)
+    q, k, v, lf = (x.to(dtype) for x in (inp.q, inp.k, inp.v, inp.gk))
+    o2, h2 = fused_recurrent_hdla_delta_rule(q.to(DEV), k.to(DEV), v.to(DEV), beta.to(dtype).to(DEV), lf.to(DEV), scale=1.0,
+                                             initial_state=inp.h0[:1].to(DEV), output_final_state=True)
+    a, b = O.parameterize_a_b(beta.to(dtype).double(), k.double(), lf.double())
+    o2_r, h2_r = O.recurrence(q, k, v, a.to(dtype), b.to(dtype), lf, 1.0, inp.h0[:1])
+    assert O.rel_l2(o2, o2_r) <= tol and O.rel_l2(h2, h2_r) <= min(tol, 1e-5)
+
+
 def test_backward_raises():
     inp = make_inputs(34, 1, 4, 1, 64, 64)
     t = [x.float().to(DEV).requires_grad_() for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
