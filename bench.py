@@ -41,6 +41,8 @@ def _args():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="train", choices=["train", "fwd", "varlen", "decode", "copy", "hdla", "hdla_decode", "norm", "layer", "layer_decode"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--brief", action="store_true", help="the named workload only: no other configurations, no keep_forward "
+                    "variant (what the profiler runs recorded under profiles/ use)")
     return ap.parse_args()
 
 
@@ -127,12 +129,12 @@ def measured_traffic(workload, kernel_key, K, V):
         if not k.startswith(name + "_kernel<"):
             continue
         targs = [a.strip() for a in k[k.index("<") + 1:k.rindex(">")].split(",")]
-        # prep<T, GKF32, K, V, BWD, HD>, scan_fwd<T, K, V, NWC, WRITE_O>, scan_pair<T, K, V, NWC>,
+        # prep<T, GKF32, K, V, MODE (0 forward, 1 backward, 2 kept forward), HD>, scan_fwd<T, K, V, NWC, WRITE_O>, scan_pair<T, K, V, NWC>,
         # chunk_grad<T, GKF32, K, V, HD>, recurrent<T, K, V, BV, HD>
         kv = targs[2:4] if name in ("prep", "chunk_grad") else targs[1:3]
         if kv != [str(K), str(V)]:
             continue
-        if name == "prep" and ((targs[4] == "true") != (pass_ == "bwd") or targs[5:] == ["true"]):
+        if name == "prep" and (targs[4] != ("1" if pass_ == "bwd" else "0") or targs[5:] == ["true"]):
             continue
         if name == "scan_fwd" and (targs[4] == "true") != (pass_ == "fwd"):
             continue
@@ -592,8 +594,8 @@ def main():
                    roofline=None)
         print(json.dumps(res))
         return
-    res.update(run_chunk_workload(wl, cfg, args.steps, args.warmup, dev))
-    if wl == "train":
+    res.update(run_chunk_workload(wl, cfg, args.steps, args.warmup, dev, keep_variant=not args.brief))
+    if wl == "train" and not args.brief:
         # the other configurations, measured in this process after the headline (fewer steps: they are reported, the
         # headline is what the step count is about)
         n_other = max(5, args.steps // 3)
@@ -617,7 +619,7 @@ def main():
     print(json.dumps(res))
 
 
-def run_chunk_workload(wl, cfg, steps, warmup, dev):
+def run_chunk_workload(wl, cfg, steps, warmup, dev, keep_variant=True):
     """One of the chunked configurations (train = 2, fwd = 1, varlen = 3): whole-step time through the public operator,
     then every kernel by itself."""
     from hdla_hip import chunk_hrdplr_delta_rule
@@ -641,7 +643,7 @@ def run_chunk_workload(wl, cfg, steps, warmup, dev):
     sec = time_steps(step, steps, warmup)
     # the same step with keep_forward=True (an option, off by default: the forward pass's per-chunk intermediates stay
     # alive until the backward pass, which then does not recompute them); `value` is the default route
-    sec_keep = time_steps(lambda: step(True), steps, warmup) if wl != "fwd" else None
+    sec_keep = time_steps(lambda: step(True), steps, warmup) if wl != "fwd" and keep_variant else None
     tokens = B * T
     # per-kernel durations
     raw = [x.detach() for x in leaves] + [None if h0 is None else h0.detach(), do, dht]
