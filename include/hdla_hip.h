@@ -147,7 +147,7 @@ int hdla_param_chunk_bwd(const hdla_dims* dims, const void* q, const void* k, co
  * hdla_chunk_bwd_kept is hdla_chunk_bwd (hdla_param_chunk_bwd with beta: dbeta is written, da and db are not) that reads
  * them there instead of recomputing them from the inputs, which saves the backward pass its first kernel.  The reference
  * keeps only the inputs between the passes and recomputes (ctx.save_for_backward at HRDPLR/hrdplr.py:137, recompute at
- * :161-198); these two trade that for about 1.2x the inputs' bytes of extra memory held between the passes.  `kept` is
+ * :161-198); these two trade that for about 1.6x the inputs' bytes of extra memory held between the passes.  `kept` is
  * only read by the backward call (it can be used again); `workspace` is scratch of
  * hdla_workspace_bytes(dims, HDLA_PASS_BWD_KEPT) bytes.  Same dims, inputs and stream ordering as the forward call. */
 int hdla_chunk_fwd_keep(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
