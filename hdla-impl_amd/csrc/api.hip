@@ -76,7 +76,7 @@ int make_layout(const hdla_dims* d, int pass, WsLayout& L, int& nch) {
         L.DVN = take(chw * 2 * 16 * V * es);
     }
     if (d->cu_seqlens && prep_out) {
-        L.CHUNK_OFF = take((size_t)(d->N + 1) * 4);
+        L.CHUNK_OFF = take((size_t)(2 * d->N + 1) * 4);          // chunk_off [N+1], then order [N]
         L.CHUNK_SEQ = take((size_t)(nch > 0 ? nch : 1) * 4);
     }
     L.total = off > 0 ? off : 256;
@@ -103,6 +103,7 @@ void bind_ws(ChunkArgs<T>& a, const hdla_dims* d, const WsLayout& LP, void* prep
     a.st.cu = d->cu_seqlens;
     a.st.chunk_off = d->cu_seqlens ? reinterpret_cast<const int32_t*>(base + LP.CHUNK_OFF) : nullptr;
     a.st.chunk_seq = d->cu_seqlens ? reinterpret_cast<const int32_t*>(base + LP.CHUNK_SEQ) : nullptr;
+    a.st.order = d->cu_seqlens ? a.st.chunk_off + d->N + 1 : nullptr;
     a.st.T = d->T;
     a.st.NT = (d->T + CHUNK - 1) / CHUNK;
     a.st.N = d->N;

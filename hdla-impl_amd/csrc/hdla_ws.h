@@ -14,11 +14,13 @@ struct bf16 { uint16_t x; };  // storage type tag for bf16 tensors (raw bits)
 
 // Tokens live on one flattened axis of B*T rows.  Without cu_seqlens sequence n covers rows [n*T, (n+1)*T) and
 // has NT = ceil(T/16) chunks; with cu_seqlens (device int64[N+1], batch 1) sequence n covers [cu[n], cu[n+1])
-// and its chunks are numbered from chunk_off[n] (device int32[N+1], built by build_chunk_table_kernel).
+// and its chunks are numbered from chunk_off[n] (device int32[N+1], built by build_chunk_table_kernel, which leaves
+// the int32[N] `order` right behind it).
 struct SeqTab {
     const int64_t* cu;        // nullable
     const int32_t* chunk_off; // valid when cu != nullptr
     const int32_t* chunk_seq; // valid when cu != nullptr: sequence of each chunk
+    const int32_t* order;     // valid when cu != nullptr: int32[N], the sequences from the one with the most chunks down
     int T, NT, N;
     int nch;                  // chunk slots the workspace is laid out for (an upper bound with cu_seqlens)
 };

@@ -331,6 +331,7 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
 }
 
 // ---- chunk table for packed variable-length batches ----------------------------------------------------------
+constexpr int ORDER_MAX_N = 2048;      // beyond this many sequences they are taken as they come (ranking is quadratic)
 __global__ void build_chunk_table_kernel(const int64_t* cu, int N, int T, int nch, int32_t* chunk_off, int32_t* chunk_seq) {
     // one workgroup; N is small (number of packed sequences)
     __shared__ int total;
@@ -354,6 +355,21 @@ __global__ void build_chunk_table_kernel(const int64_t* cu, int N, int T, int nc
             if (chunk_off[mid] <= cid) lo = mid; else hi = mid - 1;
         }
         chunk_seq[cid] = lo;
+    }
+    // order[r] = the sequence with the r-th most chunks (ties by index): the scans start their workgroups in this
+    // order, so that when there are more workgroups than compute units the long sequences are not the ones that wait
+    int32_t* order = chunk_off + N + 1;
+    for (int n = threadIdx.x; n < N; n += blockDim.x) {
+        int r = n;
+        if (N <= ORDER_MAX_N) {
+            const int len = chunk_off[n + 1] - chunk_off[n];
+            r = 0;
+            for (int m = 0; m < N; ++m) {
+                const int lm = chunk_off[m + 1] - chunk_off[m];
+                r += (lm > len || (lm == len && m < n)) ? 1 : 0;
+            }
+        }
+        order[r] = n;
     }
 }
 

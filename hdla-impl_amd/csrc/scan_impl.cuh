@@ -207,7 +207,7 @@ template <typename T, int K, int V, int NWC, int SLOT_, ScanOut OUT> struct Scan
 
 // ---- forward -------------------------------------------------------------------------------------------------
 template <typename T, int K, int V, int NWC, bool WRITE_O>
-__device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem, int split) {
+__device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem, int n, int split) {
     typedef ScanCfg<T, K, V, NWC> C;
     constexpr int KT = K / 16, KT2 = KT / 2, VT = V / 16, NM = C::NM, ES = sizeof(T);
     constexpr BlkF B = blk_fwd(K, sizeof(T), WRITE_O);
@@ -219,7 +219,7 @@ __device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem,
     constexpr int OROW = L::OROW, OB_HC = L::OB_HC, OB = L::OB;
     char* const outbox = smem + NSLOT * SLOT;
 
-    const int h = blockIdx.x, n = blockIdx.y;
+    const int h = blockIdx.x;
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int vt0 = split * NWC;                          // first column block of this workgroup
     const int l = lane_id(), g = l >> 4, c = l & 15;
@@ -484,7 +484,7 @@ __device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem,
 // ---- backward ------------------------------------------------------------------------------------------------
 // Step t handles chunk c1-1-t.
 template <typename T, int K, int V, int NWC>
-__device__ __forceinline__ void scan_bwd_body(const ChunkArgs<T>& p, char* smem, int split) {
+__device__ __forceinline__ void scan_bwd_body(const ChunkArgs<T>& p, char* smem, int n, int split) {
     typedef ScanCfg<T, K, V, NWC> C;
     constexpr int KT = K / 16, KT2 = KT / 2, VT = V / 16, NM = C::NM, ES = sizeof(T);
     // LDS slot: [BG | WT] (BGT and W of the forward-scan block, transposed on their way in) | EGL | QGT | AQBT
@@ -498,7 +498,7 @@ __device__ __forceinline__ void scan_bwd_body(const ChunkArgs<T>& p, char* smem,
     constexpr int OB_HC = L::OB_HC, OB = L::OB;
     char* const outbox = smem + NSLOT * SLOT;
 
-    const int h = blockIdx.x, n = blockIdx.y;
+    const int h = blockIdx.x;
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int vt0 = split * NWC;
     const int l = lane_id(), g = l >> 4, c = l & 15;
@@ -705,16 +705,21 @@ __device__ __forceinline__ void scan_bwd_body(const ChunkArgs<T>& p, char* smem,
 }
 
 // ---- kernels ---------------------------------------------------------------------------------------------------
-// grid = (H, N, directions * SPLIT); blockIdx.z = direction * SPLIT + split
+// grid = (H, directions * SPLIT, N): blockIdx.y = direction * SPLIT + split; blockIdx.z counts the sequences, packed
+// ones from the longest down.  Workgroups start in the order of their linear index (x fastest): the workgroups of one
+// (sequence, head) are H apart, which puts them on the same XCD (and its L2, where they share the chunk blocks) when H
+// is a multiple of 8, and when the launch has more workgroups than the device holds at once, the long sequences,
+// which decide when the launch ends, start first and the short ones fill in behind them.
+__device__ __forceinline__ int scan_sequence(const SeqTab& st) { return st.cu ? st.order[blockIdx.z] : (int)blockIdx.z; }
 template <typename T, int K, int V, int NWC, bool WRITE_O>
 __global__ __launch_bounds__((ScanCfg<T, K, V, NWC>::THREADS)) void scan_fwd_kernel(ChunkArgs<T> p) {
     __shared__ __attribute__((aligned(16))) char smem[ScanLds<T, K, V, NWC, blk_fwd(K, sizeof(T), WRITE_O).SIZE + ScanCfg<T, K, V, NWC>::OWN_FWD, WRITE_O ? OUT_O : OUT_STATE>::BYTES];
-    scan_fwd_body<T, K, V, NWC, WRITE_O>(p, smem, blockIdx.z);
+    scan_fwd_body<T, K, V, NWC, WRITE_O>(p, smem, scan_sequence(p.st), blockIdx.y);
 }
 template <typename T, int K, int V, int NWC>
 __global__ __launch_bounds__((ScanCfg<T, K, V, NWC>::THREADS)) void scan_bwd_kernel(ChunkArgs<T> p) {
     __shared__ __attribute__((aligned(16))) char smem[ScanLds<T, K, V, NWC, slot_bwd(K, sizeof(T)).SIZE, OUT_GRAD>::BYTES];
-    scan_bwd_body<T, K, V, NWC>(p, smem, blockIdx.z);
+    scan_bwd_body<T, K, V, NWC>(p, smem, scan_sequence(p.st), blockIdx.y);
 }
 // Both scans of the backward pass in one launch: they depend on the prep kernel only, not on each other.
 template <typename T, int K, int V, int NWC>
@@ -723,15 +728,16 @@ __global__ __launch_bounds__((ScanCfg<T, K, V, NWC>::THREADS)) void scan_pair_ke
     constexpr int NB = ScanLds<T, K, V, NWC, slot_bwd(K, sizeof(T)).SIZE, OUT_GRAD>::BYTES;
     constexpr int SPLIT = ScanCfg<T, K, V, NWC>::SPLIT;
     __shared__ __attribute__((aligned(16))) char smem[NF > NB ? NF : NB];
-    if (blockIdx.z < SPLIT) scan_fwd_body<T, K, V, NWC, false>(p, smem, blockIdx.z);
-    else scan_bwd_body<T, K, V, NWC>(p, smem, blockIdx.z - SPLIT);
+    const int n = scan_sequence(p.st);
+    if (blockIdx.y < SPLIT) scan_fwd_body<T, K, V, NWC, false>(p, smem, n, blockIdx.y);
+    else scan_bwd_body<T, K, V, NWC>(p, smem, n, blockIdx.y - SPLIT);
 }
 
 // ---- launchers -------------------------------------------------------------------------------------------------
 template <typename T, int K, int V, int NWC>
 static hipError_t launch_scan_nwc(const ChunkArgs<T>& a, ScanKind kind, hipStream_t stream) {
     typedef ScanCfg<T, K, V, NWC> C;
-    dim3 grid(a.H, a.st.N, C::SPLIT * (kind == SCAN_PAIR ? 2 : 1)), block(C::THREADS);
+    dim3 grid(a.H, C::SPLIT * (kind == SCAN_PAIR ? 2 : 1), a.st.N), block(C::THREADS);
     switch (kind) {
         case SCAN_FWD_O: hipLaunchKernelGGL((scan_fwd_kernel<T, K, V, NWC, true>), grid, block, 0, stream, a); break;
         case SCAN_FWD: hipLaunchKernelGGL((scan_fwd_kernel<T, K, V, NWC, false>), grid, block, 0, stream, a); break;

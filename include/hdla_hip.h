@@ -83,7 +83,9 @@ typedef struct hdla_ws_layout {
     int64_t W, UT, KGT, BGT, VTT, EGL, QG, AQK, AQB, AQBT, QGT, TM, HC, DHC, DVN;
     int64_t STRONG;            /* int32 per (head, chunk) slot: nonzero where the chunk takes the strong-decay route */
     int64_t SA_STRIDE, SB_STRIDE;
-    int64_t CHUNK_OFF, CHUNK_SEQ;
+    int64_t CHUNK_OFF, CHUNK_SEQ;  /* with cu_seqlens: int32[N+1] first chunk slot of each sequence, followed by int32[N]
+                                    * the sequences in the order the scans start them (most chunks first); int32[nch] the
+                                    * sequence of each chunk slot */
     int64_t total;
 } hdla_ws_layout;
 

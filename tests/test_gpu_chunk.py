@@ -248,6 +248,52 @@ def test_varlen_ragged_and_empty_sequences():
     _compare(_gpu(inp, torch.float32, 1.0, cu=cu), _oracle(inp, torch.float32, 1.0, cu=cu), torch.float32)
 
 
+@pytest.mark.parametrize("N,max_len", [(300, 20), (2100, 3)])
+def test_many_packed_sequences_and_their_start_order(N, max_len):
+    """Packed batches of many short sequences in no particular order, some of them empty: results against the
+    float64 recurrence per sequence, and the table the scans take their starting order from (after the chunk offsets in
+    the workspace): every sequence once, the ones with more chunks first, ties by index; beyond 2048 sequences they
+    are taken as they come."""
+    from hdla_hip import _lib
+    from hdla_hip import chunk as CK
+    g = torch.Generator().manual_seed(N)
+    lens = torch.randint(0, max_len + 1, (N,), generator=g)
+    cu = torch.cat([torch.zeros(1, dtype=torch.int64), lens.cumsum(0)])
+    T = int(cu[-1])
+    inp = make_inputs(40 + N, 1, T, 2, 64, 64, n_states=N)
+    dtype = torch.float32
+    if N <= 300:
+        _compare(_gpu(inp, dtype, 1.0, cu=cu), _oracle(inp, dtype, 1.0, cu=cu), dtype, what=f"{N} packed sequences")
+    else:
+        # many more sequences than the oracle's token loop is worth: forward pass against per-sequence calls for a sample
+        t = [x.to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+        o, ht = chunk_hrdplr_delta_rule(*t, 2, scale=1.0, initial_state=inp.h0.to(DEV), output_final_state=True, cu_seqlens=cu.to(DEV))
+        for n in [0, 1, 700, 2047, 2048, N - 1]:
+            s, e = int(cu[n]), int(cu[n + 1])
+            if e == s:
+                assert torch.equal(ht[n], inp.h0[n].to(DEV))
+                continue
+            q, k, v, a, b, gk = t
+            on, hn = chunk_hrdplr_delta_rule(q[:, s:e], k[:, s:e], v[:, s:e], a[:, 2 * s:2 * e], b[:, 2 * s:2 * e], gk[:, s:e], 2,
+                                             scale=1.0, initial_state=inp.h0[n:n + 1].to(DEV), output_final_state=True)
+            assert torch.equal(o[:, s:e], on) and torch.equal(ht[n:n + 1], hn), n
+    d = lambda x: x.to(dtype).to(DEV).contiguous()
+    out = CK.chunk_hrdplr_bwd(d(inp.q), d(inp.k), d(inp.v), d(inp.a), d(inp.b), d(inp.gk), 1.0, inp.h0.to(DEV), d(inp.do),
+                              inp.dht.to(DEV), cu_seqlens=cu.to(DEV), keep_workspace=True)
+    ws, dims = out[-2], out[-1]
+    torch.cuda.synchronize()
+    off = _lib.workspace_layout(dims, 1)["CHUNK_OFF"]
+    tab = ws[off:off + 4 * (2 * N + 1)].view(torch.int32).cpu()
+    chunks = (lens + 15) // 16
+    assert torch.equal(tab[:N + 1].long(), torch.cat([torch.zeros(1, dtype=torch.int64), chunks.cumsum(0)]))
+    order = tab[N + 1:].long()
+    if N <= 2048:
+        want = sorted(range(N), key=lambda n: (-int(chunks[n]), n))
+    else:
+        want = list(range(N))
+    assert order.tolist() == want
+
+
 def test_device_side_sequence_table_is_forced_into_the_token_range():
     """A table that is already on the GPU is not validated on the host; the kernels force its entries into [0, T], so
     one that runs past the end gives what the table cut at T gives (and rows outside every sequence stay unwritten)."""
