@@ -95,13 +95,18 @@ def algorithmic_bytes(kernel, pass_, K, V, es, gs):
 
 
 def kernel_sources_digest():
-    """Digest of the HIP sources: the counter summaries under profiles/ record the one they were taken with."""
+    """Digest of the HIP sources (comments and white space left out, so that only a change of the code changes it): the
+    counter summaries under profiles/ record the one they were taken with."""
     import glob
     import hashlib
+    import re
     h = hashlib.sha256()
     for f in sorted(glob.glob(os.path.join(ROOT, "hdla-impl_amd", "csrc", "*.*"))):
         if f.endswith((".hip", ".cuh", ".h", ".inc")):
-            h.update(open(f, "rb").read())
+            text = open(f, encoding="utf-8").read()
+            text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+            text = re.sub(r"//[^\n]*", " ", text)
+            h.update(os.path.basename(f).encode() + b"\0" + " ".join(text.split()).encode() + b"\0")
     return h.hexdigest()[:16]
 
 

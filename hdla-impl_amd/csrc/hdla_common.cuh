@@ -87,9 +87,9 @@ __device__ __forceinline__ f32x4 mm(Frag<float> frows, Frag<float> finner, f32x4
     return acc;
 }
 
-// (The 16x16x32 bf16 MFMA of gfx950 would do two of these products in the time of one.  It is not used: this
-// toolchain lets a vector ALU instruction overwrite the accumulator-input registers of such an MFMA a few cycles
-// after its issue, while the hardware still reads them, and results then depend on the register allocation.)
+// (The 16x16x32 bf16 MFMA of gfx950 would do two of these products in the time of one.  It is not used: built with
+// it, the state scans gave wrong results that depended on the register allocation, while a kernel of nothing but
+// such products was exact; the cause was not established, and no kernel here is bound by its matrix products.)
 
 // Split operands for the score products of the bf16 path: x = hi + lo with both halves bf16, and
 // P Q^T ~ Ph Qh^T + Ph Ql^T + Pl Qh^T, which removes the rounding of the decayed operands (the largest single
