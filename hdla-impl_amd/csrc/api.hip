@@ -41,7 +41,7 @@ int make_layout(const hdla_dims* d, int pass, WsLayout& L, int& nch) {
     if (d->N > 65535) return HDLA_ERR_SHAPE;
     const int NT = (d->T + CHUNK - 1) / CHUNK;
     const long long nch64 = d->cu_seqlens ? (long long)NT + d->N : (long long)d->B * NT;
-    if (nch64 * d->H > 0x7fffffffLL) return HDLA_ERR_SHAPE;        // one workgroup per (chunk, head), one grid dimension
+    if (nch64 * d->H > 0x7fff0000LL) return HDLA_ERR_SHAPE;        // one workgroup per (chunk, head), one grid dimension (and room for the strided loops over them)
     nch = (int)nch64;
     const size_t es = d->in_dtype == HDLA_BF16 ? 2 : 4;
     const size_t chw = (size_t)d->H * (size_t)nch;
