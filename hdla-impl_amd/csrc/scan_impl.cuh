@@ -393,6 +393,9 @@ __device__ __forceinline__ void scan_fwd_body(const ChunkArgs<T>& p, char* smem,
             o = mm(aqb[1], vnb[1], o);
             if (NM) st_frag(reinterpret_cast<T*>(ob + c * OROW) + 16 * wv + 4 * g, to_frag<T>(o));
             else if (c < len) st_frag(p.o + ((tok0 + c) * H + h) * V + 16 * vt + 4 * g, to_frag<T>(o));
+            // the output leaves for the outbox before the state update below, not after it: the barrier that ends the step
+            // waits for this LDS write, and behind the update's products the wait is free
+            if (NM && PIPE) __builtin_amdgcn_sched_barrier(0);
         }
         // S <- exp(g_last) S + kg^T v + sum_s bg_s^T v_new_s
 #pragma unroll
