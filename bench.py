@@ -39,7 +39,7 @@ def _args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="train", choices=["train", "fwd", "varlen", "decode", "copy", "hdla", "hdla_decode", "norm", "layer", "layer_decode"])
+    ap.add_argument("--workload", default="train", choices=["train", "fwd", "varlen", "decode", "copy", "hdla", "hdla_decode", "norm", "layer", "layer_decode", "shapes"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--brief", action="store_true", help="the named workload only: no other configurations, no keep_forward "
                     "variant (what the profiler runs recorded under profiles/ use)")
@@ -303,6 +303,34 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     wl = args.workload
+    if wl == "shapes":
+        # not a benchmark configuration: the chunked forward + backward step over a range of shapes (bf16 inputs, fp32
+        # state, h0/do/dht given), default route and keep_forward, to show where the operator stands away from the
+        # headline shape (few heads: the scans are a serial chain per head; many: everything is bound by memory)
+        shapes = [(4, 2048, 16, 64, 64), (16, 512, 16, 64, 64), (64, 256, 16, 64, 64), (32, 1024, 16, 64, 64), (8, 2048, 32, 64, 64),
+                  (1, 8192, 16, 64, 64), (2, 2048, 8, 64, 64), (1, 65536, 2, 64, 64), (4, 2048, 16, 64, 128), (4, 2048, 16, 128, 64),
+                  (4, 2048, 16, 128, 128), (8, 2048, 32, 128, 128), (1, 16384, 16, 128, 128)]
+        from hdla_hip.synthetic import make_inputs
+        rows = []
+        for (B, T, H, K, V) in shapes:
+            inp = make_inputs(1, B, T, H, K, V)
+            leaves = [x.bfloat16().to(dev).requires_grad_(True) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+            h0 = inp.h0.to(dev).requires_grad_(True)
+            do, dht = inp.do.bfloat16().to(dev), inp.dht.to(dev)
+
+            def step(keep=False):
+                o, ht = chunk_hrdplr_delta_rule(*leaves, 2, scale=1.0, initial_state=h0, output_final_state=True, keep_forward=keep)
+                torch.autograd.grad([o, ht], leaves + [h0], [do, dht])
+            sec = time_steps(step, args.steps, args.warmup)
+            sec_keep = time_steps(lambda: step(True), args.steps, args.warmup)
+            compulsory = B * T * H * (13 * (K + V)) * 2          # 26 D elements of 2 bytes per token and head, D = (K + V) / 2
+            rows.append({"B": B, "T": T, "H": H, "K": K, "V": V, "ms_per_step": sec * 1e3, "tokens/s": B * T / sec,
+                         "whole_step_frac_hbm": compulsory / sec / (HBM_PEAK_GBS * 1e9),
+                         "keep_forward_ms_per_step": sec_keep * 1e3})
+            del leaves, h0, do, dht, inp
+            torch.cuda.empty_cache()
+        print(json.dumps({"metric": "chunked fwd+bwd over shapes (bf16)", "steps": args.steps, "warmup": args.warmup, "shapes": rows}))
+        return
     if wl == "copy":
         # calibration workload, not a benchmark of the operator: the library's streaming kernel, whose traffic per
         # launch is known exactly (the HBM traffic counters are scaled by what they read for the 1:1 launches,
