@@ -294,6 +294,41 @@ def test_many_packed_sequences_and_their_start_order(N, max_len):
     assert order.tolist() == want
 
 
+def test_degenerate_inputs():
+    """No tokens at all (the final state is the initial one and its gradient passes through, on both routes); one
+    token without any state; a packed batch whose sequences are all empty but one; gradients asked for one input only;
+    keep_forward under no_grad (nothing is kept)."""
+    for keep in (False, True):
+        z = make_inputs(50, 2, 0, 3, 64, 64)
+        t = [x.bfloat16().to(DEV).requires_grad_() for x in (z.q, z.k, z.v, z.a, z.b, z.gk)]
+        h0 = z.h0.to(DEV).requires_grad_()
+        o, ht = chunk_hrdplr_delta_rule(*t, 2, scale=1.0, initial_state=h0, output_final_state=True, keep_forward=keep)
+        assert o.shape == (2, 0, 3, 64) and torch.equal(ht, h0.detach())
+        (g,) = torch.autograd.grad([ht], [h0], [z.dht.to(DEV)])
+        assert torch.equal(g, z.dht.to(DEV))
+    one = make_inputs(51, 1, 1, 1, 64, 64)
+    t = [x.bfloat16().to(DEV).requires_grad_() for x in (one.q, one.k, one.v, one.a, one.b, one.gk)]
+    o, ht = chunk_hrdplr_delta_rule(*t, 2)
+    assert ht is None and o.shape == (1, 1, 1, 64)
+    o.sum().backward()
+    o_r, _ = O.recurrence(*[x.detach().double().cpu() for x in t], 64 ** -0.5, None)
+    assert O.rel_l2(o, o_r) <= 5e-3 and all(torch.isfinite(x.grad.float()).all() for x in t)
+    inp = make_inputs(52, 1, 5, 2, 64, 64, n_states=5)
+    cu = torch.tensor([0, 0, 0, 5, 5, 5])
+    got = _gpu(inp, torch.float32, 1.0, cu=cu)
+    _compare(got, _oracle(inp, torch.float32, 1.0, cu=cu), torch.float32, what="all sequences empty but one")
+    assert torch.equal(got[1][[0, 1, 3, 4]], inp.h0[[0, 1, 3, 4]].to(DEV))
+    part = make_inputs(53, 1, 40, 2, 64, 64)
+    t = [x.bfloat16().to(DEV) for x in (part.q, part.k, part.v, part.a, part.b, part.gk)]
+    t[2].requires_grad_()
+    o, _ = chunk_hrdplr_delta_rule(*t, 2)
+    o.sum().backward()
+    assert t[2].grad is not None and t[0].grad is None
+    with torch.no_grad():
+        o2, _ = chunk_hrdplr_delta_rule(*[x.detach() for x in t], 2, keep_forward=True)
+    assert torch.equal(o2, o.detach())
+
+
 def test_device_side_sequence_table_is_forced_into_the_token_range():
     """A table that is already on the GPU is not validated on the host; the kernels force its entries into [0, T], so
     one that runs past the end gives what the table cut at T gives (and rows outside every sequence stay unwritten)."""
