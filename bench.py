@@ -67,7 +67,8 @@ def interface_bytes(kernel, pass_, K, V, es, gs):
         return interface_bytes("scan_fwd", 1, K, V, es, gs) + interface_bytes("scan_bwd", 1, K, V, es, gs) - (W + BGT + EGL)
     if kernel == "chunk_grad":
         outs = 2 * 16 * K * es + 16 * K * gs + 2 * 32 * K * es + 16 * V * es
-        return inputs + 16 * V * es + TM + W + UT + HC + DHC + DVN + outs
+        # (w itself is not read: the kernel rebuilds it from TM and a, for the plain operator with decays in the inputs' type)
+        return inputs + 16 * V * es + TM + UT + HC + DHC + DVN + outs
     raise ValueError(kernel)
 
 

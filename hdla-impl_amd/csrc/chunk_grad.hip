@@ -4,7 +4,8 @@
 // HRDPLR/bwd_triton.py:30-105, the dv kernel :239-290, the dqg/dkg/dbg/dw/dgk_last kernel :309-487, the WY
 // backward :503-612, the score backward :627-883 and the log-decay gradient :899-948.  Its inputs are the
 // original tensors, do, and per chunk the state entering it (h), the gradient of the state leaving it (dh) and
-// the gradient of v_new, left in the workspace by the two scans.  Nothing but the seven gradients is written back.
+// the gradient of v_new, left in the workspace by the two scans, and (I - A_ab)^-1 and u from the prep kernel (w as
+// well with the HDLA parameterisation; otherwise it is rebuilt here).  Nothing but the seven gradients is written back.
 //
 // Two differences from the reference's algebra, both exact:
 //  * the WY backward never forms d(Tm): with X = [w | u] = Tm R, R = [ag | A_ak v] one has dR = Tm^T dX and
@@ -45,9 +46,12 @@ template <typename T, int K, int V> struct CgLds {
     static constexpr bool STAGE_OUT = ES == 2;
     static constexpr int OPK = K * ES + 16, OPV = V * ES + 16;       // padded rows
     static constexpr int PART_B = (NW / 2) * 9 * 1024, OUT_B = STAGE_OUT ? (7 * OPK + OPV) * CH : 0;
+    // all tiles of w (2 ranks), rebuilt by the waves from (I - A_ab)^-1 and a instead of read from the workspace: behind
+    // the sums above, in what is otherwise free until the staged rows are written
+    static constexpr int WALL_B = 2 * (K / 16) * TILE * ES;
     // per wave and token: three partial sums over channels of the backward of the HDLA parameterisation
     static constexpr int RED = KG + KG_B, RED_B = NW * 3 * CH * 4;
-    static constexpr int R1 = RED + RED_B, R1_B = PART_B > OUT_B ? PART_B : OUT_B;
+    static constexpr int R1 = RED + RED_B, WALL = R1 + PART_B, R1_B = PART_B + WALL_B > OUT_B ? PART_B + WALL_B : OUT_B;
     static constexpr int BYTES = R1 + R1_B;
 };
 
