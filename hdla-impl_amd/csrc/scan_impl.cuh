@@ -10,9 +10,10 @@
 // layout of the next product: w S, qg S and the rank updates chain through registers with no cross-lane
 // movement.  A workgroup holds NWC such waves; a head's V/16 column blocks are split over (V/16)/NWC workgroups.
 //
-// What bounds a step without the measures below is not arithmetic but memory: one compute unit sustains only a few tens of GB/s of loads
-// that miss to HBM however many it has in flight, a wave may have at most 63 memory instructions outstanding and
-// they complete in order, and all column blocks of a head need the same w / kg / bg / qg tiles.  Hence
+// What bounds a step without the measures below is not arithmetic but memory: one compute unit sustains only a few
+// tens of GB/s of loads that miss to HBM however many it has in flight, a wave may have at most 63 memory
+// instructions outstanding and they complete in order, and all column blocks of a head need the same w / kg / bg /
+// qg tiles.  Hence
 //  * few heads are spread over many compute units (the split above, chosen by the launcher from the number of
 //    heads), each workgroup fetching the chunk's shared operand block (one contiguous block per chunk, written
 //    by the prep kernel) once for its NWC waves;
