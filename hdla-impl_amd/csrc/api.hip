@@ -5,6 +5,7 @@
 
 #include <atomic>
 
+#include "fused_shapes.h"
 #include "hdla_launch.h"
 #include "hdla_ws.h"
 
@@ -30,7 +31,82 @@ int check_dims(const hdla_dims* d, int max_dim = 128) {
     if (d->in_dtype == HDLA_FP32 && d->gk_dtype != HDLA_FP32) return HDLA_ERR_DTYPE;
     if (d->cu_seqlens) { if (d->B != 1) return HDLA_ERR_SEQ; }
     else if (d->N != d->B) return HDLA_ERR_SEQ;
+    if (d->route < HDLA_ROUTE_AUTO || d->route > HDLA_ROUTE_FUSED || d->segments < 0) return HDLA_ERR_ROUTE;
     return HDLA_OK;
+}
+
+// ---- the fused route (fused_impl.cuh) ----------------------------------------------------------------------------
+constexpr int FUSED_MAX_SEGMENTS = 8;        // the segments are chained serially by every workgroup that needs them
+constexpr int FUSED_MIN_SEGMENT_CHUNKS = 8;  // a segment pays for its transition matrix: not worth it for a few chunks
+constexpr int FUSED_TARGET_WORKGROUPS = 256; // one workgroup per compute unit
+
+// the shapes the fused kernels are built for
+bool fused_shape(const hdla_dims* d) { return d->in_dtype == HDLA_BF16 && d->K == 64 && d->V == 64; }
+// whether the plain entry points take the fused route for these dimensions; HDLA_ROUTE_FUSED on another shape is an error
+int pick_route(const hdla_dims* d, bool& fused) {
+    fused = d->route != HDLA_ROUTE_CLASSIC && fused_shape(d);
+    if (d->route == HDLA_ROUTE_FUSED && !fused) return HDLA_ERR_ROUTE;
+    return HDLA_OK;
+}
+// time segments per sequence: as many as give every compute unit a workgroup, within the limits above
+int fused_segments(const hdla_dims* d) {
+    if (d->segments > 0) return d->segments < FUSED_MAX_SEGMENTS ? d->segments : FUSED_MAX_SEGMENTS;
+    const long long lanes = (long long)d->N * d->H;
+    const long long chunks_per_seq = ((d->T + CHUNK - 1) / CHUNK) / (d->cu_seqlens ? d->N : 1);
+    int nseg = 1;
+    while (nseg * 2 <= FUSED_MAX_SEGMENTS && lanes * nseg * 2 <= FUSED_TARGET_WORKGROUPS &&
+           chunks_per_seq / (nseg * 2) >= FUSED_MIN_SEGMENT_CHUNKS) nseg *= 2;
+    return nseg;
+}
+
+struct FusedLayout {
+    size_t OL, GW, SLOC, MSEG, RSEG, SIN, ERR;                 // fused kernels' own
+    size_t HC, DHC, DVN, TM, UT, W, STRONG;                    // what chunk_grad reads (backward pass)
+    size_t CHUNK_OFF, CHUNK_SEQ;
+    size_t total;
+    int nch, nseg;
+};
+int make_fused_layout(const hdla_dims* d, int pass, FusedLayout& L) {
+    const int rc = check_dims(d);
+    if (rc) return rc;
+    if (d->N > 65535) return HDLA_ERR_SHAPE;
+    const int NT = (d->T + CHUNK - 1) / CHUNK;
+    const long long nch64 = d->cu_seqlens ? (long long)NT + d->N : (long long)d->B * NT;
+    if (nch64 * d->H > 0x7fff0000LL) return HDLA_ERR_SHAPE;
+    L = FusedLayout{};
+    L.nch = (int)nch64;
+    L.nseg = fused_segments(d);
+    const size_t es = 2, K = d->K, V = d->V;
+    const size_t chw = (size_t)d->H * (size_t)L.nch, recs = (size_t)d->N * d->H * L.nseg;
+    size_t off = 0;
+    auto take = [&](size_t bytes) { const size_t o = off; off += up256(bytes); return o; };
+    L.ERR = take(256);
+    L.SLOC = take(recs * K * V * 4);
+    L.MSEG = take(recs * K * K * 4);
+    if (pass == HDLA_PASS_FWD) {
+        L.OL = take(chw * 16 * V * 4);
+        L.GW = take(chw * 16 * K * es);
+    } else {
+        L.RSEG = take(recs * K * V * 4);
+        L.SIN = take(recs * K * V * 4);
+        L.HC = take(chw * K * V * es);
+        L.DHC = take(chw * K * V * es);
+        L.DVN = take(chw * 2 * 16 * V * es);
+        L.TM = take(chw * 1024 * es);
+        L.UT = take(chw * 2 * V * 16 * es);
+        L.W = take(chw * 2 * K * 16 * es);
+        L.STRONG = take(chw * 4);
+    }
+    if (d->cu_seqlens) {
+        L.CHUNK_OFF = take((size_t)(2 * d->N + 1) * 4);
+        L.CHUNK_SEQ = take((size_t)(L.nch > 0 ? L.nch : 1) * 4);
+    }
+    L.total = off;
+    return HDLA_OK;
+}
+size_t fused_boundary_bytes(const hdla_dims* d) {
+    const int nseg = fused_segments(d);
+    return nseg > 1 ? (size_t)d->N * d->H * nseg * d->K * d->V * 4 : 0;
 }
 
 // pass: HDLA_PASS_FWD, _BWD, _FWD_KEEP (a forward pass that leaves what the backward pass needs of it), _BWD_KEPT (the
@@ -181,6 +257,86 @@ int run_chunk(const hdla_dims* d, int pass, const void* q, const void* k, const 
     return HDLA_OK;
 }
 
+// The fused route's launch sequences.  Forward: fused kernel (+ fixup kernel when there are several segments); it
+// leaves the states entering the segments in `boundary` when given.  Backward: (without `boundary`: summary pass +
+// chaining, to re-derive those states) checkpoint kernel, reverse kernel, chunk_grad.
+int run_fused(const hdla_dims* d, bool fwd, const void* q, const void* k, const void* v, const void* a_, const void* b,
+              const void* beta, const void* gk, const float* h0, void* o, float* ht, const void* d_o, const float* dht,
+              void* dq, void* dk, void* dv, void* da, void* db, void* dbeta, void* dgk, float* dh0, void* boundary,
+              size_t boundary_bytes, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    typedef bf16 T;
+    FusedLayout L;
+    const int rc = make_fused_layout(d, fwd ? HDLA_PASS_FWD : HDLA_PASS_BWD, L);
+    if (rc) return rc;
+    if (bad_ws(workspace, workspace_bytes, L.total)) return HDLA_ERR_WORKSPACE;
+    if (boundary && (L.nseg > 1) && (boundary_bytes < fused_boundary_bytes(d) || (reinterpret_cast<uintptr_t>(boundary) & 15)))
+        return HDLA_ERR_WORKSPACE;
+    char* base = static_cast<char*>(workspace);
+    FusedArgs<T> f{};
+    ChunkArgs<T>& a = f.c;
+    a.q = static_cast<const T*>(q); a.k = static_cast<const T*>(k); a.v = static_cast<const T*>(v);
+    a.a = static_cast<const T*>(a_); a.b = static_cast<const T*>(b);
+    a.gk = gk; a.gk_f32 = d->gk_dtype == HDLA_FP32;
+    a.H = d->H; a.scale = d->scale;
+    a.h0 = h0; a.ht = fwd ? ht : nullptr; a.o = static_cast<T*>(o);
+    a.dout = static_cast<const T*>(d_o); a.dht = dht; a.dh0 = dh0;
+    a.dq = static_cast<T*>(dq); a.dk = static_cast<T*>(dk); a.dv = static_cast<T*>(dv);
+    a.da = static_cast<T*>(da); a.db = static_cast<T*>(db); a.dgk = dgk;
+    a.beta = static_cast<const T*>(beta); a.dbeta = static_cast<T*>(dbeta);
+    a.ws.HC = reinterpret_cast<T*>(base + L.HC); a.ws.DHC = reinterpret_cast<T*>(base + L.DHC);
+    a.ws.DVN = reinterpret_cast<T*>(base + L.DVN); a.ws.TM = reinterpret_cast<T*>(base + L.TM);
+    a.ws.UT = reinterpret_cast<T*>(base + L.UT); a.ws.W = reinterpret_cast<T*>(base + L.W);
+    a.ws.STRONG = reinterpret_cast<int32_t*>(base + L.STRONG);
+    a.ws.sa_stride = 2 * d->K * 16 * 2;                            // chunk_grad's view of w: [2][K/16] tiles per slot
+    a.st.cu = d->cu_seqlens;
+    a.st.chunk_off = d->cu_seqlens ? reinterpret_cast<const int32_t*>(base + L.CHUNK_OFF) : nullptr;
+    a.st.chunk_seq = d->cu_seqlens ? reinterpret_cast<const int32_t*>(base + L.CHUNK_SEQ) : nullptr;
+    a.st.order = d->cu_seqlens ? a.st.chunk_off + d->N + 1 : nullptr;
+    a.st.T = d->T; a.st.NT = (d->T + CHUNK - 1) / CHUNK; a.st.N = d->N; a.st.nch = L.nch;
+    f.nseg = L.nseg;
+    f.sloc = reinterpret_cast<float*>(base + L.SLOC); f.mseg = reinterpret_cast<float*>(base + L.MSEG);
+    f.rseg = reinterpret_cast<float*>(base + L.RSEG);
+    f.err = reinterpret_cast<int*>(base + L.ERR);
+    hipError_t e;
+    if (d->cu_seqlens) {
+        e = launch_chunk_table(d->cu_seqlens, d->N, d->T, L.nch, reinterpret_cast<int32_t*>(base + L.CHUNK_OFF),
+                               reinterpret_cast<int32_t*>(base + L.CHUNK_SEQ), stream);
+        if (e != hipSuccess) return (int)e;
+    }
+    if (fwd) {
+        f.ol = reinterpret_cast<float*>(base + L.OL); f.gw = reinterpret_cast<T*>(base + L.GW);
+        f.sin_out = static_cast<float*>(boundary);
+        e = launch_fused<T>(f, d->K, d->V, FUSED_FWD, stream);
+        if (e != hipSuccess) return (int)e;
+        if (L.nseg > 1) {
+            e = launch_fixup<T>(f, d->K, d->V, stream);
+            if (e != hipSuccess) return (int)e;
+        }
+        return HDLA_OK;
+    }
+    if (L.nseg > 1 && !boundary) {
+        // inputs only: one pass for the segment records, chained into the states entering the segments
+        f.sin_out = reinterpret_cast<float*>(base + L.SIN);
+        f.gw = nullptr;
+        e = launch_fused<T>(f, d->K, d->V, FUSED_SUM, stream);
+        if (e != hipSuccess) return (int)e;
+        e = launch_fixup<T>(f, d->K, d->V, stream);
+        if (e != hipSuccess) return (int)e;
+        f.sin = f.sin_out;
+    } else {
+        f.sin = static_cast<const float*>(boundary);
+    }
+    e = launch_fused<T>(f, d->K, d->V, FUSED_CKPT, stream);
+    if (e != hipSuccess) return (int)e;
+    e = launch_fused<T>(f, d->K, d->V, FUSED_REV, stream);
+    if (e != hipSuccess) return (int)e;
+    if (L.nch > 0) {
+        e = launch_chunk_grad<T>(a, d->K, d->V, stream);
+        if (e != hipSuccess) return (int)e;
+    }
+    return HDLA_OK;
+}
+
 }  // namespace
 
 // ---- scratch memory of the entry point that allocates nothing ------------------------------------------------
@@ -221,6 +377,7 @@ const char* hdla_strerror(int code) {
         case HDLA_ERR_WORKSPACE: return "workspace is NULL, not 256-byte aligned, or smaller than hdla_workspace_bytes()";
         case HDLA_ERR_ALIGN: return "tensor pointers must be 16-byte aligned";
         case HDLA_ERR_SEQ: return "cu_seqlens needs B == 1; without it N must equal B";
+        case HDLA_ERR_ROUTE: return "route must be HDLA_ROUTE_AUTO, _CLASSIC or _FUSED (the fused route: bf16 inputs, K = V = 64) and segments >= 0";
         case HDLA_ERR_STATIC_LIMIT: return "the call needs more scratch memory than the built-in HDLA_STATIC_WORKSPACE_BYTES; use hdla_chunk_fwd with a caller-owned workspace";
         default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error code";
     }
@@ -230,8 +387,21 @@ size_t hdla_workspace_bytes(const hdla_dims* dims, int pass) {
     WsLayout L;
     int nch;
     if (pass < HDLA_PASS_FWD || pass > HDLA_PASS_BWD_KEPT) return 0;
+    if (check_dims(dims)) return 0;
+    bool fused;
+    if (pick_route(dims, fused)) return 0;
+    if (fused && (pass == HDLA_PASS_FWD || pass == HDLA_PASS_BWD)) {
+        FusedLayout F;
+        return make_fused_layout(dims, pass, F) ? 0 : F.total;
+    }
     if (make_layout(dims, pass, L, nch)) return 0;
     return L.total;
+}
+
+size_t hdla_boundary_bytes(const hdla_dims* dims) {
+    bool fused;
+    if (check_dims(dims) || pick_route(dims, fused) || !fused) return 0;
+    return fused_boundary_bytes(dims);
 }
 
 int hdla_workspace_layout(const hdla_dims* dims, int pass, hdla_ws_layout* out) {
@@ -239,7 +409,25 @@ int hdla_workspace_layout(const hdla_dims* dims, int pass, hdla_ws_layout* out) 
     if (pass < HDLA_PASS_FWD || pass > HDLA_PASS_BWD_KEPT) return HDLA_ERR_SHAPE;
     WsLayout L;
     int nch;
-    const int rc = make_layout(dims, pass, L, nch);
+    int rc = check_dims(dims);
+    if (rc) return rc;
+    bool fused;
+    rc = pick_route(dims, fused);
+    if (rc) return rc;
+    if (fused && (pass == HDLA_PASS_FWD || pass == HDLA_PASS_BWD)) {
+        FusedLayout F;
+        rc = make_fused_layout(dims, pass, F);
+        if (rc) return rc;
+        *out = hdla_ws_layout{};
+        out->nch = F.nch;
+        out->UT = F.UT; out->TM = F.TM; out->HC = F.HC; out->DHC = F.DHC; out->DVN = F.DVN; out->STRONG = F.STRONG;
+        out->W = F.W; out->SA_STRIDE = pass == HDLA_PASS_BWD ? 2 * dims->K * 16 * 2 : 0;
+        out->CHUNK_OFF = F.CHUNK_OFF; out->CHUNK_SEQ = F.CHUNK_SEQ;
+        out->total = F.total;
+        out->ERR = F.ERR;
+        return HDLA_OK;
+    }
+    rc = make_layout(dims, pass, L, nch);
     if (rc) return rc;
     out->nch = nch;
     out->W = L.W; out->UT = L.UT; out->KGT = L.KGT; out->BGT = L.BGT; out->VTT = L.VTT; out->EGL = L.EGL;
@@ -249,23 +437,65 @@ int hdla_workspace_layout(const hdla_dims* dims, int pass, hdla_ws_layout* out) 
     out->HC = L.HC; out->DHC = L.DHC; out->DVN = L.DVN; out->STRONG = L.STRONG;
     out->CHUNK_OFF = L.CHUNK_OFF; out->CHUNK_SEQ = L.CHUNK_SEQ;
     out->total = L.total;
+    out->ERR = -1;
     return HDLA_OK;
+}
+
+// forward pass of either form (a, b given, or beta) on the route the dimensions select
+static int chunk_fwd_any(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a, const void* b,
+                         const void* beta, const void* gk, const float* h0, void* o, float* ht, void* boundary,
+                         size_t boundary_bytes, void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_dims(dims);
+    if (rc) return rc;
+    if (dims->T > 0 && (!q || !k || !v || !gk || !o || (!beta && (!a || !b)))) return HDLA_ERR_NULL;
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(a) || !aligned16(b) || !aligned16(gk) ||
+        !aligned16(o) || !aligned16(h0) || !aligned16(ht)) return HDLA_ERR_ALIGN;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (beta) { a = nullptr; b = nullptr; }
+    bool fused;
+    rc = pick_route(dims, fused);
+    if (rc) return rc;
+    if (fused)
+        return run_fused(dims, true, q, k, v, a, b, beta, gk, h0, o, ht, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
+                         nullptr, nullptr, nullptr, nullptr, boundary, boundary_bytes, workspace, workspace_bytes, s);
+    if (dims->in_dtype == HDLA_BF16)
+        return run_chunk<bf16>(dims, 0, q, k, v, a, b, gk, h0, o, ht, nullptr, nullptr, nullptr, nullptr, nullptr,
+                               nullptr, nullptr, nullptr, nullptr, workspace, workspace_bytes, s, HDLA_STAGE_ALL, beta, nullptr);
+    return run_chunk<float>(dims, 0, q, k, v, a, b, gk, h0, o, ht, nullptr, nullptr, nullptr, nullptr, nullptr,
+                            nullptr, nullptr, nullptr, nullptr, workspace, workspace_bytes, s, HDLA_STAGE_ALL, beta, nullptr);
+}
+
+static int chunk_bwd_any(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a, const void* b,
+                         const void* beta, const void* gk, const float* h0, const void* d_o, const float* dht, void* dq,
+                         void* dk, void* dv, void* da, void* db, void* dbeta, void* dgk, float* dh0, const void* boundary,
+                         size_t boundary_bytes, void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_dims(dims);
+    if (rc) return rc;
+    if (dims->T > 0 && (!q || !k || !v || !gk || !d_o || !dq || !dk || !dv || !dgk)) return HDLA_ERR_NULL;
+    if (dims->T > 0 && (beta ? !dbeta : (!a || !b || !da || !db))) return HDLA_ERR_NULL;
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(a) || !aligned16(b) || !aligned16(gk) ||
+        !aligned16(d_o) || !aligned16(dq) || !aligned16(dk) || !aligned16(dv) || !aligned16(da) || !aligned16(db) ||
+        !aligned16(dgk) || !aligned16(h0) || !aligned16(dht) || !aligned16(dh0)) return HDLA_ERR_ALIGN;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (beta) { a = nullptr; b = nullptr; da = nullptr; db = nullptr; }
+    bool fused;
+    rc = pick_route(dims, fused);
+    if (rc) return rc;
+    if (fused)
+        return run_fused(dims, false, q, k, v, a, b, beta, gk, h0, nullptr, nullptr, d_o, dht, dq, dk, dv, da, db, dbeta, dgk,
+                         dh0, const_cast<void*>(boundary), boundary_bytes, workspace, workspace_bytes, s);
+    if (dims->in_dtype == HDLA_BF16)
+        return run_chunk<bf16>(dims, 1, q, k, v, a, b, gk, h0, nullptr, nullptr, d_o, dht, dq, dk, dv, da, db, dgk,
+                               dh0, workspace, workspace_bytes, s, HDLA_STAGE_ALL, beta, dbeta);
+    return run_chunk<float>(dims, 1, q, k, v, a, b, gk, h0, nullptr, nullptr, d_o, dht, dq, dk, dv, da, db, dgk,
+                            dh0, workspace, workspace_bytes, s, HDLA_STAGE_ALL, beta, dbeta);
 }
 
 int hdla_chunk_fwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
                    const void* b, const void* gk, const float* h0, void* o, float* ht,
                    void* workspace, size_t workspace_bytes, void* stream) {
-    const int rc = check_dims(dims);
-    if (rc) return rc;
-    if (dims->T > 0 && (!q || !k || !v || !a || !b || !gk || !o)) return HDLA_ERR_NULL;
-    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(a) || !aligned16(b) || !aligned16(gk) ||
-        !aligned16(o) || !aligned16(h0) || !aligned16(ht)) return HDLA_ERR_ALIGN;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dims->in_dtype == HDLA_BF16)
-        return run_chunk<bf16>(dims, 0, q, k, v, a, b, gk, h0, o, ht, nullptr, nullptr, nullptr, nullptr, nullptr,
-                               nullptr, nullptr, nullptr, nullptr, workspace, workspace_bytes, s);
-    return run_chunk<float>(dims, 0, q, k, v, a, b, gk, h0, o, ht, nullptr, nullptr, nullptr, nullptr, nullptr,
-                            nullptr, nullptr, nullptr, nullptr, workspace, workspace_bytes, s);
+    if (dims && dims->T > 0 && (!a || !b)) return HDLA_ERR_NULL;
+    return chunk_fwd_any(dims, q, k, v, a, b, nullptr, gk, h0, o, ht, nullptr, 0, workspace, workspace_bytes, stream);
 }
 
 int hdla_chunk_fwd_static(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,
@@ -285,56 +515,38 @@ int hdla_chunk_bwd(const hdla_dims* dims, const void* q, const void* k, const vo
                    const void* b, const void* gk, const float* h0, const void* d_o, const float* dht,
                    void* dq, void* dk, void* dv, void* da, void* db, void* dgk, float* dh0,
                    void* workspace, size_t workspace_bytes, void* stream) {
-    const int rc = check_dims(dims);
-    if (rc) return rc;
-    if (dims->T > 0 && (!q || !k || !v || !a || !b || !gk || !d_o || !dq || !dk || !dv || !da || !db || !dgk))
-        return HDLA_ERR_NULL;
-    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(a) || !aligned16(b) || !aligned16(gk) ||
-        !aligned16(d_o) || !aligned16(dq) || !aligned16(dk) || !aligned16(dv) || !aligned16(da) || !aligned16(db) ||
-        !aligned16(dgk) || !aligned16(h0) || !aligned16(dht) || !aligned16(dh0)) return HDLA_ERR_ALIGN;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dims->in_dtype == HDLA_BF16)
-        return run_chunk<bf16>(dims, 1, q, k, v, a, b, gk, h0, nullptr, nullptr, d_o, dht, dq, dk, dv, da, db, dgk,
-                               dh0, workspace, workspace_bytes, s);
-    return run_chunk<float>(dims, 1, q, k, v, a, b, gk, h0, nullptr, nullptr, d_o, dht, dq, dk, dv, da, db, dgk,
-                            dh0, workspace, workspace_bytes, s);
+    return chunk_bwd_any(dims, q, k, v, a, b, nullptr, gk, h0, d_o, dht, dq, dk, dv, da, db, nullptr, dgk, dh0, nullptr, 0,
+                         workspace, workspace_bytes, stream);
 }
 
 int hdla_param_chunk_fwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* beta,
                          const void* gk, const float* h0, void* o, float* ht,
                          void* workspace, size_t workspace_bytes, void* stream) {
-    const int rc = check_dims(dims);
-    if (rc) return rc;
-    if (!beta || (dims->T > 0 && (!q || !k || !v || !gk || !o))) return HDLA_ERR_NULL;
-    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(gk) || !aligned16(o) || !aligned16(h0) ||
-        !aligned16(ht)) return HDLA_ERR_ALIGN;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dims->in_dtype == HDLA_BF16)
-        return run_chunk<bf16>(dims, 0, q, k, v, nullptr, nullptr, gk, h0, o, ht, nullptr, nullptr, nullptr, nullptr,
-                               nullptr, nullptr, nullptr, nullptr, nullptr, workspace, workspace_bytes, s,
-                               HDLA_STAGE_ALL, beta, nullptr);
-    return run_chunk<float>(dims, 0, q, k, v, nullptr, nullptr, gk, h0, o, ht, nullptr, nullptr, nullptr, nullptr,
-                            nullptr, nullptr, nullptr, nullptr, nullptr, workspace, workspace_bytes, s,
-                            HDLA_STAGE_ALL, beta, nullptr);
+    if (!beta) return HDLA_ERR_NULL;
+    return chunk_fwd_any(dims, q, k, v, nullptr, nullptr, beta, gk, h0, o, ht, nullptr, 0, workspace, workspace_bytes, stream);
 }
 
 int hdla_param_chunk_bwd(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* beta,
                          const void* gk, const float* h0, const void* d_o, const float* dht,
                          void* dq, void* dk, void* dv, void* dbeta, void* dgk, float* dh0,
                          void* workspace, size_t workspace_bytes, void* stream) {
-    const int rc = check_dims(dims);
-    if (rc) return rc;
-    if (!beta || (dims->T > 0 && (!q || !k || !v || !gk || !d_o || !dq || !dk || !dv || !dbeta || !dgk)))
-        return HDLA_ERR_NULL;
-    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(gk) || !aligned16(d_o) || !aligned16(dq) ||
-        !aligned16(dk) || !aligned16(dv) || !aligned16(dgk) || !aligned16(h0) || !aligned16(dht) || !aligned16(dh0))
-        return HDLA_ERR_ALIGN;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    if (dims->in_dtype == HDLA_BF16)
-        return run_chunk<bf16>(dims, 1, q, k, v, nullptr, nullptr, gk, h0, nullptr, nullptr, d_o, dht, dq, dk, dv,
-                               nullptr, nullptr, dgk, dh0, workspace, workspace_bytes, s, HDLA_STAGE_ALL, beta, dbeta);
-    return run_chunk<float>(dims, 1, q, k, v, nullptr, nullptr, gk, h0, nullptr, nullptr, d_o, dht, dq, dk, dv,
-                            nullptr, nullptr, dgk, dh0, workspace, workspace_bytes, s, HDLA_STAGE_ALL, beta, dbeta);
+    if (!beta) return HDLA_ERR_NULL;
+    return chunk_bwd_any(dims, q, k, v, nullptr, nullptr, beta, gk, h0, d_o, dht, dq, dk, dv, nullptr, nullptr, dbeta, dgk,
+                         dh0, nullptr, 0, workspace, workspace_bytes, stream);
+}
+
+int hdla_chunk_fwd_b(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a, const void* b,
+                     const void* beta, const void* gk, const float* h0, void* o, float* ht, void* boundary,
+                     size_t boundary_bytes, void* workspace, size_t workspace_bytes, void* stream) {
+    return chunk_fwd_any(dims, q, k, v, a, b, beta, gk, h0, o, ht, boundary, boundary_bytes, workspace, workspace_bytes, stream);
+}
+
+int hdla_chunk_bwd_b(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a, const void* b,
+                     const void* beta, const void* gk, const float* h0, const void* d_o, const float* dht, void* dq,
+                     void* dk, void* dv, void* da, void* db, void* dbeta, void* dgk, float* dh0, const void* boundary,
+                     size_t boundary_bytes, void* workspace, size_t workspace_bytes, void* stream) {
+    return chunk_bwd_any(dims, q, k, v, a, b, beta, gk, h0, d_o, dht, dq, dk, dv, da, db, dbeta, dgk, dh0, boundary,
+                         boundary_bytes, workspace, workspace_bytes, stream);
 }
 
 int hdla_chunk_fwd_keep(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a,

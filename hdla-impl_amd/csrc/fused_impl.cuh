@@ -1,0 +1,995 @@
+// Fused chunk kernels: the per-chunk preparation (cumulative decays, score tiles, (I - A_ab)^-1, w, u, gated copies:
+// HRDPLR/fwd_triton.py:22-790 and fla's chunk_rwkv6_fwd_cumsum) and the inter-chunk state scan that consumes it
+// (HRDPLR/fwd_triton.py:808-1095, HRDPLR/bwd_triton.py:127-222) in ONE kernel, so that what the preparation produces
+// for the scan -- 14 to 20 KB per (16-token chunk, head) -- goes through LDS and never through HBM.
+//
+// Work division.  A workgroup owns one (sequence, head, time segment): the chunks of a sequence are cut into `nseg`
+// consecutive segments so that few (sequence, head) pairs still fill the device.  It has
+//   * FNP = 4 producer waves.  Producer p prepares the chunks p, p+4, ... of the segment, each entirely by itself (one
+//     wave holds all 64 channels), and leaves the operands in LDS slot p;
+//   * V/16 consumer waves.  Consumer j owns column block j of the fp32 state for the whole segment, in registers, and
+//     walks the chunks in order, exactly as the stand-alone scan kernels do.
+// A segment other than the first does not know the state that enters it.  The state leaving a chunk is affine in the
+// state entering it, so such a segment runs from zero and, beside it, carries the K x K transition matrix M (the same
+// update applied to K more columns that start from the identity: consumer j also owns column block j of M).  What the
+// chunk's output gains per unit of entering state, G = (qg + A_qb w) M (16 x K), comes out of the same products.
+//   forward pass:   o_local and G go to the workspace; fixup_kernel chains the segments' (M, S_local) into the true
+//                   entering states and adds G S_in.
+//   backward pass:  the entering states are known (kept by the forward pass, or re-derived by a summary-only pass), so
+//                   the state checkpoints are exact; M and R = sum_t G_t^T do_t give the gradient entering each
+//                   segment from the right, d S_in(s) = M_s^T d S_in(s+1) + R_s, which the reverse kernel's consumers
+//                   chain themselves before they start.
+//
+// Synchronisation.  Producers and consumers run at their own pace; a slot is handed over through two counters in LDS
+// that only ever grow: ready[p] (chunks producer p has completed) and consumed[p] (consumer-steps finished on slot p).
+// Waiting is polling with s_sleep; every wait is bounded (FUSED_SPIN_LIMIT polls), and a wave that runs into the bound
+// raises an abort flag that ends every other wave's waits as well and is reported through FusedArgs::err, so the grid
+// always drains.  There are no workgroup barriers after the first.
+#pragma once
+#include "hdla_common.cuh"
+#include "fused_shapes.h"
+
+namespace hdla {
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int FNP = 4;                    // producer waves = LDS slots
+constexpr int FLDP = 36;                  // padded row length of the 32 x 32 matrices of the triangular solve
+constexpr int FUSED_SPIN_LIMIT = 1 << 20; // polls of ~256 cycles: a tenth of a second, four orders above any real wait
+// What a wave that gave up writes to FusedArgs::err (+1 producer, +2 forward consumer, +3 reverse consumer).  The word is
+// never cleared (that would take a launch of its own): it is a diagnostic that reads as this pattern only after an
+// abort, or by a one-in-a-billion coincidence with what the caller's memory held before.
+constexpr int FUSED_ABORTED = 0x48444c00;
+
+// chunk range [s0, s1) of time segment `seg` of sequence n
+__device__ __forceinline__ void seg_range(const SeqTab& st, int n, int nseg, int seg, int& s0, int& s1) {
+    int c0, c1;
+    seq_chunks(st, n, c0, c1);
+    const int len = (c1 - c0 + nseg - 1) / nseg;
+    s0 = min(c0 + seg * len, c1);
+    s1 = min(s0 + len, c1);
+}
+
+// LDS of a fused workgroup (byte offsets): per producer one slot = [operands | outbox | solver scratch], then the flags
+template <typename T, int K, int V, int MODE> struct FusedLds {
+    static constexpr int ES = sizeof(T), TB = TILE * ES, KT = K / 16, VT = V / 16;
+    static constexpr bool REV = MODE == FUSED_REV;
+    static constexpr BlkF BF = blk_fwd(K, ES, true);
+    static constexpr SlotB SB = slot_bwd(K, ES);
+    // forward direction: the forward-scan block, then u^T (VT tile pairs), v^T (VT tiles), and in checkpoint mode do^T
+    // (VT tiles) and the inverse for chunk_grad
+    static constexpr int UT = BF.SIZE, VTT = UT + 2 * VT * TB, DOT_F = VTT + VT * TB;
+    // reverse direction: the reverse-scan slot, then do^T
+    static constexpr int DOT = REV ? SB.SIZE : DOT_F;
+    static constexpr int TMB = DOT_F + VT * TB;          // checkpoint mode: (I - A_ab)^-1 as chunk_grad reads it (2 tile pairs)
+    static constexpr int OPER = REV ? SB.SIZE + VT * TB : (MODE == FUSED_CKPT ? TMB + 4 * TB : DOT_F);
+    // outbox of the forward pass: 16 rows of o (fp32 in segments > 0, element type in segment 0) and 16 rows of G
+    static constexpr int OROW = V * 4 + 16, GROW = K * ES + 16;
+    static constexpr int OBOX = OPER, GBOX = OBOX + (MODE == FUSED_FWD ? CH * OROW : 0);
+    static constexpr int SOLVE = GBOX + (MODE == FUSED_FWD ? CH * GROW : 0);
+    static constexpr int SLOT = SOLVE + 2 * 32 * FLDP * 4;
+    static constexpr int FLAGS = FNP * SLOT;        // int ready[4], consumed[4], abort
+    static constexpr int BYTES = FLAGS + 64;
+};
+
+// ---- hand-over counters ------------------------------------------------------------------------------------------
+__device__ __forceinline__ bool wait_ge(int* flag, int want, int* abort_flag) {
+    int spins = 0;
+    while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < want) {
+        if (__hip_atomic_load(abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != 0 || ++spins > FUSED_SPIN_LIMIT) {
+            __hip_atomic_store(abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            return false;
+        }
+        __builtin_amdgcn_s_sleep(4);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    return true;
+}
+// all LDS accesses of the wave so far are complete before the counter moves
+__device__ __forceinline__ void signal_set(int* flag, int value) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    if (lane_id() == 0) __hip_atomic_store(flag, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ void signal_add(int* flag) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    if (lane_id() == 0) __hip_atomic_fetch_add(flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
+// the log-decay of four channels as it sits in memory (element type or fp32), converted and masked only where it is used
+template <typename T, bool GKF32> struct GkRaw {
+    typedef Frag<T> type;
+    static __device__ __forceinline__ type load(const char* p) { return ld_frag(reinterpret_cast<const T*>(p)); }
+    static __device__ __forceinline__ f32x4 value(type x, bool ok) { return ok ? to_f32(x) : zero4(); }
+};
+template <typename T> struct GkRaw<T, true> {
+    typedef f32x4 type;
+    static __device__ __forceinline__ type load(const char* p) { return *reinterpret_cast<const f32x4*>(p); }
+    static __device__ __forceinline__ f32x4 value(type x, bool ok) { return ok ? x : zero4(); }
+};
+
+// ---- producer ----------------------------------------------------------------------------------------------------
+// Everything of a chunk that does not depend on the state, by one wave, into LDS slot `pw`.  The arithmetic is the
+// stand-alone prep kernel's, operation for operation (prep.hip), so both routes hand the scans the same bits.
+template <typename T, bool GKF32, int K, int V, int MODE, bool HD>
+__device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem, int n, int h, int seg, int s0, int s1, int pw) {
+    static_assert(K == 64 && sizeof(T) == 2, "one producer wave holds all channels of a chunk: K = 64, 2-byte elements");
+    typedef FusedLds<T, K, V, MODE> L;
+    constexpr bool REV = MODE == FUSED_REV, CKPT = MODE == FUSED_CKPT, FWD = MODE == FUSED_FWD;
+    constexpr int KT = K / 16, VT = V / 16, KT2 = KT / 2;
+    constexpr BlkF BF = L::BF;
+    constexpr SlotB SB = L::SB;
+    const ChunkArgs<T>& p = a.c;
+    char* const slot = smem + pw * L::SLOT;
+    float* const sN = reinterpret_cast<float*>(slot + L::SOLVE);
+    float* const sT = sN + 32 * FLDP;
+    int* const flags = reinterpret_cast<int*>(smem + L::FLAGS);
+    const int l = lane_id(), g = l >> 4, c = l & 15;
+    const int H = p.H;
+    const float scale = p.scale;
+    const int nst = s1 - s0;
+    int64_t bos, eos;
+    seq_bounds(p.st, n, bos, eos);
+    int c0, c1;
+    seq_chunks(p.st, n, c0, c1);
+    const Frag<T> ident = ident_frag<T>();
+
+    // rows of the previous chunk's results, left in the outbox by the consumers, out to global memory (forward pass)
+    auto copy_out = [&](int cid) __attribute__((always_inline)) {
+        if constexpr (FWD) {
+            // the lane's offsets below are formed afresh in every call: hoisted out of the chunk loop they would be held
+            // in registers through all of it
+            int l = lane_id();
+            asm volatile("" : "+v"(l));
+            const int64_t tok0 = bos + (int64_t)(cid - c0) * CH;
+            const int len = (int)min((int64_t)CH, eos - tok0);
+            const int64_t chw = (int64_t)h * p.st.nch + cid;
+            if (seg == 0) {
+                constexpr int LPR = V * (int)sizeof(T) / 16, RPI = 64 / LPR;
+#pragma unroll
+                for (int r0 = 0; r0 < CH; r0 += RPI) {
+                    const int r = r0 + l / LPR, e = (l % LPR) * 16;
+                    const i32x4 x = *reinterpret_cast<const i32x4*>(slot + L::OBOX + r * L::OROW + e);
+                    if (r < len) *reinterpret_cast<i32x4*>(reinterpret_cast<char*>(p.o + ((tok0 + r) * H + h) * V) + e) = x;
+                }
+            } else {
+                constexpr int LPO = V * 4 / 16, RPO = 64 / LPO;
+                char* ol = reinterpret_cast<char*>(a.ol + chw * (CH * V));
+#pragma unroll
+                for (int r0 = 0; r0 < CH; r0 += RPO) {
+                    const int r = r0 + l / LPO, e = (l % LPO) * 16;
+                    *reinterpret_cast<i32x4*>(ol + r * (V * 4) + e) = *reinterpret_cast<const i32x4*>(slot + L::OBOX + r * L::OROW + e);
+                }
+                constexpr int LPG = K * (int)sizeof(T) / 16, RPG = 64 / LPG;
+                char* gw = reinterpret_cast<char*>(a.gw + chw * (CH * K));
+#pragma unroll
+                for (int r0 = 0; r0 < CH; r0 += RPG) {
+                    const int r = r0 + l / LPG, e = (l % LPG) * 16;
+                    *reinterpret_cast<i32x4*>(gw + r * (K * (int)sizeof(T)) + e) = *reinterpret_cast<const i32x4*>(slot + L::GBOX + r * L::GROW + e);
+                }
+            }
+        }
+    };
+
+    // The chunk's inputs as loaded, four elements a lane (lane (g,c): token c, channels 16kt + 4g ..): requested one
+    // chunk of this wave ahead (as soon as the registers are free), so that the round trip to HBM runs behind the rest
+    // of the previous chunk.  Nothing is done to them at the load (a select or a conversion would wait for the data).
+    Frag<T> nq[KT], nk[KT], na[2][KT], nb[2][KT], nv[VT], ndo[VT];
+    typename GkRaw<T, GKF32>::type ng[KT];
+    T nbeta;
+    auto request = [&](int t) __attribute__((always_inline)) {
+        const int cid = REV ? s1 - 1 - t : s0 + t;
+        const int64_t tok0 = bos + (int64_t)(cid - c0) * CH;
+        const int len = (int)min((int64_t)CH, eos - tok0);
+        // uniform base of the chunk's first row + a 32-bit byte offset per lane, formed afresh in every call (see copy_out);
+        // rows past the end alias the last valid row and are masked at use
+        int cc = c, gg = g;
+        asm volatile("" : "+v"(cc), "+v"(gg));
+        const uint32_t row = (uint32_t)min(cc, max(len, 1) - 1);
+        constexpr uint32_t ES = sizeof(T), GS = GKF32 ? 4 : 2;
+        const uint32_t qe = row * (uint32_t)(H * K) + 4 * gg, ae = row * (uint32_t)(RANK * H * K) + 4 * gg;
+        const uint32_t ve = row * (uint32_t)(H * V) + 4 * gg;
+        const int64_t qb = (tok0 * H + h) * K, ab = (tok0 * RANK * H + h) * K, vb = (tok0 * H + h) * V;
+        const char* gkp = reinterpret_cast<const char*>(p.gk) + qb * GS;
+        if (!REV) {
+#pragma unroll
+            for (int vt = 0; vt < VT; ++vt) nv[vt] = ld_frag(at(p.v + vb, (ve + 16 * vt) * ES));
+        }
+        if (REV || CKPT) {
+#pragma unroll
+            for (int vt = 0; vt < VT; ++vt) ndo[vt] = ld_frag(at(p.dout + vb, (ve + 16 * vt) * ES));
+        }
+        if (HD) nbeta = *at(p.beta + tok0 * H + h, row * (uint32_t)H * ES);
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            const uint32_t ko = 16 * kt;
+            ng[kt] = GkRaw<T, GKF32>::load(gkp + (qe + ko) * GS);
+            nq[kt] = ld_frag(at(p.q + qb, (qe + ko) * ES));
+            nk[kt] = ld_frag(at(p.k + qb, (qe + ko) * ES));
+            if (!HD) {
+                na[0][kt] = ld_frag(at(p.a + ab, (ae + ko) * ES));
+                na[1][kt] = ld_frag(at(p.a + ab, (ae + (uint32_t)(H * K) + ko) * ES));
+                nb[0][kt] = ld_frag(at(p.b + ab, (ae + ko) * ES));
+                nb[1][kt] = ld_frag(at(p.b + ab, (ae + (uint32_t)(H * K) + ko) * ES));
+            }
+        }
+    };
+    auto sel = [](Frag<T> f, bool ok) __attribute__((always_inline)) {
+        Frag<T> r;
+        r.v = ok ? f.v : zero_frag<T>().v;
+        return r;
+    };
+    if (pw < nst) request(pw);
+
+    int it = 0, prev_cid = -1;
+    for (int t = pw; t < nst; t += FNP, ++it) {
+        const int cid = REV ? s1 - 1 - t : s0 + t;
+        const int64_t tok0 = bos + (int64_t)(cid - c0) * CH;
+        const int len = (int)min((int64_t)CH, eos - tok0);
+        const int64_t chw = (int64_t)h * p.st.nch + cid;
+        const bool rowok = c < len;
+
+        // ---- phase A: cumulative decays and the score tiles (prep.hip, phase A) ------------------------------------
+        // (the cumulative decays of a channel tile are formed again wherever they are needed, from the log-decays as
+        // loaded, instead of being kept: the same values for fewer registers)
+        auto decays = [&](int kt, f32x4& gi, f32x4& ge) __attribute__((always_inline)) {
+            const f32x4 g4 = GkRaw<T, GKF32>::value(ng[kt], rowok);
+            gi = scan16_incl(g4);
+            ge = gi - g4;
+        };
+        float big = 0.f;                                  // see strong_decay()
+        f32x4 aqk = zero4(), aqb[2] = {zero4(), zero4()}, aak[2] = {zero4(), zero4()};
+        f32x4 aab[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
+        f32x4 aqbT[2] = {zero4(), zero4()};
+        Frag<T> rq[KT], rk[KT], ra[2][KT], rb[2][KT];
+        Frag<T> rv[VT], rdo[VT];
+        if (!REV) {
+#pragma unroll
+            for (int vt = 0; vt < VT; ++vt) rv[vt] = sel(nv[vt], rowok);
+        }
+        if (REV || CKPT) {
+#pragma unroll
+            for (int vt = 0; vt < VT; ++vt) rdo[vt] = sel(ndo[vt], rowok);
+        }
+        float beta_t = 0.f, s_t = 0.f;
+        if (HD) {
+            beta_t = rowok ? ld_elem(&nbeta) : 0.f;
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+                const f32x4 g4 = GkRaw<T, GKF32>::value(ng[kt], rowok);
+                const f32x4 k4 = to_f32(sel(nk[kt], rowok));
+                const f32x4 kf = k4 * k4 * exp4<T>(g4);
+                s_t += kf[0] + kf[1] + kf[2] + kf[3];
+            }
+            s_t += __shfl_xor(s_t, 16);
+            s_t += __shfl_xor(s_t, 32);
+        }
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            const f32x4 g4 = GkRaw<T, GKF32>::value(ng[kt], rowok);
+            rq[kt] = sel(nq[kt], rowok);
+            rk[kt] = sel(nk[kt], rowok);
+            if (HD) {
+                const f32x4 kk = to_f32(rk[kt]), f4 = exp4<T>(g4);
+                ra[0][kt] = to_frag<T>(kk * (-beta_t));
+                ra[1][kt] = to_frag<T>(kk * ((beta_t * s_t - f4) * beta_t));
+                rb[0][kt] = to_frag<T>(f4 * kk);
+                rb[1][kt] = rk[kt];
+            } else {
+                ra[0][kt] = sel(na[0][kt], rowok);
+                ra[1][kt] = sel(na[1][kt], rowok);
+                rb[0][kt] = sel(nb[0][kt], rowok);
+                rb[1][kt] = sel(nb[1][kt], rowok);
+            }
+            const f32x4 gi = scan16_incl(g4), ge = gi - g4;
+            const f32x4 m = bcast16<MID>(gi);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) big = fmaxf(big, fmaxf(fabsf(gi[i] - m[i]), fabsf(ge[i] - m[i])));
+            const f32x4 eq = exp4<T>(gi - m), ek = exp4<T>(m - gi), ea = exp4<T>(ge - m);
+            const f32x4 q4 = to_f32(rq[kt]), k4 = to_f32(rk[kt]);
+            const f32x4 a0 = to_f32(ra[0][kt]), a1 = to_f32(ra[1][kt]), b0 = to_f32(rb[0][kt]), b1 = to_f32(rb[1][kt]);
+            Split<T> qh, kh, ah[2], bh[2];
+            split(q4 * eq * scale, qh);
+            split(k4 * ek, kh);
+            split(a0 * ea, ah[0]);
+            split(a1 * ea, ah[1]);
+            split(b0 * ek, bh[0]);
+            split(b1 * ek, bh[1]);
+            if (FWD) aqk = mm3(qh, kh, aqk);
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                if (!REV) aqb[s] = mm3(qh, bh[s], aqb[s]);
+                if (!REV) aak[s] = mm3(ah[s], kh, aak[s]);
+                if (REV) aqbT[s] = mm3(bh[s], qh, aqbT[s]);
+#pragma unroll
+                for (int r = 0; r < 2; ++r) aab[r][s] = mm3(ah[r], bh[s], aab[r][s]);
+            }
+        }
+        const bool strong = __any(big > SAFE_RANGE) != 0;  // the same answer on every lane of the wave
+        if (CKPT && l == 0) p.ws.STRONG[chw] = strong;
+        if (strong) {
+            aqk = zero4();
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                aqb[s] = zero4(); aak[s] = zero4(); aqbT[s] = zero4(); aab[0][s] = zero4(); aab[1][s] = zero4();
+            }
+#pragma unroll 1
+            for (int ps = 0; ps < DecayPass::COUNT; ++ps) {
+                const DecayPass dp(ps, c);
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+                    f32x4 gi, ge, eq, ek, ea;
+                    decays(kt, gi, ge);
+                    dp.factors<T>(gi, ge, eq, ek, ea);
+                    pin(rk[kt]); pin(rq[kt]); pin(ra[0][kt]); pin(ra[1][kt]); pin(rb[0][kt]); pin(rb[1][kt]);
+                    Split<T> qh, kh, bh[2];
+                    split(to_f32(rk[kt]) * ek, kh);
+                    split(to_f32(rq[kt]) * eq * scale, qh);
+                    if (FWD) aqk = mm3(qh, kh, aqk);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        split(to_f32(rb[s][kt]) * ek, bh[s]);
+                        if (!REV) aqb[s] = mm3(qh, bh[s], aqb[s]);
+                        if (REV) aqbT[s] = mm3(bh[s], qh, aqbT[s]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+#pragma unroll
+                    for (int r = 0; r < 2; ++r) {
+                        Split<T> ah;
+                        split(to_f32(ra[r][kt]) * ea, ah);
+                        if (!REV) aak[r] = mm3(ah, kh, aak[r]);
+                        aab[r][0] = mm3(ah, bh[0], aab[r][0]);
+                        aab[r][1] = mm3(ah, bh[1], aab[r][1]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+        }
+        // causal masks: lane (g,c) reg i is entry (row c, inner 4g+i)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int j = 4 * g + i;
+            const bool le = j <= c, lt = j < c, tle = c <= j;
+            if (!le) { aqk[i] = 0.f; aqb[0][i] = 0.f; aqb[1][i] = 0.f; }
+            if (!lt) { aak[0][i] = 0.f; aak[1][i] = 0.f; aab[0][0][i] = 0.f; aab[0][1][i] = 0.f; aab[1][0][i] = 0.f; aab[1][1][i] = 0.f; }
+            if (!tle) { aqbT[0][i] = 0.f; aqbT[1][i] = 0.f; }
+        }
+        // the solver's scratch is this wave's own: nobody else reads it
+        // (the scheduling barriers stand where the stand-alone kernel has workgroup barriers: they keep the phases from
+        // being interleaved, which the register file has no room for)
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+                *reinterpret_cast<f32x4*>(&sN[(16 * r + c) * FLDP + 16 * s + 4 * g]) = aab[r][s];
+
+        // ---- the slot: wait until the consumers have left the chunk it held ---------------------------------------------
+        if (!wait_ge(&flags[4 + pw], VT * it, &flags[8])) { if (l == 0) *a.err = FUSED_ABORTED + 1; return; }
+        __builtin_amdgcn_sched_barrier(0);
+        // The rows the consumers left in the outbox for that chunk go out first (the consumers write the outbox again
+        // only after the signal at the end): these stores are then ahead of the next chunk's loads in the wave's
+        // in-order memory counter, not behind them.
+        if (it > 0) copy_out(prev_cid);
+        prev_cid = cid;
+        __builtin_amdgcn_sched_barrier(0);
+
+        // ---- everything that needs the inputs but not (I - A_ab)^-1: score tiles, gated copies, ag (prep.hip, phase C) --
+        if (!REV) {
+            if (FWD) st_tile(reinterpret_cast<T*>(slot + BF.AQK), to_frag<T>(aqk));
+            st_pair2(reinterpret_cast<T*>(slot + BF.AQB), to_frag<T>(aqb[0]), to_frag<T>(aqb[1]));
+        } else {
+            st_pair2(reinterpret_cast<T*>(slot + SB.AQBT), to_frag<T>(aqbT[0]), to_frag<T>(aqbT[1]));
+        }
+        // (ag^T waits in the slot where w will go: w = Tm ag is formed further down, when the inverse is there)
+        T* const sWW = reinterpret_cast<T*>(slot + (REV ? SB.W : BF.W));
+#pragma unroll
+        for (int kp = 0; kp < KT2; ++kp) {
+            Frag<T> fagT[2][2], fkgT[2], fbg[2][2], fbgT[2][2], fqg[2], fqgT[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int kt = 2 * kp + e;
+                f32x4 gi, ge;
+                decays(kt, gi, ge);
+                const f32x4 gl = bcast16<CH - 1>(gi);
+                const f32x4 egi = exp4<T>(gi), ege = exp4<T>(ge), edn = exp4<T>(gl - gi);
+                fagT[0][e] = transpose(to_frag<T>(to_f32(ra[0][kt]) * ege), ident);
+                fagT[1][e] = transpose(to_frag<T>(to_f32(ra[1][kt]) * ege), ident);
+                fqg[e] = to_frag<T>(to_f32(rq[kt]) * egi * scale);
+                fbg[0][e] = to_frag<T>(to_f32(rb[0][kt]) * edn);
+                fbg[1][e] = to_frag<T>(to_f32(rb[1][kt]) * edn);
+                if (!REV) {
+                    fkgT[e] = transpose(to_frag<T>(to_f32(rk[kt]) * edn), ident);
+                    fbgT[0][e] = transpose(fbg[0][e], ident);
+                    fbgT[1][e] = transpose(fbg[1][e], ident);
+                } else {
+                    fqgT[e] = transpose(fqg[e], ident);
+                }
+                if (c == 0) {
+                    const f32x4 egl = exp4<T>(gl);
+                    *reinterpret_cast<f32x4*>(slot + (REV ? SB.EGL : BF.EGL) + (16 * kt + 4 * g) * 4) = egl;
+                }
+            }
+#pragma unroll
+            for (int s = 0; s < 2; ++s) st_pair2(sWW + (s * KT2 + kp) * PAIR, fagT[s][0], fagT[s][1]);
+            if (!REV) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s) st_pair2(reinterpret_cast<T*>(slot + BF.BGT) + (s * KT2 + kp) * PAIR, fbgT[s][0], fbgT[s][1]);
+                st_pair2(reinterpret_cast<T*>(slot + BF.KGT) + kp * PAIR, fkgT[0], fkgT[1]);
+                st_pair2(reinterpret_cast<T*>(slot + BF.QG) + kp * PAIR, fqg[0], fqg[1]);
+            } else {
+                // the reverse scan takes bg as it is and w transposed (the stand-alone kernel turns the stored tiles on
+                // their way into LDS: the same values)
+#pragma unroll
+                for (int s = 0; s < 2; ++s) st_pair2(reinterpret_cast<T*>(slot + SB.BGT) + (s * KT2 + kp) * PAIR, fbg[s][0], fbg[s][1]);
+                st_pair2(reinterpret_cast<T*>(slot + SB.QGT) + kp * PAIR, fqgT[0], fqgT[1]);
+            }
+        }
+        Frag<T> vT[VT];
+        if (!REV) {
+#pragma unroll
+            for (int vt = 0; vt < VT; ++vt) {
+                vT[vt] = transpose(rv[vt], ident);
+                st_tile(reinterpret_cast<T*>(slot + L::VTT) + vt * TILE, vT[vt]);
+            }
+        }
+        if (REV || CKPT) {
+            // rows past the end of a ragged chunk were taken as zeros
+#pragma unroll
+            for (int vt = 0; vt < VT; ++vt) st_tile(reinterpret_cast<T*>(slot + L::DOT) + vt * TILE, transpose(rdo[vt], ident));
+        }
+        const Frag<T> aakf[2] = {to_frag<T>(aak[0]), to_frag<T>(aak[1])};
+        // the inputs are used up: the next chunk's may come
+        __builtin_amdgcn_sched_barrier(0);
+        if (t + FNP < nst) request(t + FNP);
+        __builtin_amdgcn_sched_barrier(0);
+
+        // ---- phase B: (I - A_ab)^-1 by forward substitution (prep.hip, phase B) -------------------------------------
+        {
+            int lb = l;                                   // formed afresh per chunk (see copy_out)
+            asm volatile("" : "+v"(lb));
+            const int r = lb >> 5, col = lb & 31;
+            float x[16], y[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const float* nrow = &sN[(16 * r + i) * FLDP];
+                float acc0 = (col == 16 * r + i) ? 1.f : 0.f, acc1 = 0.f;
+#pragma unroll
+                for (int j4 = 0; j4 < (i + 3) / 4; ++j4) {
+                    const f32x4 co = *reinterpret_cast<const f32x4*>(nrow + 16 * r + 4 * j4);
+                    const f32x4 cx = *reinterpret_cast<const f32x4*>(nrow + 16 * (1 - r) + 4 * j4);
+#pragma unroll
+                    for (int jj = 0; jj < 4; ++jj) {
+                        const int j = 4 * j4 + jj;
+                        if (j < i) { acc0 = fmaf(co[jj], x[j], acc0); acc1 = fmaf(cx[jj], y[j], acc1); }
+                    }
+                }
+                x[i] = acc0 + acc1;
+                y[i] = xor32(x[i]);
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) sT[(16 * r + i) * FLDP + col] = x[i];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        Frag<T> tm[2][2];
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2)
+                tm[s][s2] = to_frag<T>(*reinterpret_cast<const f32x4*>(&sT[(16 * s + c) * FLDP + 16 * s2 + 4 * g]));
+        if (CKPT) {
+            // What the checkpoint pass leaves in the workspace for chunk_grad ((I - A_ab)^-1 here, u and where needed w
+            // below) goes there from the consumers, which have no loads to wait for: a store issued here would stand
+            // behind the next chunk's loads in this wave's in-order memory counter, and the wait for them would be a
+            // wait for it.
+            T* tmw = reinterpret_cast<T*>(slot + L::TMB);
+#pragma unroll
+            for (int s = 0; s < 2; ++s) st_pair2(tmw + s * PAIR, transpose(tm[s][0], ident), transpose(tm[s][1], ident));
+        }
+        // ---- w = Tm ag, in place of ag^T -------------------------------------------------------------------------------
+#pragma unroll
+        for (int kp = 0; kp < KT2; ++kp) {
+            Frag<T> agT[2][2], fw[2][2];
+            ld_pair(sWW + (0 * KT2 + kp) * PAIR, agT[0][0], agT[0][1]);
+            ld_pair(sWW + (1 * KT2 + kp) * PAIR, agT[1][0], agT[1][1]);
+#pragma unroll
+            for (int e = 0; e < 2; ++e)
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    f32x4 w = mm(tm[s][0], agT[0][e], zero4());
+                    w = mm(tm[s][1], agT[1][e], w);
+                    fw[s][e] = to_frag<T>(w);
+                }
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                if (!REV) st_pair2(sWW + (s * KT2 + kp) * PAIR, fw[s][0], fw[s][1]);
+                else st_pair2(sWW + (s * KT2 + kp) * PAIR, transpose(fw[s][0], ident), transpose(fw[s][1], ident));
+            }
+        }
+        // ---- phase D: u = Tm (A_ak v), transposed (prep.hip, phase D) ---------------------------------------------------
+        if (!REV) {
+#pragma unroll
+            for (int vt = 0; vt < VT; ++vt) {
+                const Frag<T> mT[2] = {to_frag<T>(mm(vT[vt], aakf[0], zero4())), to_frag<T>(mm(vT[vt], aakf[1], zero4()))};
+                Frag<T> fu[2];
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    f32x4 uT = mm(mT[0], tm[s][0], zero4());
+                    uT = mm(mT[1], tm[s][1], uT);
+                    fu[s] = to_frag<T>(uT);
+                }
+                st_pair2(reinterpret_cast<T*>(slot + L::UT) + vt * PAIR, fu[0], fu[1]);
+            }
+        }
+        signal_set(&flags[pw], it + 1);
+    }
+    // the last chunk's rows
+    if (FWD && it > 0) {
+        if (!wait_ge(&flags[4 + pw], VT * it, &flags[8])) { if (l == 0) *a.err = FUSED_ABORTED + 1; return; }
+        copy_out(prev_cid);
+    }
+}
+
+// ---- consumers, forward direction ----------------------------------------------------------------------------------
+// Fragment-order records in the workspace (256 fp32 per tile, lane l owns elements 4l..4l+3), per (sequence, head,
+// segment):
+//   sloc  [V/16][K/16] tiles  F(S^T): the state leaving the segment (started from h0 / the given boundary in segment
+//                             0 and in checkpoint mode, from zero otherwise)
+//   mseg  [K/16][K/16] tiles  the segment's transition M (segments > 0).  Forward pass: tile (kt, k't) = F(M block),
+//                             rows k, inner k'; checkpoint mode: the transposed block, rows k', inner k
+//   rseg  [V/16][K/16] tiles  F(R^T), R = sum_t G_t^T do_t (checkpoint mode, segments > 0)
+//   sin   [V/16][K/16] tiles  F(S_in^T): the state entering the segment (segments > 0)
+// W_GLOBAL: chunk_grad reads w from the workspace where it cannot rebuild it (chunk_grad_body.inc: REBUILD_W)
+template <typename T, int K, int V, int MODE, bool W_GLOBAL>
+__device__ __forceinline__ void fused_consumer_fwd(const FusedArgs<T>& a, char* smem, int n, int h, int seg, int s0, int s1, int wv) {
+    typedef FusedLds<T, K, V, MODE> L;
+    constexpr bool CKPT = MODE == FUSED_CKPT, FWD = MODE == FUSED_FWD;
+    constexpr int KT = K / 16, VT = V / 16, KT2 = KT / 2;
+    static_assert(KT == VT, "consumer j owns column block j of the state and of the transition matrix");
+    constexpr BlkF BF = L::BF;
+    const ChunkArgs<T>& p = a.c;
+    int* const flags = reinterpret_cast<int*>(smem + L::FLAGS);
+    const int l = lane_id(), g = l >> 4, c = l & 15;
+    const int H = p.H, vt = wv;
+    const int nst = s1 - s0;
+    const bool pblk = seg > 0;                            // uniform over the workgroup
+    const int64_t rec = ((int64_t)n * H + h) * a.nseg + seg;
+    const int64_t soff = ((int64_t)n * H + h) * K * V + 16 * vt + c;
+
+    // state block: lane (g,c) reg i of tile kt = S[16kt + 4g + i][16vt + c]; likewise M with column 16vt + c
+    f32x4 S[KT], M[KT], R[VT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+        S[kt] = zero4();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) M[kt][i] = (16 * kt + 4 * g + i == 16 * vt + c) ? 1.f : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < VT; ++j) R[j] = zero4();
+    if (seg == 0) {
+        if (p.h0) {
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) S[kt][i] = p.h0[soff + (int64_t)(16 * kt + 4 * g + i) * V];
+        }
+    } else if (CKPT) {
+        const float* sin = a.sin + rec * (K * V);
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) S[kt] = *reinterpret_cast<const f32x4*>(sin + (vt * KT + kt) * TILE + 4 * l);
+    }
+    const Frag<T> ident = ident_frag<T>();
+
+    for (int t = 0; t < nst; ++t) {
+        const int pp = t & (FNP - 1), it = t / FNP;
+        if (!wait_ge(&flags[pp], it + 1, &flags[8])) { if (l == 0) *a.err = FUSED_ABORTED + 2; return; }
+        const char* slot = smem + pp * L::SLOT;
+        const int cid = s0 + t;
+        const int64_t chw = (int64_t)h * p.st.nch + cid;
+        const T* sW = reinterpret_cast<const T*>(slot + BF.W);
+        const T* sBGT = reinterpret_cast<const T*>(slot + BF.BGT);
+        const T* sKGT = reinterpret_cast<const T*>(slot + BF.KGT);
+        const float* sEGL = reinterpret_cast<const float*>(slot + BF.EGL);
+        Frag<T> w[2][KT], qg[KT], aqb[2], aqk, kgt[KT], bgt[2][KT], ut[2], vtt;
+        f32x4 egl[KT];
+#pragma unroll
+        for (int kp = 0; kp < KT2; ++kp) {
+            ld_pair(sW + (0 * KT2 + kp) * PAIR, w[0][2 * kp], w[0][2 * kp + 1]);
+            ld_pair(sW + (1 * KT2 + kp) * PAIR, w[1][2 * kp], w[1][2 * kp + 1]);
+        }
+        ld_pair(reinterpret_cast<const T*>(slot + L::UT) + wv * PAIR, ut[0], ut[1]);
+        vtt = ld_tile(reinterpret_cast<const T*>(slot + L::VTT) + wv * TILE);
+        if (FWD || pblk) {
+#pragma unroll
+            for (int kp = 0; kp < KT2; ++kp) ld_pair(reinterpret_cast<const T*>(slot + BF.QG) + kp * PAIR, qg[2 * kp], qg[2 * kp + 1]);
+            ld_pair(reinterpret_cast<const T*>(slot + BF.AQB), aqb[0], aqb[1]);
+        }
+        if (FWD) aqk = ld_tile(reinterpret_cast<const T*>(slot + BF.AQK));
+#pragma unroll
+        for (int kp = 0; kp < KT2; ++kp) {
+            ld_pair(sKGT + kp * PAIR, kgt[2 * kp], kgt[2 * kp + 1]);
+            ld_pair(sBGT + (0 * KT2 + kp) * PAIR, bgt[0][2 * kp], bgt[0][2 * kp + 1]);
+            ld_pair(sBGT + (1 * KT2 + kp) * PAIR, bgt[1][2 * kp], bgt[1][2 * kp + 1]);
+            egl[2 * kp] = *reinterpret_cast<const f32x4*>(sEGL + 16 * (2 * kp) + 4 * g);
+            egl[2 * kp + 1] = *reinterpret_cast<const f32x4*>(sEGL + 16 * (2 * kp + 1) + 4 * g);
+        }
+
+        // ---- the state's column block: the stand-alone scan's step (scan_impl.cuh), operation for operation ---------
+        Frag<T> sb[KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) sb[kt] = to_frag<T>(S[kt]);
+        f32x4 vn[2] = {to_f32(ut[0]), to_f32(ut[1])};
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            vn[0] = mm(sb[kt], w[0][kt], vn[0]);
+            vn[1] = mm(sb[kt], w[1][kt], vn[1]);
+        }
+        f32x4 o = zero4();
+        if (FWD) {
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) o = mm(qg[kt], sb[kt], o);
+            o = mm(aqk, vtt, o);
+        }
+        const Frag<T> vnb[2] = {to_frag<T>(vn[0]), to_frag<T>(vn[1])};
+        if (CKPT) {
+            T* hc = p.ws.HC + chw * (K * V) + vt * PAIR;
+#pragma unroll
+            for (int kp = 0; kp < KT2; ++kp) st_pair2(hc + kp * (VT * PAIR), sb[2 * kp], sb[2 * kp + 1]);
+            // the producer's results that chunk_grad reads: this wave's tiles of u, and between the waves the two tile
+            // pairs of (I - A_ab)^-1 and (where wanted) the 2 KT/2 pairs of w
+            st_pair2(p.ws.UT + (chw * VT + vt) * PAIR, ut[0], ut[1]);
+            if (wv < 2) {
+                Frag<T> t0, t1;
+                ld_pair(reinterpret_cast<const T*>(slot + L::TMB) + wv * PAIR, t0, t1);
+                st_pair2(p.ws.TM + chw * 1024 + wv * PAIR, t0, t1);
+            }
+            if (W_GLOBAL) {
+                static_assert(!W_GLOBAL || 2 * KT2 == VT, "one pair of w per consumer");
+                T* wg = p.ws.W + chw * (p.ws.sa_stride / (int)sizeof(T));
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+#pragma unroll
+                    for (int kp = 0; kp < KT2; ++kp)
+                        if (wv == s * KT2 + kp) st_pair2(wg + (s * KT2 + kp) * PAIR, w[s][2 * kp], w[s][2 * kp + 1]);
+            }
+        }
+        if (FWD) {
+            o = mm(aqb[0], vnb[0], o);
+            o = mm(aqb[1], vnb[1], o);
+            char* ob = smem + pp * L::SLOT + L::OBOX + c * L::OROW;
+            if (seg == 0) st_frag(reinterpret_cast<T*>(ob) + 16 * wv + 4 * g, to_frag<T>(o));
+            else *reinterpret_cast<f32x4*>(ob + (16 * wv + 4 * g) * 4) = o;
+        }
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            f32x4 x = S[kt] * egl[kt];
+            x = mm(vtt, kgt[kt], x);
+            x = mm(vnb[0], bgt[0][kt], x);
+            x = mm(vnb[1], bgt[1][kt], x);
+            S[kt] = x;
+        }
+        // ---- the transition matrix's column block: the same update without the chunk's own input --------------------
+        if (pblk) {
+            Frag<T> mb[KT];
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) mb[kt] = to_frag<T>(M[kt]);
+            f32x4 vp[2] = {zero4(), zero4()};
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+                vp[0] = mm(mb[kt], w[0][kt], vp[0]);
+                vp[1] = mm(mb[kt], w[1][kt], vp[1]);
+            }
+            f32x4 G = zero4();
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) G = mm(qg[kt], mb[kt], G);
+            const Frag<T> vpb[2] = {to_frag<T>(vp[0]), to_frag<T>(vp[1])};
+            G = mm(aqb[0], vpb[0], G);
+            G = mm(aqb[1], vpb[1], G);
+            const Frag<T> Gf = to_frag<T>(G);             // rows token, inner k' (the block's columns)
+            if (FWD) st_frag(reinterpret_cast<T*>(smem + pp * L::SLOT + L::GBOX + c * L::GROW) + 16 * wv + 4 * g, Gf);
+            if (CKPT) {
+                // R[k'][v] += sum_tok G[tok][k'] do[tok][v]
+                const Frag<T> GT = transpose(Gf, ident);
+#pragma unroll
+                for (int j = 0; j < VT; ++j) R[j] = mm(GT, ld_tile(reinterpret_cast<const T*>(slot + L::DOT) + j * TILE), R[j]);
+            }
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+                f32x4 x = M[kt] * egl[kt];
+                x = mm(vpb[0], bgt[0][kt], x);
+                x = mm(vpb[1], bgt[1][kt], x);
+                M[kt] = x;
+            }
+        }
+        signal_add(&flags[4 + pp]);
+    }
+
+    // ---- what the segment leaves behind ------------------------------------------------------------------------------
+    if (a.nseg == 1) {
+        if (p.ht && !CKPT) {
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) p.ht[soff + (int64_t)(16 * kt + 4 * g + i) * V] = S[kt][i];
+        }
+        return;
+    }
+    if (!CKPT) {
+        float* sloc = a.sloc + rec * (K * V);
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<f32x4*>(sloc + (vt * KT + kt) * TILE + 4 * l) = S[kt];
+    }
+    if (pblk) {
+        float* mseg = a.mseg + rec * (K * K);
+        const Frag<float> identf = ident_frag<float>();
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            Frag<float> f;
+            f.v = M[kt];
+            if (!CKPT) f = transpose(f, identf);          // exact: fp32 products with ones and zeros
+            *reinterpret_cast<f32x4*>(mseg + (kt * KT + wv) * TILE + 4 * l) = f.v;
+        }
+        if (CKPT) {
+            float* rseg = a.rseg + rec * (K * V);
+#pragma unroll
+            for (int j = 0; j < VT; ++j) {
+                Frag<float> f;
+                f.v = R[j];
+                f = transpose(f, identf);
+                *reinterpret_cast<f32x4*>(rseg + (j * KT + wv) * TILE + 4 * l) = f.v;
+            }
+        }
+    }
+}
+
+// One step of chaining two segments, in split 2-byte products (three per tile pair: the error is that of fp32 products):
+//   X^T <- X^T Q^T + A^T   with X^T as KT fragments (rows value, inner channel) and Q as KT x KT tiles qt[kt_out][kt_in]
+template <typename T, int KT>
+__device__ __forceinline__ void chain_step(f32x4 (&X)[KT], const float* q_tiles, const float* add_tiles, int add_stride, bool out_major) {
+    const int l = lane_id();
+    Split<T> xs[KT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) split(X[kt], xs[kt]);
+    f32x4 Y[KT];
+#pragma unroll
+    for (int ko = 0; ko < KT; ++ko) {
+        f32x4 acc = *reinterpret_cast<const f32x4*>(add_tiles + ko * add_stride + 4 * l);
+#pragma unroll
+        for (int ki = 0; ki < KT; ++ki) {
+            // tile (out, in) of the transition record
+            const float* qt = q_tiles + (out_major ? (ko * KT + ki) : (ki * KT + ko)) * TILE;
+            Split<T> qs;
+            split(*reinterpret_cast<const f32x4*>(qt + 4 * l), qs);
+            acc = mm3(xs[ki], qs, acc);
+        }
+        Y[ko] = acc;
+    }
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) X[kt] = Y[kt];
+}
+
+// ---- consumers, reverse direction ------------------------------------------------------------------------------------
+template <typename T, int K, int V>
+__device__ __forceinline__ void fused_consumer_rev(const FusedArgs<T>& a, char* smem, int n, int h, int seg, int s0, int s1, int wv) {
+    typedef FusedLds<T, K, V, FUSED_REV> L;
+    constexpr int KT = K / 16, VT = V / 16, KT2 = KT / 2;
+    constexpr SlotB B = L::SB;
+    const ChunkArgs<T>& p = a.c;
+    int* const flags = reinterpret_cast<int*>(smem + L::FLAGS);
+    const int l = lane_id(), g = l >> 4, c = l & 15;
+    const int H = p.H, vt = wv;
+    const int nst = s1 - s0;
+    const int64_t soff = ((int64_t)n * H + h) * K * V + 16 * vt + c;
+
+    f32x4 dS[KT];   // lane (g,c) reg i of tile kt = dS[16kt + 4g + i][16vt + c]
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) dS[kt] = zero4();
+    if (p.dht) {
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dS[kt][i] = p.dht[soff + (int64_t)(16 * kt + 4 * g + i) * V];
+    }
+    // the gradient entering this segment from the right: through the later segments, last one first
+    for (int s = a.nseg - 1; s > seg; --s) {
+        int q0, q1;
+        seg_range(p.st, n, a.nseg, s, q0, q1);
+        if (q1 <= q0) continue;                            // uniform
+        const int64_t rec = ((int64_t)n * H + h) * a.nseg + s;
+        // tile (kt, k't) of the record holds rows k', inner k: the output index is the tile's second index
+        chain_step<T, KT>(dS, a.mseg + rec * (K * K), a.rseg + rec * (K * V) + vt * KT * TILE, TILE, false);
+    }
+
+    for (int t = 0; t < nst; ++t) {
+        const int pp = t & (FNP - 1), it = t / FNP;
+        if (!wait_ge(&flags[pp], it + 1, &flags[8])) { if (l == 0) *a.err = FUSED_ABORTED + 3; return; }
+        const char* slot = smem + pp * L::SLOT;
+        const int cid = s1 - 1 - t;
+        const int64_t chw = (int64_t)h * p.st.nch + cid;
+        const T* sWT = reinterpret_cast<const T*>(slot + B.W);
+        const T* sBG = reinterpret_cast<const T*>(slot + B.BGT);
+        const T* sQGT = reinterpret_cast<const T*>(slot + B.QGT);
+        const float* sEGL = reinterpret_cast<const float*>(slot + B.EGL);
+        Frag<T> aq[2], bg[2][KT], qgt[KT], wt[2][KT];
+        f32x4 egl[KT];
+        ld_pair(reinterpret_cast<const T*>(slot + B.AQBT), aq[0], aq[1]);
+        const Frag<T> doT = ld_tile(reinterpret_cast<const T*>(slot + L::DOT) + wv * TILE);
+#pragma unroll
+        for (int kp = 0; kp < KT2; ++kp) {
+            ld_pair(sBG + (0 * KT2 + kp) * PAIR, bg[0][2 * kp], bg[0][2 * kp + 1]);
+            ld_pair(sBG + (1 * KT2 + kp) * PAIR, bg[1][2 * kp], bg[1][2 * kp + 1]);
+            ld_pair(sQGT + kp * PAIR, qgt[2 * kp], qgt[2 * kp + 1]);
+            ld_pair(sWT + (0 * KT2 + kp) * PAIR, wt[0][2 * kp], wt[0][2 * kp + 1]);
+            ld_pair(sWT + (1 * KT2 + kp) * PAIR, wt[1][2 * kp], wt[1][2 * kp + 1]);
+            egl[2 * kp] = *reinterpret_cast<const f32x4*>(sEGL + 16 * (2 * kp) + 4 * g);
+            egl[2 * kp + 1] = *reinterpret_cast<const f32x4*>(sEGL + 16 * (2 * kp + 1) + 4 * g);
+        }
+        // the stand-alone reverse scan's step (scan_impl.cuh), operation for operation
+        Frag<T> dsb[KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) dsb[kt] = to_frag<T>(dS[kt]);
+        f32x4 dvn[2];
+        dvn[0] = mm(doT, aq[0], zero4());
+        dvn[1] = mm(doT, aq[1], zero4());
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            dvn[0] = mm(dsb[kt], bg[0][kt], dvn[0]);
+            dvn[1] = mm(dsb[kt], bg[1][kt], dvn[1]);
+        }
+        const Frag<T> dvb[2] = {to_frag<T>(dvn[0]), to_frag<T>(dvn[1])};
+        T* dhc = p.ws.DHC + chw * (K * V) + vt * PAIR;
+        T* dvp = p.ws.DVN + chw * (2 * CH * V) + vt * PAIR;
+#pragma unroll
+        for (int kp = 0; kp < KT2; ++kp) st_pair2(dhc + kp * (VT * PAIR), dsb[2 * kp], dsb[2 * kp + 1]);
+        st_pair2(dvp, dvb[0], dvb[1]);
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            f32x4 x = dS[kt] * egl[kt];
+            x = mm(doT, qgt[kt], x);
+            x = mm(dvb[0], wt[0][kt], x);
+            x = mm(dvb[1], wt[1][kt], x);
+            dS[kt] = x;
+        }
+        signal_add(&flags[4 + pp]);
+    }
+    if (seg == 0 && p.dh0) {
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) p.dh0[soff + (int64_t)(16 * kt + 4 * g + i) * V] = dS[kt][i];
+    }
+}
+
+// ---- the kernel ------------------------------------------------------------------------------------------------------
+// grid = (H, nseg, N); block = 64 (V/16 + FNP): waves 0 .. V/16-1 consume, the rest produce
+template <typename T, bool GKF32, int K, int V, int MODE, bool HD>
+__global__ __launch_bounds__(64 * (V / 16 + FNP)) void fused_kernel(FusedArgs<T> a) {
+    typedef FusedLds<T, K, V, MODE> L;
+    __shared__ __attribute__((aligned(16))) char smem[L::BYTES];
+    const int h = blockIdx.x, seg = blockIdx.y;
+    const int n = a.c.st.cu ? a.c.st.order[blockIdx.z] : (int)blockIdx.z;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    int s0, s1;
+    seg_range(a.c.st, n, a.nseg, seg, s0, s1);
+    // an empty segment leaves nothing behind (whoever chains the segments skips it), except that the first one of an
+    // empty sequence still passes the state through
+    if (s1 <= s0 && seg > 0) return;
+    if (threadIdx.x < 16) reinterpret_cast<int*>(smem + L::FLAGS)[threadIdx.x] = 0;
+    __syncthreads();
+    if (wv < V / 16) {
+        if constexpr (MODE == FUSED_REV) fused_consumer_rev<T, K, V>(a, smem, n, h, seg, s0, s1, wv);
+        else fused_consumer_fwd<T, K, V, MODE, MODE == FUSED_CKPT && (HD || GKF32)>(a, smem, n, h, seg, s0, s1, wv);
+    } else {
+        fused_producer<T, GKF32, K, V, MODE, HD>(a, smem, n, h, seg, s0, s1, wv - V / 16);
+    }
+}
+
+// ---- forward pass, second kernel: the true entering states, and their part of the output ----------------------------
+// grid = (H, nseg, N), 256 threads.  blockIdx.y = s in 1 .. nseg-1: segment s (chain the records of segments 0 .. s-1
+// into S_in(s), keep it as the boundary record, add G S_in(s) to the segment's local outputs); blockIdx.y = 0: the
+// final state (all segments chained).  Every wave chains for itself (a few dozen products), so there is no exchange.
+template <typename T, int K, int V>
+__global__ __launch_bounds__(256) void fixup_kernel(FusedArgs<T> a) {
+    constexpr int KT = K / 16, VT = V / 16;
+    constexpr int OROW = V * (int)sizeof(T) + 16;
+    __shared__ __attribute__((aligned(16))) char stage[4][CH * OROW];
+    const ChunkArgs<T>& p = a.c;
+    const int h = blockIdx.x;
+    const int n = p.st.cu ? p.st.order[blockIdx.z] : (int)blockIdx.z;
+    const int target = blockIdx.y == 0 ? a.nseg : (int)blockIdx.y;       // chain segments 0 .. target-1
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int l = lane_id(), g = l >> 4, c = l & 15;
+    const int H = p.H;
+    int s0, s1;
+    if (target < a.nseg) {
+        seg_range(p.st, n, a.nseg, target, s0, s1);
+        if (s1 <= s0) return;
+    } else if (!p.ht) return;
+    const int64_t rec0 = ((int64_t)n * H + h) * a.nseg;
+
+    // S[vt][kt]: lane (g,c) reg i = S[16kt + 4g + i][16vt + c]
+    f32x4 S[VT][KT];
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt)
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            S[vt][kt] = zero4();
+            if (p.h0) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    S[vt][kt][i] = p.h0[((int64_t)n * H + h) * K * V + (int64_t)(16 * kt + 4 * g + i) * V + 16 * vt + c];
+            }
+        }
+    for (int s = 0; s < target; ++s) {
+        int q0, q1;
+        seg_range(p.st, n, a.nseg, s, q0, q1);
+        if (q1 <= q0) continue;
+        const float* sloc = a.sloc + (rec0 + s) * (K * V);
+        if (s == 0) {
+#pragma unroll
+            for (int vt = 0; vt < VT; ++vt)
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) S[vt][kt] = *reinterpret_cast<const f32x4*>(sloc + (vt * KT + kt) * TILE + 4 * l);
+        } else {
+#pragma unroll
+            for (int vt = 0; vt < VT; ++vt) chain_step<T, KT>(S[vt], a.mseg + (rec0 + s) * (K * K), sloc + vt * KT * TILE, TILE, true);
+        }
+    }
+    if (target == a.nseg) {
+        if (wv == 0) {
+#pragma unroll
+            for (int vt = 0; vt < VT; ++vt)
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        p.ht[((int64_t)n * H + h) * K * V + (int64_t)(16 * kt + 4 * g + i) * V + 16 * vt + c] = S[vt][kt][i];
+        }
+        return;
+    }
+    if (wv == 0 && a.sin_out) {
+        float* so = a.sin_out + (rec0 + target) * (K * V);
+#pragma unroll
+        for (int vt = 0; vt < VT; ++vt)
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<f32x4*>(so + (vt * KT + kt) * TILE + 4 * l) = S[vt][kt];
+    }
+    if (!a.gw) return;                                    // chaining only (the backward pass re-deriving the states)
+    Frag<T> Sb[VT][KT];
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt)
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) Sb[vt][kt] = to_frag<T>(S[vt][kt]);
+    int c0, c1;
+    seq_chunks(p.st, n, c0, c1);
+    int64_t bos, eos;
+    seq_bounds(p.st, n, bos, eos);
+    char* const st = stage[wv];
+    for (int cid = s0 + wv; cid < s1; cid += 4) {
+        const int64_t chw = (int64_t)h * p.st.nch + cid;
+        const int64_t tok0 = bos + (int64_t)(cid - c0) * CH;
+        const int len = (int)min((int64_t)CH, eos - tok0);
+        const T* gw = a.gw + chw * (CH * K) + c * K + 4 * g;
+        const float* ol = a.ol + chw * (CH * V) + c * V + 4 * g;
+        Frag<T> G[KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) G[kt] = ld_frag(gw + 16 * kt);
+#pragma unroll
+        for (int vt = 0; vt < VT; ++vt) {
+            f32x4 o = *reinterpret_cast<const f32x4*>(ol + 16 * vt);
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) o = mm(G[kt], Sb[vt][kt], o);
+            st_frag(reinterpret_cast<T*>(st + c * OROW) + 16 * vt + 4 * g, to_frag<T>(o));
+        }
+        // whole rows, 16 bytes a lane (the wave's own staging area: LDS accesses of one wave complete in order)
+        constexpr int LPR = V * (int)sizeof(T) / 16, RPI = 64 / LPR;
+#pragma unroll
+        for (int r0 = 0; r0 < CH; r0 += RPI) {
+            const int r = r0 + l / LPR, e = (l % LPR) * 16;
+            const i32x4 x = *reinterpret_cast<const i32x4*>(st + r * OROW + e);
+            if (r < len) *reinterpret_cast<i32x4*>(reinterpret_cast<char*>(p.o + ((tok0 + r) * H + h) * V) + e) = x;
+        }
+    }
+}
+
+}  // namespace hdla

@@ -9,6 +9,9 @@ from typing import Optional
 import torch
 
 HDLA_BF16, HDLA_FP32 = 0, 1
+HDLA_VERSION = 200          # the header this binding was written against (struct layouts, entry points)
+ROUTE_AUTO, ROUTE_CLASSIC, ROUTE_FUSED = 0, 1, 2
+_ROUTES = {"": ROUTE_AUTO, "auto": ROUTE_AUTO, "classic": ROUTE_CLASSIC, "fused": ROUTE_FUSED}
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_NAME = "libhdla_hip.so"
 _lib = None
@@ -19,13 +22,13 @@ class HdlaDims(ctypes.Structure):
         ("B", ctypes.c_int32), ("T", ctypes.c_int32), ("H", ctypes.c_int32), ("K", ctypes.c_int32),
         ("V", ctypes.c_int32), ("R", ctypes.c_int32), ("N", ctypes.c_int32),
         ("in_dtype", ctypes.c_int32), ("gk_dtype", ctypes.c_int32), ("scale", ctypes.c_float),
-        ("cu_seqlens", ctypes.c_void_p),
+        ("cu_seqlens", ctypes.c_void_p), ("route", ctypes.c_int32), ("segments", ctypes.c_int32),
     ]
 
 
 class HdlaWsLayout(ctypes.Structure):
     _names = ["nch", "W", "UT", "KGT", "BGT", "VTT", "EGL", "QG", "AQK", "AQB", "AQBT", "QGT", "TM",
-              "HC", "DHC", "DVN", "STRONG", "SA_STRIDE", "SB_STRIDE", "CHUNK_OFF", "CHUNK_SEQ", "total"]
+              "HC", "DHC", "DVN", "STRONG", "SA_STRIDE", "SB_STRIDE", "CHUNK_OFF", "CHUNK_SEQ", "total", "ERR"]
     _fields_ = [(n, ctypes.c_int64) for n in _names]
 
 
@@ -65,6 +68,9 @@ def load():
     P, F = ctypes.c_void_p, ctypes.POINTER(HdlaDims)
     lib.hdla_version.restype = ctypes.c_int
     lib.hdla_version.argtypes = []
+    if lib.hdla_version() != HDLA_VERSION:
+        raise HdlaError(f"{path} is version {lib.hdla_version()} of the C ABI, this binding needs {HDLA_VERSION}: "
+                        "rebuild the library (make -C hdla-impl_amd/csrc)")
     lib.hdla_strerror.restype = ctypes.c_char_p
     lib.hdla_strerror.argtypes = [ctypes.c_int]
     lib.hdla_workspace_bytes.restype = ctypes.c_size_t
@@ -81,6 +87,12 @@ def load():
     lib.hdla_param_chunk_fwd.argtypes = [F] + [P] * 8 + [P, ctypes.c_size_t, P]
     lib.hdla_param_chunk_bwd.restype = ctypes.c_int
     lib.hdla_param_chunk_bwd.argtypes = [F] + [P] * 14 + [P, ctypes.c_size_t, P]
+    lib.hdla_boundary_bytes.restype = ctypes.c_size_t
+    lib.hdla_boundary_bytes.argtypes = [F]
+    lib.hdla_chunk_fwd_b.restype = ctypes.c_int
+    lib.hdla_chunk_fwd_b.argtypes = [F] + [P] * 10 + [P, ctypes.c_size_t, P, ctypes.c_size_t, P]
+    lib.hdla_chunk_bwd_b.restype = ctypes.c_int
+    lib.hdla_chunk_bwd_b.argtypes = [F] + [P] * 18 + [P, ctypes.c_size_t, P, ctypes.c_size_t, P]
     lib.hdla_chunk_fwd_keep.restype = ctypes.c_int
     lib.hdla_chunk_fwd_keep.argtypes = [F] + [P] * 10 + [P, ctypes.c_size_t, P]
     lib.hdla_chunk_bwd_kept.restype = ctypes.c_int
@@ -136,9 +148,38 @@ def dtype_code(dt: torch.dtype) -> int:
     raise HdlaError(f"unsupported dtype {dt}")
 
 
-def make_dims(B, T, H, K, V, R, N, in_dtype, gk_dtype, scale, cu_seqlens: Optional[torch.Tensor]) -> HdlaDims:
+def default_route() -> int:
+    """Launch plan of the chunked operators when the caller does not say: environment variable HDLA_HIP_ROUTE =
+    auto (the library chooses: the fused kernels where they are built), classic or fused."""
+    name = os.environ.get("HDLA_HIP_ROUTE", "auto").lower()
+    if name not in _ROUTES:
+        raise HdlaError(f"HDLA_HIP_ROUTE must be one of auto, classic, fused (got {name!r})")
+    return _ROUTES[name]
+
+
+def default_segments() -> int:
+    """Time segments per sequence on the fused route: environment variable HDLA_HIP_SEGMENTS, 0 = the library chooses."""
+    return int(os.environ.get("HDLA_HIP_SEGMENTS", "0"))
+
+
+def make_dims(B, T, H, K, V, R, N, in_dtype, gk_dtype, scale, cu_seqlens: Optional[torch.Tensor],
+              route: Optional[int] = None, segments: Optional[int] = None) -> HdlaDims:
     return HdlaDims(B, T, H, K, V, R, N, dtype_code(in_dtype), dtype_code(gk_dtype), float(scale),
-                    None if cu_seqlens is None else cu_seqlens.data_ptr())
+                    None if cu_seqlens is None else cu_seqlens.data_ptr(),
+                    default_route() if route is None else route, default_segments() if segments is None else segments)
+
+
+def keep_boundaries_default() -> bool:
+    """Whether the forward pass of the chunked operators hands the states at the time-segment boundaries (fused route:
+    64 KiB per sequence, head and segment) to the backward pass, which otherwise re-derives them from the inputs with
+    one more pass.  On by default; HDLA_HIP_INPUTS_ONLY=1 keeps strictly the inputs between the passes."""
+    return os.environ.get("HDLA_HIP_INPUTS_ONLY", "0") in ("", "0", "false", "False")
+
+
+def boundary(dims: HdlaDims, device) -> Optional[torch.Tensor]:
+    """An empty boundary record for these dimensions, or None where the route has none."""
+    n = load().hdla_boundary_bytes(ctypes.byref(dims))
+    return torch.empty(n, dtype=torch.uint8, device=device) if n else None
 
 
 def check_cu_seqlens(cu_seqlens: torch.Tensor, T: int) -> None:

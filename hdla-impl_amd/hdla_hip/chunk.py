@@ -64,17 +64,19 @@ def _dims(q, v, gk, scale, cu_seqlens, n_seq):
 
 
 def chunk_hrdplr_fwd(q, k, v, a, b, gk, scale, initial_state, output_final_state, cu_seqlens=None, keep=False,
-                     beta=None):
-    """Forward launch sequence (HRDPLR/hrdplr.py:25-99) on native shapes: returns (o, final_state), and with ``keep``
-    also the workspace the backward pass can run on instead of recomputing it (``hdla_chunk_fwd_keep``).  With ``beta``
-    a and b are formed in the kernels (they may be None)."""
+                     beta=None, want_boundary=False):
+    """Forward launch sequence (HRDPLR/hrdplr.py:25-99) on native shapes: returns (o, final_state), with ``keep`` also
+    the workspace the backward pass can run on instead of recomputing it (``hdla_chunk_fwd_keep``), with
+    ``want_boundary`` also the record of the states at the time-segment boundaries (None where the route has none).
+    With ``beta`` a and b are formed in the kernels (they may be None)."""
     lib = _lib.load()
     B, T, H, K = q.shape
     V = v.shape[-1]
     N = B if cu_seqlens is None else cu_seqlens.numel() - 1
     with torch.cuda.device(q.device):
         dims = _dims(q, v, gk, scale, cu_seqlens, N)
-        o = torch.empty_like(v)
+        # with a packed-sequence table that was not validated on the host, rows outside every sequence stay unwritten
+        o = torch.zeros_like(v) if cu_seqlens is not None else torch.empty_like(v)
         ht = torch.empty(N, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
         if keep:
             ws = _lib.workspace(dims, _lib.PASS_FWD_KEEP, q.device)
@@ -83,12 +85,15 @@ def chunk_hrdplr_fwd(q, k, v, a, b, gk, scale, initial_state, output_final_state
                                          _lib.ptr(ht), _lib.ptr(ws), ws.numel(), _lib.current_stream(q.device))
             _lib.check(rc, "hdla_chunk_fwd_keep")
             return o, ht, ws
-        assert beta is None
         ws = _lib.workspace(dims, _lib.PASS_FWD, q.device)
-        rc = lib.hdla_chunk_fwd(ctypes.byref(dims), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(a), _lib.ptr(b),
-                                _lib.ptr(gk), _lib.ptr(initial_state), _lib.ptr(o), _lib.ptr(ht),
-                                _lib.ptr(ws), ws.numel(), _lib.current_stream(q.device))
-        _lib.check(rc, "hdla_chunk_fwd")
+        bnd = _lib.boundary(dims, q.device) if want_boundary else None
+        rc = lib.hdla_chunk_fwd_b(ctypes.byref(dims), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(a), _lib.ptr(b),
+                                  _lib.ptr(beta), _lib.ptr(gk), _lib.ptr(initial_state), _lib.ptr(o), _lib.ptr(ht),
+                                  _lib.ptr(bnd), 0 if bnd is None else bnd.numel(),
+                                  _lib.ptr(ws), ws.numel(), _lib.current_stream(q.device))
+        _lib.check(rc, "hdla_chunk_fwd_b")
+    if want_boundary:
+        return o, ht, bnd
     return o, ht
 
 
@@ -123,23 +128,34 @@ def chunk_hrdplr_bwd_kept(q, k, v, a, b, gk, scale, initial_state, do, dht, kept
 
 
 def chunk_hrdplr_bwd(q, k, v, a, b, gk, scale, initial_state, do, dht, cu_seqlens=None, want_dh0=True,
-                     keep_workspace=False):
-    """Backward launch sequence (HRDPLR/hrdplr.py:149-284) on native shapes."""
+                     keep_workspace=False, beta=None, boundary=None):
+    """Backward launch sequence (HRDPLR/hrdplr.py:149-284) on native shapes.  Returns (dq, dk, dv, da, db, dgk, dh0), or
+    with ``beta`` (dq, dk, dv, dbeta, dgk, dh0).  ``boundary``: the record a forward pass left (see chunk_hrdplr_fwd)."""
     lib = _lib.load()
     B, T, H, K = q.shape
     V = v.shape[-1]
     N = B if cu_seqlens is None else cu_seqlens.numel() - 1
+    # rows outside every sequence of a packed batch stay unwritten: they must not carry garbage upstream
+    new = torch.zeros_like if cu_seqlens is not None else torch.empty_like
     with torch.cuda.device(q.device):
         dims = _dims(q, v, gk, scale, cu_seqlens, N)
         ws = _lib.workspace(dims, 1, q.device)
-        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-        da, db, dgk = torch.empty_like(a), torch.empty_like(b), torch.empty_like(gk)
+        dq, dk, dv, dgk = new(q), new(k), new(v), new(gk)
+        da = db = dbeta = None
+        if beta is None:
+            da, db = new(a), new(b)
+        else:
+            dbeta = new(beta)
         dh0 = torch.empty(N, H, K, V, dtype=torch.float32, device=q.device) if want_dh0 else None
-        rc = lib.hdla_chunk_bwd(ctypes.byref(dims), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(a), _lib.ptr(b),
-                                _lib.ptr(gk), _lib.ptr(initial_state), _lib.ptr(do), _lib.ptr(dht),
-                                _lib.ptr(dq), _lib.ptr(dk), _lib.ptr(dv), _lib.ptr(da), _lib.ptr(db), _lib.ptr(dgk),
-                                _lib.ptr(dh0), _lib.ptr(ws), ws.numel(), _lib.current_stream(q.device))
-        _lib.check(rc, "hdla_chunk_bwd")
+        rc = lib.hdla_chunk_bwd_b(ctypes.byref(dims), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(a), _lib.ptr(b),
+                                  _lib.ptr(beta), _lib.ptr(gk), _lib.ptr(initial_state), _lib.ptr(do), _lib.ptr(dht),
+                                  _lib.ptr(dq), _lib.ptr(dk), _lib.ptr(dv), _lib.ptr(da), _lib.ptr(db), _lib.ptr(dbeta),
+                                  _lib.ptr(dgk), _lib.ptr(dh0), _lib.ptr(boundary),
+                                  0 if boundary is None else boundary.numel(),
+                                  _lib.ptr(ws), ws.numel(), _lib.current_stream(q.device))
+        _lib.check(rc, "hdla_chunk_bwd_b")
+    if beta is not None:
+        return dq, dk, dv, dbeta, dgk, dh0
     if keep_workspace:
         return dq, dk, dv, da, db, dgk, dh0, ws, dims
     return dq, dk, dv, da, db, dgk, dh0
@@ -157,11 +173,17 @@ class ChunkDPLRDeltaRuleFunction(torch.autograd.Function):
         # keep_forward (off unless asked for): the per-chunk intermediates of this pass stay alive on ctx until the
         # backward pass, which then does not recompute them; only when a gradient can be asked for at all
         ctx.kept = None
+        boundary = None
         if keep_forward and any(ctx.needs_input_grad):
             o, final_state, ctx.kept = chunk_hrdplr_fwd(q, k, v, a, b, gk, scale, h0, output_final_state, cu_seqlens, keep=True)
+        elif any(ctx.needs_input_grad) and _lib.keep_boundaries_default():
+            o, final_state, boundary = chunk_hrdplr_fwd(q, k, v, a, b, gk, scale, h0, output_final_state, cu_seqlens,
+                                                        want_boundary=True)
         else:
             o, final_state = chunk_hrdplr_fwd(q, k, v, a, b, gk, scale, h0, output_final_state, cu_seqlens)
-        ctx.save_for_backward(q, k, v, a, b, gk, initial_state, cu_seqlens)     # inputs only (hrdplr.py:137)
+        # the inputs (hrdplr.py:137) and, where the route cuts sequences into time segments, the states at the segment
+        # boundaries (64 KiB per sequence, head and segment; HDLA_HIP_INPUTS_ONLY=1: not even those)
+        ctx.save_for_backward(q, k, v, a, b, gk, initial_state, cu_seqlens, boundary)
         ctx.scale = scale
         ctx.chunk_size = chunk_size
         ctx.output_final_state = output_final_state
@@ -173,7 +195,7 @@ class ChunkDPLRDeltaRuleFunction(torch.autograd.Function):
     @contiguous
     @autocast_custom_bwd
     def backward(ctx, do, dht):
-        q, k, v, a, b, gk, initial_state, cu_seqlens = ctx.saved_tensors
+        q, k, v, a, b, gk, initial_state, cu_seqlens, boundary = ctx.saved_tensors
         if do is None:
             do = torch.zeros_like(v)
         do = do.to(v.dtype).contiguous()
@@ -185,7 +207,7 @@ class ChunkDPLRDeltaRuleFunction(torch.autograd.Function):
                                                                  cu_seqlens, want_dh0=initial_state is not None)
         else:
             dq, dk, dv, da, db, dgk, dh0 = chunk_hrdplr_bwd(q, k, v, a, b, gk, ctx.scale, h0, do, dht, cu_seqlens,
-                                                            want_dh0=initial_state is not None)
+                                                            want_dh0=initial_state is not None, boundary=boundary)
         if dh0 is not None:
             dh0 = dh0.to(initial_state.dtype)
         # one slot per forward argument (hrdplr.py:284), plus one each for cu_seqlens and keep_forward

@@ -21,7 +21,8 @@ import torch
 import torch.nn.functional as F
 
 from . import _lib
-from .chunk import _dims, _native_dim, _pad_last, _require_gpu, chunk_hrdplr_bwd_kept, chunk_hrdplr_fwd
+from .chunk import (_dims, _native_dim, _pad_last, _require_gpu, chunk_hrdplr_bwd, chunk_hrdplr_bwd_kept,
+                    chunk_hrdplr_fwd)
 from .utils import autocast_custom_bwd, autocast_custom_fwd, contiguous
 
 
@@ -39,40 +40,14 @@ def parameterize_a_b(beta: torch.Tensor, k: torch.Tensor, log_f: torch.Tensor) -
     return a, b
 
 
-def _fwd(q, k, v, beta, gk, scale, initial_state, output_final_state, cu_seqlens):
-    lib = _lib.load()
-    B, T, H, K = q.shape
-    V = v.shape[-1]
-    N = B if cu_seqlens is None else cu_seqlens.numel() - 1
-    with torch.cuda.device(q.device):
-        dims = _dims(q, v, gk, scale, cu_seqlens, N)
-        ws = _lib.workspace(dims, 0, q.device)
-        o = torch.empty_like(v)
-        ht = torch.empty(N, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
-        rc = lib.hdla_param_chunk_fwd(ctypes.byref(dims), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(beta),
-                                      _lib.ptr(gk), _lib.ptr(initial_state), _lib.ptr(o), _lib.ptr(ht),
-                                      _lib.ptr(ws), ws.numel(), _lib.current_stream(q.device))
-        _lib.check(rc, "hdla_param_chunk_fwd")
-    return o, ht
+def _fwd(q, k, v, beta, gk, scale, initial_state, output_final_state, cu_seqlens, want_boundary=False):
+    return chunk_hrdplr_fwd(q, k, v, None, None, gk, scale, initial_state, output_final_state, cu_seqlens, beta=beta,
+                            want_boundary=want_boundary)
 
 
-def _bwd(q, k, v, beta, gk, scale, initial_state, do, dht, cu_seqlens, want_dh0):
-    lib = _lib.load()
-    B, T, H, K = q.shape
-    V = v.shape[-1]
-    N = B if cu_seqlens is None else cu_seqlens.numel() - 1
-    with torch.cuda.device(q.device):
-        dims = _dims(q, v, gk, scale, cu_seqlens, N)
-        ws = _lib.workspace(dims, 1, q.device)
-        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-        dbeta, dgk = torch.empty_like(beta), torch.empty_like(gk)
-        dh0 = torch.empty(N, H, K, V, dtype=torch.float32, device=q.device) if want_dh0 else None
-        rc = lib.hdla_param_chunk_bwd(ctypes.byref(dims), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(beta),
-                                      _lib.ptr(gk), _lib.ptr(initial_state), _lib.ptr(do), _lib.ptr(dht),
-                                      _lib.ptr(dq), _lib.ptr(dk), _lib.ptr(dv), _lib.ptr(dbeta), _lib.ptr(dgk),
-                                      _lib.ptr(dh0), _lib.ptr(ws), ws.numel(), _lib.current_stream(q.device))
-        _lib.check(rc, "hdla_param_chunk_bwd")
-    return dq, dk, dv, dbeta, dgk, dh0
+def _bwd(q, k, v, beta, gk, scale, initial_state, do, dht, cu_seqlens, want_dh0, boundary=None):
+    return chunk_hrdplr_bwd(q, k, v, None, None, gk, scale, initial_state, do, dht, cu_seqlens, want_dh0=want_dh0,
+                            beta=beta, boundary=boundary)
 
 
 class ChunkHDLAFunction(torch.autograd.Function):
@@ -85,12 +60,15 @@ class ChunkHDLAFunction(torch.autograd.Function):
     def forward(ctx, q, k, v, beta, gk, scale, initial_state, output_final_state, cu_seqlens=None, keep_forward=False):
         h0 = None if initial_state is None else initial_state.to(torch.float32).contiguous()
         ctx.kept = None
+        boundary = None
         if keep_forward and any(ctx.needs_input_grad):     # see ChunkDPLRDeltaRuleFunction.forward
             o, final_state, ctx.kept = chunk_hrdplr_fwd(q, k, v, None, None, gk, scale, h0, output_final_state, cu_seqlens,
                                                         keep=True, beta=beta)
+        elif any(ctx.needs_input_grad) and _lib.keep_boundaries_default():
+            o, final_state, boundary = _fwd(q, k, v, beta, gk, scale, h0, output_final_state, cu_seqlens, want_boundary=True)
         else:
             o, final_state = _fwd(q, k, v, beta, gk, scale, h0, output_final_state, cu_seqlens)
-        ctx.save_for_backward(q, k, v, beta, gk, initial_state, cu_seqlens)
+        ctx.save_for_backward(q, k, v, beta, gk, initial_state, cu_seqlens, boundary)
         ctx.scale = scale
         return o.to(q.dtype), final_state
 
@@ -98,7 +76,7 @@ class ChunkHDLAFunction(torch.autograd.Function):
     @contiguous
     @autocast_custom_bwd
     def backward(ctx, do, dht):
-        q, k, v, beta, gk, initial_state, cu_seqlens = ctx.saved_tensors
+        q, k, v, beta, gk, initial_state, cu_seqlens, boundary = ctx.saved_tensors
         if do is None:
             do = torch.zeros_like(v)
         do = do.to(v.dtype).contiguous()
@@ -110,7 +88,7 @@ class ChunkHDLAFunction(torch.autograd.Function):
                                                                 cu_seqlens, want_dh0=initial_state is not None, beta=beta)
         else:
             dq, dk, dv, dbeta, dgk, dh0 = _bwd(q, k, v, beta, gk, ctx.scale, h0, do, dht, cu_seqlens,
-                                               want_dh0=initial_state is not None)
+                                               want_dh0=initial_state is not None, boundary=boundary)
         if dh0 is not None:
             dh0 = dh0.to(initial_state.dtype)
         return dq.to(q), dk.to(k), dv.to(v), dbeta.to(beta), dgk.to(gk), None, dh0, None, None, None

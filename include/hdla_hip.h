@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define HDLA_VERSION 100
+#define HDLA_VERSION 200
 
 enum { HDLA_BF16 = 0, HDLA_FP32 = 1 };
 
@@ -59,8 +59,18 @@ enum {
     HDLA_ERR_WORKSPACE = -5,   /* workspace NULL, misaligned or too small */
     HDLA_ERR_ALIGN = -6,       /* a tensor pointer is not 16-byte aligned */
     HDLA_ERR_SEQ = -7,         /* cu_seqlens given with B != 1, or N inconsistent with B */
-    HDLA_ERR_STATIC_LIMIT = -8 /* hdla_chunk_fwd_static: the shape needs more than HDLA_STATIC_WORKSPACE_BYTES */
+    HDLA_ERR_STATIC_LIMIT = -8,/* hdla_chunk_fwd_static: the shape needs more than HDLA_STATIC_WORKSPACE_BYTES */
+    HDLA_ERR_ROUTE = -9        /* unknown route, negative segments, or HDLA_ROUTE_FUSED on a shape it is not built for */
 };
+
+/* Launch plans of the chunked entry points.  HDLA_ROUTE_CLASSIC: one kernel prepares every chunk (scores,
+ * (I - A_ab)^-1, w, u, gated copies) into the workspace and the state scans read it back, a head's value columns
+ * split over workgroups.  HDLA_ROUTE_FUSED (bf16 inputs, K = V = 64): the preparation runs inside the scan kernels'
+ * workgroups and reaches the scan through LDS; a sequence is cut into `segments` time segments whose affine maps are
+ * chained afterwards, so that few (sequence, head) pairs still fill the device.  HDLA_ROUTE_AUTO takes the fused route
+ * where it is built.  Both routes compute the same function; they differ in rounding only where segments > 1. */
+enum { HDLA_ROUTE_AUTO = 0, HDLA_ROUTE_CLASSIC = 1, HDLA_ROUTE_FUSED = 2 };
+#define HDLA_FUSED_ABORTED 0x48444c00
 
 typedef struct hdla_dims {
     int32_t B, T, H, K, V, R;
@@ -69,6 +79,8 @@ typedef struct hdla_dims {
     int32_t gk_dtype;          /* gk and dgk */
     float scale;               /* applied to q (HRDPLR/hrdplr.py:302) */
     const int64_t* cu_seqlens; /* DEVICE int64[N+1] cumulative sequence starts on the T axis, or NULL */
+    int32_t route;             /* HDLA_ROUTE_*; 0 = the library chooses */
+    int32_t segments;          /* fused route: time segments per sequence (at most 8); 0 = the library chooses */
 } hdla_dims;
 
 /* Byte offsets of the named intermediates inside the workspace (0 = not part of this pass); for tests and
@@ -77,7 +89,8 @@ typedef struct hdla_dims {
  * tile pairs are stored interleaved, element 8*lane + 4*which + i), "rows" are row-major, all laid out
  * [H][nch][...].  W, BGT, KGT, QG, AQB, AQK, EGL are parts of one block per (head, chunk) slot: the value given
  * is the offset for slot 0 and consecutive slots are SA_STRIDE bytes apart; likewise QGT, AQBT
- * with SB_STRIDE. */
+ * with SB_STRIDE.  On the fused route the scans' operands never reach the workspace: only UT, TM, HC, DHC, DVN,
+ * STRONG (and W where chunk_grad reads it) exist, in the backward pass. */
 typedef struct hdla_ws_layout {
     int64_t nch;               /* chunk slots per head */
     int64_t W, UT, KGT, BGT, VTT, EGL, QG, AQK, AQB, AQBT, QGT, TM, HC, DHC, DVN;
@@ -87,6 +100,9 @@ typedef struct hdla_ws_layout {
                                     * the sequences in the order the scans start them (most chunks first); int32[nch] the
                                     * sequence of each chunk slot */
     int64_t total;
+    int64_t ERR;               /* fused route: int32 that reads (HDLA_FUSED_ABORTED | 1..3) only if a wave's bounded wait for
+                                * another wave ran out (the kernels then stop early and the results are invalid); the
+                                * library never clears it; -1 on the classic route */
 } hdla_ws_layout;
 
 int hdla_version(void);
@@ -126,6 +142,25 @@ int hdla_chunk_bwd(const hdla_dims* dims, const void* q, const void* k, const vo
                    const void* b, const void* gk, const float* h0, const void* d_o, const float* dht,
                    void* dq, void* dk, void* dv, void* da, void* db, void* dgk, float* dh0,
                    void* workspace, size_t workspace_bytes, void* stream);
+
+/* hdla_chunk_fwd / hdla_chunk_bwd (or, with beta given, hdla_param_chunk_fwd / _bwd: a, b, da, db are then ignored and
+ * may be NULL) with the states at the segment boundaries handed from the forward to the backward pass.  On the fused
+ * route with several segments the backward pass needs the state entering every segment before it can checkpoint the
+ * states inside it.  The forward pass has them: given `boundary` (hdla_boundary_bytes(dims) bytes, 16-byte aligned;
+ * 64 KiB per (sequence, head, segment) at K = V = 64, i.e. under 2 % of the inputs of 512-token segments) it leaves them
+ * there, and the backward pass reads them instead of re-deriving them from the inputs with one more pass over them
+ * (which is what hdla_chunk_bwd does, and hdla_chunk_bwd_b with boundary = NULL).  The reference keeps the inputs only
+ * (ctx.save_for_backward, HRDPLR/hrdplr.py:137) and recomputes everything (:161-198); the record is what this route
+ * adds to that.  hdla_boundary_bytes returns 0 where the route has no such record (classic route, one segment):
+ * boundary is then ignored. */
+size_t hdla_boundary_bytes(const hdla_dims* dims);
+int hdla_chunk_fwd_b(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a, const void* b,
+                     const void* beta, const void* gk, const float* h0, void* o, float* ht, void* boundary,
+                     size_t boundary_bytes, void* workspace, size_t workspace_bytes, void* stream);
+int hdla_chunk_bwd_b(const hdla_dims* dims, const void* q, const void* k, const void* v, const void* a, const void* b,
+                     const void* beta, const void* gk, const float* h0, const void* d_o, const float* dht, void* dq,
+                     void* dk, void* dv, void* da, void* db, void* dbeta, void* dgk, float* dh0, const void* boundary,
+                     size_t boundary_bytes, void* workspace, size_t workspace_bytes, void* stream);
 
 /* The same operator with a and b formed inside the kernels the way the HDLA layer forms them
  * (parameterize_a_b, HRDPLR/hdla_custom.py:19-43, called at :290 right before the operator):

@@ -16,10 +16,10 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def _dims(**kw):
     d = dict(B=2, T=64, H=2, K=64, V=64, R=2, N=2, in_dtype=torch.bfloat16, gk_dtype=torch.bfloat16, scale=1.0,
-             cu_seqlens=None)
+             cu_seqlens=None, route=_lib.ROUTE_AUTO, segments=0)
     d.update(kw)
     dims = _lib.make_dims(d["B"], d["T"], d["H"], d["K"], d["V"], d["R"], d["N"], d["in_dtype"], d["gk_dtype"],
-                          d["scale"], None)
+                          d["scale"], None, route=d["route"], segments=d["segments"])
     if d["cu_seqlens"] is not None:
         dims.cu_seqlens = d["cu_seqlens"]
     return dims
@@ -33,16 +33,17 @@ def test_library_exports_every_declared_symbol():
             "hdla_chunk_bwd", "hdla_chunk_stages", "hdla_recurrent_fwd", "hdla_param_chunk_fwd", "hdla_param_chunk_bwd",
             "hdla_param_recurrent_fwd", "hdla_calib_stream", "hdla_normalize_fwd", "hdla_normalize_bwd",
             "hdla_normalize_workspace_bytes", "hdla_layer_pre_fwd", "hdla_layer_pre_bwd", "hdla_logsigmoid_fwd",
-            "hdla_logsigmoid_bwd", "hdla_skinny_wgrad", "hdla_skinny_wgrad_workspace_bytes"} <= names
+            "hdla_logsigmoid_bwd", "hdla_skinny_wgrad", "hdla_skinny_wgrad_workspace_bytes", "hdla_boundary_bytes",
+            "hdla_chunk_fwd_b", "hdla_chunk_bwd_b"} <= names
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.hdla_version() == 100
+    assert lib.hdla_version() == _lib.HDLA_VERSION == int(re.search(r"#define HDLA_VERSION (\d+)", header).group(1))
     assert lib.hdla_strerror(0) == b"success"
 
 
 def test_workspace_size_and_layout():
     lib = _lib.load()
-    d = _dims()
+    d = _dims(route=_lib.ROUTE_CLASSIC)
     fwd, bwd = lib.hdla_workspace_bytes(ctypes.byref(d), 0), lib.hdla_workspace_bytes(ctypes.byref(d), 1)
     assert 0 < fwd < bwd
     L = _lib.workspace_layout(d, 1)
@@ -60,8 +61,8 @@ def test_workspace_size_and_layout():
     assert Lf["EGL"] < Lf["AQK"] < Lf["QG"] < Lf["AQB"] < Lf["W"] + Lf["SA_STRIDE"] and Lf["SB_STRIDE"] == 0
     assert Lf["SA_STRIDE"] > L["SA_STRIDE"]
     # ragged T and packed sequences reserve one extra chunk per sequence
-    assert _lib.workspace_layout(_dims(T=65), 0)["nch"] == 2 * 5
-    assert _lib.workspace_layout(_dims(B=1, N=3, T=64, cu_seqlens=256), 0)["nch"] == 4 + 3
+    assert _lib.workspace_layout(_dims(T=65, route=_lib.ROUTE_CLASSIC), 0)["nch"] == 2 * 5
+    assert _lib.workspace_layout(_dims(B=1, N=3, T=64, cu_seqlens=256, route=_lib.ROUTE_CLASSIC), 0)["nch"] == 4 + 3
     # a forward pass that keeps its intermediates for the backward pass, and the scratch of that backward pass
     keep, kept = lib.hdla_workspace_bytes(ctypes.byref(d), 2), lib.hdla_workspace_bytes(ctypes.byref(d), 3)
     assert fwd < keep and 0 < kept < bwd and keep + kept > bwd
@@ -69,6 +70,40 @@ def test_workspace_size_and_layout():
     assert Lk["SA_STRIDE"] == Lf["SA_STRIDE"] and Lk["TM"] > Lk["AQBT"] > Lk["QGT"] > Lk["VTT"] and Lk["STRONG"] > Lk["TM"]
     assert Ls["HC"] == 0 and Ls["HC"] < Ls["DHC"] < Ls["DVN"] < Ls["total"] == kept
     assert lib.hdla_workspace_bytes(ctypes.byref(d), 4) == 0 and lib.hdla_workspace_bytes(ctypes.byref(d), -1) == 0
+
+
+def test_routes_workspaces_and_boundary_records():
+    lib = _lib.load()
+    B = lambda d: lib.hdla_boundary_bytes(ctypes.byref(d))
+    W = lambda d, p: lib.hdla_workspace_bytes(ctypes.byref(d), p)
+    # bf16 with K = V = 64 takes the fused route unless told otherwise: its scratch holds no scan operands
+    big = dict(B=4, N=4, T=2048, H=16)
+    auto, classic, fused = _dims(**big), _dims(route=_lib.ROUTE_CLASSIC, **big), _dims(route=_lib.ROUTE_FUSED, **big)
+    assert W(auto, 0) == W(fused, 0) < W(classic, 0) / 2 and W(auto, 1) == W(fused, 1) < W(classic, 1)
+    L = _lib.workspace_layout(fused, 1)
+    assert L["ERR"] >= 0 and L["total"] == W(fused, 1) and L["KGT"] == 0 and 0 < L["HC"] < L["DHC"] < L["DVN"]
+    assert _lib.workspace_layout(classic, 1)["ERR"] == -1
+    # other shapes have the classic route only
+    assert W(_dims(K=128, V=128), 0) == W(_dims(K=128, V=128, route=_lib.ROUTE_CLASSIC), 0) > 0
+    assert W(_dims(K=128, V=128, route=_lib.ROUTE_FUSED), 0) == 0
+    assert W(_dims(in_dtype=torch.float32, gk_dtype=torch.float32, route=_lib.ROUTE_FUSED), 1) == 0
+    assert W(_dims(route=3), 0) == 0 and W(_dims(segments=-1), 0) == 0
+    ok = ctypes.c_void_p(4096)
+    assert lib.hdla_chunk_fwd(ctypes.byref(_dims(route=7)), ok, ok, ok, ok, ok, ok, None, ok, None, ok, 1 << 40, None) == -9
+    assert lib.hdla_chunk_fwd(ctypes.byref(_dims(K=128, V=128, route=_lib.ROUTE_FUSED)), ok, ok, ok, ok, ok, ok, None, ok,
+                              None, ok, 1 << 40, None) == -9
+    # boundary record: one fp32 K x V state per (sequence, head, segment); none for one segment or the classic route
+    assert B(classic) == 0 and B(_dims(segments=1)) == 0
+    assert B(_dims(segments=4)) == 2 * 2 * 4 * 64 * 64 * 4
+    assert B(_dims(segments=100)) == 2 * 2 * 8 * 64 * 64 * 4                     # capped
+    # chosen by the library: enough segments to give every compute unit a workgroup, never segments of a few chunks
+    assert B(_dims(B=4, N=4, T=2048, H=16)) == 4 * 16 * 4 * 64 * 64 * 4
+    assert B(_dims(B=64, N=64, T=2048, H=16)) == 0 and B(_dims(T=64)) == 0
+    # a boundary record that is too small or misaligned is refused
+    f = lib.hdla_chunk_fwd_b
+    d4 = _dims(segments=4)
+    assert f(ctypes.byref(d4), ok, ok, ok, ok, ok, None, ok, None, ok, None, ok, 16, ok, 1 << 40, None) == -5
+    assert f(ctypes.byref(d4), ok, ok, ok, ok, ok, None, ok, None, ok, None, ctypes.c_void_p(4096 + 8), 1 << 30, ok, 1 << 40, None) == -5
 
 
 @pytest.mark.parametrize("kw,code", [
