@@ -33,7 +33,7 @@ namespace hdla {
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int FNP = 4;                    // producer waves = LDS slots
+constexpr int FNP = 4;                    // producer pairs = LDS slots
 constexpr int FLDP = 36;                  // padded row length of the 32 x 32 matrices of the triangular solve
 constexpr int FUSED_SPIN_LIMIT = 1 << 20; // polls of ~256 cycles: a tenth of a second, four orders above any real wait
 // What a wave that gave up writes to FusedArgs::err (+1 producer, +2 forward consumer, +3 reverse consumer).  The word is
@@ -68,8 +68,9 @@ template <typename T, int K, int V, int MODE> struct FusedLds {
     static constexpr int OBOX = OPER, GBOX = OBOX + (MODE == FUSED_FWD ? CH * OROW : 0);
     static constexpr int SOLVE = GBOX + (MODE == FUSED_FWD ? CH * GROW : 0);
     static constexpr int SLOT = SOLVE + 2 * 32 * FLDP * 4;
-    static constexpr int FLAGS = FNP * SLOT;        // int ready[4], consumed[4], abort
-    static constexpr int BYTES = FLAGS + 64;
+    // int ready[4], consumed[4], abort, -, -, -, part[4], inv[4], strong[4] (per producer pair; see fused_producer)
+    static constexpr int FLAGS = FNP * SLOT;
+    static constexpr int BYTES = FLAGS + 128;
 };
 
 // ---- hand-over counters ------------------------------------------------------------------------------------------
@@ -107,33 +108,54 @@ template <typename T> struct GkRaw<T, true> {
     static __device__ __forceinline__ f32x4 value(type x, bool ok) { return ok ? x : zero4(); }
 };
 
-// ---- producer ----------------------------------------------------------------------------------------------------
-// Everything of a chunk that does not depend on the state, by one wave, into LDS slot `pw`.  The arithmetic is the
-// stand-alone prep kernel's, operation for operation (prep.hip), so both routes hand the scans the same bits.
+// F(I16) for lane (g, c), like ident_frag() but from the caller's lane coordinates
+template <typename T> __device__ __forceinline__ Frag<T> ident_of(int g, int c) {
+    f32x4 e;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) e[i] = (c == 4 * g + i) ? 1.f : 0.f;
+    return to_frag<T>(e);
+}
+
+// ---- producers -----------------------------------------------------------------------------------------------------
+// Everything of a chunk that does not depend on the state, by a PAIR of waves, into LDS slot `pp`.  Wave `half` of the
+// pair takes the channel tiles 2 half, 2 half + 1 (one stored tile pair of every operand) and half of the value tiles.
+// The score tiles are sums over all channels: the other wave hands its parts to the pair's `lead` wave through LDS, the
+// lead solves the (small) triangular system and hands (I - A_ab)^-1 and A_ak back, and each forms w and u for its own
+// tiles.  The formulas are the stand-alone prep kernel's (prep.hip); what differs from its one-wave form is the order
+// in which the two halves of a score tile's sum over channels are added.
+//
+// One wave per chunk (the first form of this kernel) took 19,000 cycles a chunk, most of them waiting for its own
+// previous instruction: alone on its SIMD nothing fills those gaps.  Two waves per chunk on three waves per SIMD do.
 template <typename T, bool GKF32, int K, int V, int MODE, bool HD>
-__device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem, int n, int h, int seg, int s0, int s1, int pw) {
-    static_assert(K == 64 && sizeof(T) == 2, "one producer wave holds all channels of a chunk: K = 64, 2-byte elements");
+__device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem, int n, int h, int seg, int s0, int s1, int pp, int half) {
+    static_assert(K == 64 && sizeof(T) == 2 && V % 32 == 0, "a producer pair holds all channels of a chunk: K = 64, 2-byte elements");
     typedef FusedLds<T, K, V, MODE> L;
     constexpr bool REV = MODE == FUSED_REV, CKPT = MODE == FUSED_CKPT, FWD = MODE == FUSED_FWD;
-    constexpr int KT = K / 16, VT = V / 16, KT2 = KT / 2;
+    constexpr int KT = K / 16, VT = V / 16, KT2 = KT / 2, KH = 2, VH = VT / 2;
     constexpr BlkF BF = L::BF;
     constexpr SlotB SB = L::SB;
     const ChunkArgs<T>& p = a.c;
-    char* const slot = smem + pw * L::SLOT;
-    float* const sN = reinterpret_cast<float*>(slot + L::SOLVE);
-    float* const sT = sN + 32 * FLDP;
+    char* slot = smem + pp * L::SLOT;
+    // the pair's scratch: first the other wave's parts of the nine score tiles (fp32, 9 KiB); then, in the same bytes,
+    // A_ab and its inverse for the solve; then the inverse and A_ak as operand tiles for the other wave
+    float *sP, *sN, *sT;
+    T* sPub;
     int* const flags = reinterpret_cast<int*>(smem + L::FLAGS);
-    const int l = lane_id(), g = l >> 4, c = l & 15;
+    int* const f_ready = flags + pp, * const f_consumed = flags + 4 + pp, * const f_abort = flags + 8;
+    int* const f_part = flags + 12 + pp, * const f_inv = flags + 16 + pp, * const f_strong = flags + 20 + pp;
+    const bool lead = half == (pp >> 1);                  // spreads the leads over the SIMDs
+    int l = lane_id(), g = l >> 4, c = l & 15;
     const int H = p.H;
     const float scale = p.scale;
     const int nst = s1 - s0;
+    const int kt0 = half * KH, vt0 = half * VH;
     int64_t bos, eos;
     seq_bounds(p.st, n, bos, eos);
     int c0, c1;
     seq_chunks(p.st, n, c0, c1);
-    const Frag<T> ident = ident_frag<T>();
 
-    // rows of the previous chunk's results, left in the outbox by the consumers, out to global memory (forward pass)
+    // rows of the previous chunk's results, left in the outbox by the consumers, out to global memory (forward pass);
+    // each wave of the pair takes half of the rows
     auto copy_out = [&](int cid) __attribute__((always_inline)) {
         if constexpr (FWD) {
             // the lane's offsets below are formed afresh in every call: hoisted out of the chunk loop they would be held
@@ -143,11 +165,12 @@ __device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem
             const int64_t tok0 = bos + (int64_t)(cid - c0) * CH;
             const int len = (int)min((int64_t)CH, eos - tok0);
             const int64_t chw = (int64_t)h * p.st.nch + cid;
+            const int rb = half * (CH / 2);
             if (seg == 0) {
                 constexpr int LPR = V * (int)sizeof(T) / 16, RPI = 64 / LPR;
 #pragma unroll
-                for (int r0 = 0; r0 < CH; r0 += RPI) {
-                    const int r = r0 + l / LPR, e = (l % LPR) * 16;
+                for (int r0 = 0; r0 < CH / 2; r0 += RPI) {
+                    const int r = rb + r0 + l / LPR, e = (l % LPR) * 16;
                     const i32x4 x = *reinterpret_cast<const i32x4*>(slot + L::OBOX + r * L::OROW + e);
                     if (r < len) *reinterpret_cast<i32x4*>(reinterpret_cast<char*>(p.o + ((tok0 + r) * H + h) * V) + e) = x;
                 }
@@ -155,28 +178,33 @@ __device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem
                 constexpr int LPO = V * 4 / 16, RPO = 64 / LPO;
                 char* ol = reinterpret_cast<char*>(a.ol + chw * (CH * V));
 #pragma unroll
-                for (int r0 = 0; r0 < CH; r0 += RPO) {
-                    const int r = r0 + l / LPO, e = (l % LPO) * 16;
+                for (int r0 = 0; r0 < CH / 2; r0 += RPO) {
+                    const int r = rb + r0 + l / LPO, e = (l % LPO) * 16;
                     *reinterpret_cast<i32x4*>(ol + r * (V * 4) + e) = *reinterpret_cast<const i32x4*>(slot + L::OBOX + r * L::OROW + e);
                 }
                 constexpr int LPG = K * (int)sizeof(T) / 16, RPG = 64 / LPG;
                 char* gw = reinterpret_cast<char*>(a.gw + chw * (CH * K));
 #pragma unroll
-                for (int r0 = 0; r0 < CH; r0 += RPG) {
-                    const int r = r0 + l / LPG, e = (l % LPG) * 16;
+                for (int r0 = 0; r0 < CH / 2; r0 += RPG) {
+                    const int r = rb + r0 + l / LPG, e = (l % LPG) * 16;
                     *reinterpret_cast<i32x4*>(gw + r * (K * (int)sizeof(T)) + e) = *reinterpret_cast<const i32x4*>(slot + L::GBOX + r * L::GROW + e);
                 }
             }
         }
     };
 
-    // The chunk's inputs as loaded, four elements a lane (lane (g,c): token c, channels 16kt + 4g ..): requested one
-    // chunk of this wave ahead (as soon as the registers are free), so that the round trip to HBM runs behind the rest
-    // of the previous chunk.  Nothing is done to them at the load (a select or a conversion would wait for the data).
-    Frag<T> nq[KT], nk[KT], na[2][KT], nb[2][KT], nv[VT], ndo[VT];
-    typename GkRaw<T, GKF32>::type ng[KT];
+    // The wave's share of the chunk's inputs as loaded, four elements a lane (lane (g,c): token c, channels 16kt + 4g ..):
+    // requested one chunk of this pair ahead, as soon as the registers are free, so that the round trip to HBM runs
+    // behind the rest of the previous chunk.  Nothing is done to them at the load (a select or a conversion would wait
+    // for the data).  With the HDLA parameterisation the sum over ALL channels of k^2 f is needed: the other half's k and
+    // gk come along.
+    Frag<T> nq[KH], nk[KH], na[2][KH], nb[2][KH], nv[VH], ndo[VH], ok_[KH];
+    typename GkRaw<T, GKF32>::type ng[KH], og[KH];
     T nbeta;
-    auto request = [&](int t) __attribute__((always_inline)) {
+    // first: the first own channel tile's operands (requested a chunk ahead); !first: everything else of the chunk
+    // (requested when its turn begins: it arrives behind the work on the first tile).  More a chunk ahead would be more
+    // registers held through the whole chunk than three waves per SIMD leave.
+    auto request = [&](int t, bool first) __attribute__((always_inline)) {
         const int cid = REV ? s1 - 1 - t : s0 + t;
         const int64_t tok0 = bos + (int64_t)(cid - c0) * CH;
         const int len = (int)min((int64_t)CH, eos - tok0);
@@ -190,26 +218,40 @@ __device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem
         const uint32_t ve = row * (uint32_t)(H * V) + 4 * gg;
         const int64_t qb = (tok0 * H + h) * K, ab = (tok0 * RANK * H + h) * K, vb = (tok0 * H + h) * V;
         const char* gkp = reinterpret_cast<const char*>(p.gk) + qb * GS;
-        if (!REV) {
+        if (!first) {
+            if (!REV) {
 #pragma unroll
-            for (int vt = 0; vt < VT; ++vt) nv[vt] = ld_frag(at(p.v + vb, (ve + 16 * vt) * ES));
+                for (int j = 0; j < VH; ++j) nv[j] = ld_frag(at(p.v + vb, (ve + 16 * (vt0 + j)) * ES));
+            }
+            if (REV || CKPT) {
+#pragma unroll
+                for (int j = 0; j < VH; ++j) ndo[j] = ld_frag(at(p.dout + vb, (ve + 16 * (vt0 + j)) * ES));
+            }
         }
-        if (REV || CKPT) {
+        if (HD && first) nbeta = *at(p.beta + tok0 * H + h, row * (uint32_t)H * ES);
 #pragma unroll
-            for (int vt = 0; vt < VT; ++vt) ndo[vt] = ld_frag(at(p.dout + vb, (ve + 16 * vt) * ES));
-        }
-        if (HD) nbeta = *at(p.beta + tok0 * H + h, row * (uint32_t)H * ES);
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt) {
-            const uint32_t ko = 16 * kt;
-            ng[kt] = GkRaw<T, GKF32>::load(gkp + (qe + ko) * GS);
-            nq[kt] = ld_frag(at(p.q + qb, (qe + ko) * ES));
-            nk[kt] = ld_frag(at(p.k + qb, (qe + ko) * ES));
+        for (int j = 0; j < KH; ++j) {
+            const uint32_t ko = 16 * (kt0 + j), kx = 16 * (KH - kt0 + j);
+            if (HD && first) {
+                // the sum over all channels comes before everything else: k and gk of every tile a chunk ahead
+                if (j > 0) {
+                    ng[j] = GkRaw<T, GKF32>::load(gkp + (qe + ko) * GS);
+                    nk[j] = ld_frag(at(p.k + qb, (qe + ko) * ES));
+                }
+                og[j] = GkRaw<T, GKF32>::load(gkp + (qe + kx) * GS);
+                ok_[j] = ld_frag(at(p.k + qb, (qe + kx) * ES));
+            }
+            if ((j == 0) != first) continue;
+            nq[j] = ld_frag(at(p.q + qb, (qe + ko) * ES));
+            if (!(HD && j > 0)) {
+                ng[j] = GkRaw<T, GKF32>::load(gkp + (qe + ko) * GS);
+                nk[j] = ld_frag(at(p.k + qb, (qe + ko) * ES));
+            }
             if (!HD) {
-                na[0][kt] = ld_frag(at(p.a + ab, (ae + ko) * ES));
-                na[1][kt] = ld_frag(at(p.a + ab, (ae + (uint32_t)(H * K) + ko) * ES));
-                nb[0][kt] = ld_frag(at(p.b + ab, (ae + ko) * ES));
-                nb[1][kt] = ld_frag(at(p.b + ab, (ae + (uint32_t)(H * K) + ko) * ES));
+                na[0][j] = ld_frag(at(p.a + ab, (ae + ko) * ES));
+                na[1][j] = ld_frag(at(p.a + ab, (ae + (uint32_t)(H * K) + ko) * ES));
+                nb[0][j] = ld_frag(at(p.b + ab, (ae + ko) * ES));
+                nb[1][j] = ld_frag(at(p.b + ab, (ae + (uint32_t)(H * K) + ko) * ES));
             }
         }
     };
@@ -218,94 +260,161 @@ __device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem
         r.v = ok ? f.v : zero_frag<T>().v;
         return r;
     };
-    if (pw < nst) request(pw);
+    if (pp < nst) request(pp, true);
 
     int it = 0, prev_cid = -1;
-    for (int t = pw; t < nst; t += FNP, ++it) {
+    for (int t = pp; t < nst; t += FNP, ++it) {
         const int cid = REV ? s1 - 1 - t : s0 + t;
         const int64_t tok0 = bos + (int64_t)(cid - c0) * CH;
         const int len = (int)min((int64_t)CH, eos - tok0);
         const int64_t chw = (int64_t)h * p.st.nch + cid;
+        // What depends on the lane only (offsets into the slot, masks, the identity tile) is formed afresh for every chunk:
+        // hoisted out of the loop it would be held in registers, or spilled, through all of it.
+        asm volatile("" : "+v"(l));
+        g = l >> 4;
+        c = l & 15;
+        {
+            int so = pp * L::SLOT;
+            asm volatile("" : "+s"(so));
+            slot = smem + so;
+            sP = reinterpret_cast<float*>(slot + L::SOLVE);
+            sN = sP;
+            sT = sP + 32 * FLDP;
+            sPub = reinterpret_cast<T*>(sP);
+        }
+        const Frag<T> ident = ident_of<T>(g, c);
         const bool rowok = c < len;
 
-        // ---- phase A: cumulative decays and the score tiles (prep.hip, phase A) ------------------------------------
-        // (the cumulative decays of a channel tile are formed again wherever they are needed, from the log-decays as
-        // loaded, instead of being kept: the same values for fewer registers)
-        auto decays = [&](int kt, f32x4& gi, f32x4& ge) __attribute__((always_inline)) {
-            const f32x4 g4 = GkRaw<T, GKF32>::value(ng[kt], rowok);
-            gi = scan16_incl(g4);
-            ge = gi - g4;
-        };
-        float big = 0.f;                                  // see strong_decay()
+        // ---- the slot: wait until the consumers have left the chunk it held ---------------------------------------------
+        // (at the top, so that every tile can go to the slot as it is formed instead of being held in registers; the
+        // consumers are through with the slot a step of theirs after this pair's last signal, long before this pair is
+        // back here, unless they are what limits the kernel anyway)
+        if (!wait_ge(f_consumed, VT * it, f_abort)) { if (l == 0) *a.err = FUSED_ABORTED + 1; return; }
+        __builtin_amdgcn_sched_barrier(0);
+        // The rows the consumers left in the outbox for that chunk go out first (the consumers write the outbox again
+        // only after both signals at the end).
+        if (it > 0) copy_out(prev_cid);
+        prev_cid = cid;
+        __builtin_amdgcn_sched_barrier(0);
+        request(t, false);                                // the rest of this chunk's inputs, behind those stores
+        __builtin_amdgcn_sched_barrier(0);
+        // (ag^T waits in the slot where w will go: w = Tm ag is formed further down, when the inverse is there)
+        T* const sWW = reinterpret_cast<T*>(slot + (REV ? SB.W : BF.W));
+
+        // ---- own channel tiles: decays, parts of the score tiles, gated copies (prep.hip, phases A and C) -------------
         f32x4 aqk = zero4(), aqb[2] = {zero4(), zero4()}, aak[2] = {zero4(), zero4()};
         f32x4 aab[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
         f32x4 aqbT[2] = {zero4(), zero4()};
-        Frag<T> rq[KT], rk[KT], ra[2][KT], rb[2][KT];
-        Frag<T> rv[VT], rdo[VT];
-        if (!REV) {
-#pragma unroll
-            for (int vt = 0; vt < VT; ++vt) rv[vt] = sel(nv[vt], rowok);
-        }
-        if (REV || CKPT) {
-#pragma unroll
-            for (int vt = 0; vt < VT; ++vt) rdo[vt] = sel(ndo[vt], rowok);
-        }
+        float big = 0.f;                                  // see strong_decay()
         float beta_t = 0.f, s_t = 0.f;
         if (HD) {
             beta_t = rowok ? ld_elem(&nbeta) : 0.f;
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt) {
-                const f32x4 g4 = GkRaw<T, GKF32>::value(ng[kt], rowok);
-                const f32x4 k4 = to_f32(sel(nk[kt], rowok));
-                const f32x4 kf = k4 * k4 * exp4<T>(g4);
+            for (int j = 0; j < KH; ++j) {
+                const f32x4 g4 = GkRaw<T, GKF32>::value(ng[j], rowok), gx = GkRaw<T, GKF32>::value(og[j], rowok);
+                const f32x4 k4 = to_f32(sel(nk[j], rowok)), kx = to_f32(sel(ok_[j], rowok));
+                const f32x4 kf = k4 * k4 * exp4<T>(g4) + kx * kx * exp4<T>(gx);
                 s_t += kf[0] + kf[1] + kf[2] + kf[3];
             }
             s_t += __shfl_xor(s_t, 16);
             s_t += __shfl_xor(s_t, 32);
         }
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt) {
-            const f32x4 g4 = GkRaw<T, GKF32>::value(ng[kt], rowok);
-            rq[kt] = sel(nq[kt], rowok);
-            rk[kt] = sel(nk[kt], rowok);
+        // the operands of channel tile j as the products take them: as loaded, or (HDLA parameterisation) formed from k,
+        // gk, beta and s
+        auto operands = [&](int j, f32x4 g4, Frag<T>& rq, Frag<T>& rk, Frag<T> (&ra)[2], Frag<T> (&rb)[2]) __attribute__((always_inline)) {
+            rq = sel(nq[j], rowok);
+            rk = sel(nk[j], rowok);
             if (HD) {
-                const f32x4 kk = to_f32(rk[kt]), f4 = exp4<T>(g4);
-                ra[0][kt] = to_frag<T>(kk * (-beta_t));
-                ra[1][kt] = to_frag<T>(kk * ((beta_t * s_t - f4) * beta_t));
-                rb[0][kt] = to_frag<T>(f4 * kk);
-                rb[1][kt] = rk[kt];
+                const f32x4 kk = to_f32(rk), f4 = exp4<T>(g4);
+                ra[0] = to_frag<T>(kk * (-beta_t));
+                ra[1] = to_frag<T>(kk * ((beta_t * s_t - f4) * beta_t));
+                rb[0] = to_frag<T>(f4 * kk);
+                rb[1] = rk;
             } else {
-                ra[0][kt] = sel(na[0][kt], rowok);
-                ra[1][kt] = sel(na[1][kt], rowok);
-                rb[0][kt] = sel(nb[0][kt], rowok);
-                rb[1][kt] = sel(nb[1][kt], rowok);
+                ra[0] = sel(na[0][j], rowok);
+                ra[1] = sel(na[1][j], rowok);
+                rb[0] = sel(nb[0][j], rowok);
+                rb[1] = sel(nb[1][j], rowok);
             }
+        };
+        auto decays = [&](int j, f32x4& gi, f32x4& ge) __attribute__((always_inline)) {
+            const f32x4 g4 = GkRaw<T, GKF32>::value(ng[j], rowok);
+            gi = scan16_incl(g4);
+            ge = gi - g4;
+        };
+#pragma unroll
+        for (int j = 0; j < KH; ++j) {
+            const f32x4 g4 = GkRaw<T, GKF32>::value(ng[j], rowok);
+            Frag<T> rq, rk, ra[2], rb[2];
+            operands(j, g4, rq, rk, ra, rb);
             const f32x4 gi = scan16_incl(g4), ge = gi - g4;
             const f32x4 m = bcast16<MID>(gi);
 #pragma unroll
             for (int i = 0; i < 4; ++i) big = fmaxf(big, fmaxf(fabsf(gi[i] - m[i]), fabsf(ge[i] - m[i])));
-            const f32x4 eq = exp4<T>(gi - m), ek = exp4<T>(m - gi), ea = exp4<T>(ge - m);
-            const f32x4 q4 = to_f32(rq[kt]), k4 = to_f32(rk[kt]);
-            const f32x4 a0 = to_f32(ra[0][kt]), a1 = to_f32(ra[1][kt]), b0 = to_f32(rb[0][kt]), b1 = to_f32(rb[1][kt]);
-            Split<T> qh, kh, ah[2], bh[2];
-            split(q4 * eq * scale, qh);
-            split(k4 * ek, kh);
-            split(a0 * ea, ah[0]);
-            split(a1 * ea, ah[1]);
-            split(b0 * ek, bh[0]);
-            split(b1 * ek, bh[1]);
-            if (FWD) aqk = mm3(qh, kh, aqk);
+            // One row-side operand at a time against the three inner-side ones, the scheduler kept from interleaving the
+            // groups (each tile still gets its products in the order of the channel tiles): all six split operands
+            // at once are more registers than three waves per SIMD leave.
+            {
+                const f32x4 ek = exp4<T>(m - gi);
+                Split<T> kh, bh[2];
+                split(to_f32(rk) * ek, kh);
+                split(to_f32(rb[0]) * ek, bh[0]);
+                split(to_f32(rb[1]) * ek, bh[1]);
+                __builtin_amdgcn_sched_barrier(0);
+                {
+                    Split<T> qh;
+                    split(to_f32(rq) * exp4<T>(gi - m) * scale, qh);
+                    if (FWD) aqk = mm3(qh, kh, aqk);
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                if (!REV) aqb[s] = mm3(qh, bh[s], aqb[s]);
-                if (!REV) aak[s] = mm3(ah[s], kh, aak[s]);
-                if (REV) aqbT[s] = mm3(bh[s], qh, aqbT[s]);
+                    for (int s = 0; s < 2; ++s) {
+                        if (!REV) aqb[s] = mm3(qh, bh[s], aqb[s]);
+                        if (REV) aqbT[s] = mm3(bh[s], qh, aqbT[s]);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                const f32x4 ea = exp4<T>(ge - m);
 #pragma unroll
-                for (int r = 0; r < 2; ++r) aab[r][s] = mm3(ah[r], bh[s], aab[r][s]);
+                for (int r = 0; r < 2; ++r) {
+                    Split<T> ah;
+                    split(to_f32(ra[r]) * ea, ah);
+                    if (!REV) aak[r] = mm3(ah, kh, aak[r]);
+                    aab[r][0] = mm3(ah, bh[0], aab[r][0]);
+                    aab[r][1] = mm3(ah, bh[1], aab[r][1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
+            pin(rq); pin(rk); pin(ra[0]); pin(ra[1]); pin(rb[0]); pin(rb[1]);
+            const f32x4 q4 = to_f32(rq), k4 = to_f32(rk);
+            const f32x4 a0 = to_f32(ra[0]), a1 = to_f32(ra[1]), b0 = to_f32(rb[0]), b1 = to_f32(rb[1]);
+            // the gated copies, while the operands are at hand: each tile goes to its half of the stored pair
+            // (scheduling barriers: the products above, the copies below and the next tile are kept apart, or their
+            // temporaries would all be live at once)
+            __builtin_amdgcn_sched_barrier(0);
+            const f32x4 gl = bcast16<CH - 1>(gi);
+            const f32x4 egi = exp4<T>(gi), ege = exp4<T>(ge), edn = exp4<T>(gl - gi);
+            st_pair(sWW + (0 * KT2 + half) * PAIR, j, transpose(to_frag<T>(a0 * ege), ident));
+            st_pair(sWW + (1 * KT2 + half) * PAIR, j, transpose(to_frag<T>(a1 * ege), ident));
+            const Frag<T> fqg = to_frag<T>(q4 * egi * scale);
+            const Frag<T> fbg[2] = {to_frag<T>(b0 * edn), to_frag<T>(b1 * edn)};
+            if (!REV) {
+                st_pair(reinterpret_cast<T*>(slot + BF.KGT) + half * PAIR, j, transpose(to_frag<T>(k4 * edn), ident));
+                st_pair(reinterpret_cast<T*>(slot + BF.BGT) + (0 * KT2 + half) * PAIR, j, transpose(fbg[0], ident));
+                st_pair(reinterpret_cast<T*>(slot + BF.BGT) + (1 * KT2 + half) * PAIR, j, transpose(fbg[1], ident));
+                st_pair(reinterpret_cast<T*>(slot + BF.QG) + half * PAIR, j, fqg);
+            } else {
+                // the reverse scan takes bg as it is and w transposed (the stand-alone kernel turns the stored tiles on
+                // their way into LDS: the same values)
+                st_pair(reinterpret_cast<T*>(slot + SB.BGT) + (0 * KT2 + half) * PAIR, j, fbg[0]);
+                st_pair(reinterpret_cast<T*>(slot + SB.BGT) + (1 * KT2 + half) * PAIR, j, fbg[1]);
+                st_pair(reinterpret_cast<T*>(slot + SB.QGT) + half * PAIR, j, transpose(fqg, ident));
+            }
+            if (c == 0) *reinterpret_cast<f32x4*>(slot + (REV ? SB.EGL : BF.EGL) + (16 * (kt0 + j) + 4 * g) * 4) = exp4<T>(gl);
+            __builtin_amdgcn_sched_barrier(0);
         }
+        // Each wave decides for its own channels (the parts of the score tiles add up whichever way they were formed).
+        // Where a channel decays too strongly for the single centre, what was accumulated above may hold infinities: it
+        // is thrown away and the parts are formed again by passes whose exponents cannot overflow (see DecayPass).
         const bool strong = __any(big > SAFE_RANGE) != 0;  // the same answer on every lane of the wave
-        if (CKPT && l == 0) p.ws.STRONG[chw] = strong;
         if (strong) {
             aqk = zero4();
 #pragma unroll
@@ -316,19 +425,21 @@ __device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem
             for (int ps = 0; ps < DecayPass::COUNT; ++ps) {
                 const DecayPass dp(ps, c);
 #pragma unroll
-                for (int kt = 0; kt < KT; ++kt) {
+                for (int j = 0; j < KH; ++j) {
                     f32x4 gi, ge, eq, ek, ea;
-                    decays(kt, gi, ge);
+                    decays(j, gi, ge);
                     dp.factors<T>(gi, ge, eq, ek, ea);
-                    pin(rk[kt]); pin(rq[kt]); pin(ra[0][kt]); pin(ra[1][kt]); pin(rb[0][kt]); pin(rb[1][kt]);
+                    Frag<T> rq, rk, ra[2], rb[2];
+                    operands(j, gi - ge, rq, rk, ra, rb);
+                    pin(rk); pin(rq); pin(ra[0]); pin(ra[1]); pin(rb[0]); pin(rb[1]);
                     Split<T> qh, kh, bh[2];
-                    split(to_f32(rk[kt]) * ek, kh);
-                    split(to_f32(rq[kt]) * eq * scale, qh);
+                    split(to_f32(rk) * ek, kh);
+                    split(to_f32(rq) * eq * scale, qh);
                     if (FWD) aqk = mm3(qh, kh, aqk);
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int s = 0; s < 2; ++s) {
-                        split(to_f32(rb[s][kt]) * ek, bh[s]);
+                        split(to_f32(rb[s]) * ek, bh[s]);
                         if (!REV) aqb[s] = mm3(qh, bh[s], aqb[s]);
                         if (REV) aqbT[s] = mm3(bh[s], qh, aqbT[s]);
                         __builtin_amdgcn_sched_barrier(0);
@@ -336,7 +447,7 @@ __device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem
 #pragma unroll
                     for (int r = 0; r < 2; ++r) {
                         Split<T> ah;
-                        split(to_f32(ra[r][kt]) * ea, ah);
+                        split(to_f32(ra[r]) * ea, ah);
                         if (!REV) aak[r] = mm3(ah, kh, aak[r]);
                         aab[r][0] = mm3(ah, bh[0], aab[r][0]);
                         aab[r][1] = mm3(ah, bh[1], aab[r][1]);
@@ -345,153 +456,131 @@ __device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem
                 }
             }
         }
-        // causal masks: lane (g,c) reg i is entry (row c, inner 4g+i)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int j = 4 * g + i;
-            const bool le = j <= c, lt = j < c, tle = c <= j;
-            if (!le) { aqk[i] = 0.f; aqb[0][i] = 0.f; aqb[1][i] = 0.f; }
-            if (!lt) { aak[0][i] = 0.f; aak[1][i] = 0.f; aab[0][0][i] = 0.f; aab[0][1][i] = 0.f; aab[1][0][i] = 0.f; aab[1][1][i] = 0.f; }
-            if (!tle) { aqbT[0][i] = 0.f; aqbT[1][i] = 0.f; }
-        }
-        // the solver's scratch is this wave's own: nobody else reads it
-        // (the scheduling barriers stand where the stand-alone kernel has workgroup barriers: they keep the phases from
-        // being interleaved, which the register file has no room for)
+        // the first tile's inputs are used up: the next chunk's may come
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int r = 0; r < 2; ++r)
-#pragma unroll
-            for (int s = 0; s < 2; ++s)
-                *reinterpret_cast<f32x4*>(&sN[(16 * r + c) * FLDP + 16 * s + 4 * g]) = aab[r][s];
-
-        // ---- the slot: wait until the consumers have left the chunk it held ---------------------------------------------
-        if (!wait_ge(&flags[4 + pw], VT * it, &flags[8])) { if (l == 0) *a.err = FUSED_ABORTED + 1; return; }
-        __builtin_amdgcn_sched_barrier(0);
-        // The rows the consumers left in the outbox for that chunk go out first (the consumers write the outbox again
-        // only after the signal at the end): these stores are then ahead of the next chunk's loads in the wave's
-        // in-order memory counter, not behind them.
-        if (it > 0) copy_out(prev_cid);
-        prev_cid = cid;
+        if (t + FNP < nst) request(t + FNP, true);
         __builtin_amdgcn_sched_barrier(0);
 
-        // ---- everything that needs the inputs but not (I - A_ab)^-1: score tiles, gated copies, ag (prep.hip, phase C) --
-        if (!REV) {
-            if (FWD) st_tile(reinterpret_cast<T*>(slot + BF.AQK), to_frag<T>(aqk));
-            st_pair2(reinterpret_cast<T*>(slot + BF.AQB), to_frag<T>(aqb[0]), to_frag<T>(aqb[1]));
-        } else {
-            st_pair2(reinterpret_cast<T*>(slot + SB.AQBT), to_frag<T>(aqbT[0]), to_frag<T>(aqbT[1]));
+        // ---- the other wave's parts travel to the lead ------------------------------------------------------------------
+        // tile order in the scratch: A_ab (4), then A_ak (2; the reverse kernel: A_qb^T), A_qb (2), A_qk: as many as the mode forms
+        constexpr int NPART = REV ? 6 : FWD ? 9 : 8;    // A_ab, (A_ak), A_qb or its transpose, (A_qk)
+        if (!lead) {
+            f32x4* const tiles[9] = {&aab[0][0], &aab[0][1], &aab[1][0], &aab[1][1], REV ? &aqbT[0] : &aak[0], REV ? &aqbT[1] : &aak[1],
+                                     &aqb[0], &aqb[1], &aqk};
+#pragma unroll
+            for (int i = 0; i < NPART; ++i) *reinterpret_cast<f32x4*>(sP + (i * 64 + l) * 4) = *tiles[i];
+            if (l == 0) *f_strong = strong;
+            signal_set(f_part, it + 1);
         }
-        // (ag^T waits in the slot where w will go: w = Tm ag is formed further down, when the inverse is there)
-        T* const sWW = reinterpret_cast<T*>(slot + (REV ? SB.W : BF.W));
-#pragma unroll
-        for (int kp = 0; kp < KT2; ++kp) {
-            Frag<T> fagT[2][2], fkgT[2], fbg[2][2], fbgT[2][2], fqg[2], fqgT[2];
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                const int kt = 2 * kp + e;
-                f32x4 gi, ge;
-                decays(kt, gi, ge);
-                const f32x4 gl = bcast16<CH - 1>(gi);
-                const f32x4 egi = exp4<T>(gi), ege = exp4<T>(ge), edn = exp4<T>(gl - gi);
-                fagT[0][e] = transpose(to_frag<T>(to_f32(ra[0][kt]) * ege), ident);
-                fagT[1][e] = transpose(to_frag<T>(to_f32(ra[1][kt]) * ege), ident);
-                fqg[e] = to_frag<T>(to_f32(rq[kt]) * egi * scale);
-                fbg[0][e] = to_frag<T>(to_f32(rb[0][kt]) * edn);
-                fbg[1][e] = to_frag<T>(to_f32(rb[1][kt]) * edn);
-                if (!REV) {
-                    fkgT[e] = transpose(to_frag<T>(to_f32(rk[kt]) * edn), ident);
-                    fbgT[0][e] = transpose(fbg[0][e], ident);
-                    fbgT[1][e] = transpose(fbg[1][e], ident);
-                } else {
-                    fqgT[e] = transpose(fqg[e], ident);
-                }
-                if (c == 0) {
-                    const f32x4 egl = exp4<T>(gl);
-                    *reinterpret_cast<f32x4*>(slot + (REV ? SB.EGL : BF.EGL) + (16 * kt + 4 * g) * 4) = egl;
-                }
-            }
-#pragma unroll
-            for (int s = 0; s < 2; ++s) st_pair2(sWW + (s * KT2 + kp) * PAIR, fagT[s][0], fagT[s][1]);
-            if (!REV) {
-#pragma unroll
-                for (int s = 0; s < 2; ++s) st_pair2(reinterpret_cast<T*>(slot + BF.BGT) + (s * KT2 + kp) * PAIR, fbgT[s][0], fbgT[s][1]);
-                st_pair2(reinterpret_cast<T*>(slot + BF.KGT) + kp * PAIR, fkgT[0], fkgT[1]);
-                st_pair2(reinterpret_cast<T*>(slot + BF.QG) + kp * PAIR, fqg[0], fqg[1]);
-            } else {
-                // the reverse scan takes bg as it is and w transposed (the stand-alone kernel turns the stored tiles on
-                // their way into LDS: the same values)
-#pragma unroll
-                for (int s = 0; s < 2; ++s) st_pair2(reinterpret_cast<T*>(slot + SB.BGT) + (s * KT2 + kp) * PAIR, fbg[s][0], fbg[s][1]);
-                st_pair2(reinterpret_cast<T*>(slot + SB.QGT) + kp * PAIR, fqgT[0], fqgT[1]);
-            }
-        }
-        Frag<T> vT[VT];
+
+        Frag<T> vT[VH];
         if (!REV) {
 #pragma unroll
-            for (int vt = 0; vt < VT; ++vt) {
-                vT[vt] = transpose(rv[vt], ident);
-                st_tile(reinterpret_cast<T*>(slot + L::VTT) + vt * TILE, vT[vt]);
+            for (int j = 0; j < VH; ++j) {
+                vT[j] = transpose(sel(nv[j], rowok), ident);
+                st_tile(reinterpret_cast<T*>(slot + L::VTT) + (vt0 + j) * TILE, vT[j]);
             }
         }
         if (REV || CKPT) {
             // rows past the end of a ragged chunk were taken as zeros
 #pragma unroll
-            for (int vt = 0; vt < VT; ++vt) st_tile(reinterpret_cast<T*>(slot + L::DOT) + vt * TILE, transpose(rdo[vt], ident));
+            for (int j = 0; j < VH; ++j) st_tile(reinterpret_cast<T*>(slot + L::DOT) + (vt0 + j) * TILE, transpose(sel(ndo[j], rowok), ident));
         }
-        const Frag<T> aakf[2] = {to_frag<T>(aak[0]), to_frag<T>(aak[1])};
-        // the inputs are used up: the next chunk's may come
-        __builtin_amdgcn_sched_barrier(0);
-        if (t + FNP < nst) request(t + FNP);
-        __builtin_amdgcn_sched_barrier(0);
 
-        // ---- phase B: (I - A_ab)^-1 by forward substitution (prep.hip, phase B) -------------------------------------
-        {
-            int lb = l;                                   // formed afresh per chunk (see copy_out)
-            asm volatile("" : "+v"(lb));
-            const int r = lb >> 5, col = lb & 31;
-            float x[16], y[16];
+        // ---- the lead: whole score tiles, (I - A_ab)^-1 by forward substitution (prep.hip, phase B) ---------------------
+        Frag<T> tm[2][2], aakf[2];
+        if (lead) {
+            if (!wait_ge(f_part, it + 1, f_abort)) { if (l == 0) *a.err = FUSED_ABORTED + 1; return; }
+            f32x4* const tiles[9] = {&aab[0][0], &aab[0][1], &aab[1][0], &aab[1][1], REV ? &aqbT[0] : &aak[0], REV ? &aqbT[1] : &aak[1],
+                                     &aqb[0], &aqb[1], &aqk};
+            // the lower channel tiles' part first, as a single wave adds them
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const float* nrow = &sN[(16 * r + i) * FLDP];
-                float acc0 = (col == 16 * r + i) ? 1.f : 0.f, acc1 = 0.f;
-#pragma unroll
-                for (int j4 = 0; j4 < (i + 3) / 4; ++j4) {
-                    const f32x4 co = *reinterpret_cast<const f32x4*>(nrow + 16 * r + 4 * j4);
-                    const f32x4 cx = *reinterpret_cast<const f32x4*>(nrow + 16 * (1 - r) + 4 * j4);
-#pragma unroll
-                    for (int jj = 0; jj < 4; ++jj) {
-                        const int j = 4 * j4 + jj;
-                        if (j < i) { acc0 = fmaf(co[jj], x[j], acc0); acc1 = fmaf(cx[jj], y[j], acc1); }
-                    }
-                }
-                x[i] = acc0 + acc1;
-                y[i] = xor32(x[i]);
+            for (int i = 0; i < NPART; ++i) {
+                const f32x4 o = *reinterpret_cast<const f32x4*>(sP + (i * 64 + l) * 4);
+                *tiles[i] = half == 0 ? *tiles[i] + o : o + *tiles[i];
             }
+            if (CKPT && l == 0) p.ws.STRONG[chw] = (strong || *f_strong != 0) ? 1 : 0;
+            // causal masks: lane (g,c) reg i is entry (row c, inner 4g+i)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) sT[(16 * r + i) * FLDP + col] = x[i];
+            for (int i = 0; i < 4; ++i) {
+                const int j = 4 * g + i;
+                const bool le = j <= c, lt = j < c, tle = c <= j;
+                if (!le) { aqk[i] = 0.f; aqb[0][i] = 0.f; aqb[1][i] = 0.f; }
+                if (!lt) { aak[0][i] = 0.f; aak[1][i] = 0.f; aab[0][0][i] = 0.f; aab[0][1][i] = 0.f; aab[1][0][i] = 0.f; aab[1][1][i] = 0.f; }
+                if (!tle) { aqbT[0][i] = 0.f; aqbT[1][i] = 0.f; }
+            }
+            if (!REV) {
+                if (FWD) st_tile(reinterpret_cast<T*>(slot + BF.AQK), to_frag<T>(aqk));
+                st_pair2(reinterpret_cast<T*>(slot + BF.AQB), to_frag<T>(aqb[0]), to_frag<T>(aqb[1]));
+            } else {
+                st_pair2(reinterpret_cast<T*>(slot + SB.AQBT), to_frag<T>(aqbT[0]), to_frag<T>(aqbT[1]));
+            }
+            aakf[0] = to_frag<T>(aak[0]);
+            aakf[1] = to_frag<T>(aak[1]);
+            // (all of the other wave's parts have been read: the scratch may be written)
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int r = 0; r < 2; ++r)
+#pragma unroll
+                for (int s = 0; s < 2; ++s)
+                    *reinterpret_cast<f32x4*>(&sN[(16 * r + c) * FLDP + 16 * s + 4 * g]) = aab[r][s];
+            __builtin_amdgcn_sched_barrier(0);
+            {
+                int lb = l;                               // formed afresh per chunk (see copy_out)
+                asm volatile("" : "+v"(lb));
+                const int r = lb >> 5, col = lb & 31;
+                float x[16], y[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float* nrow = &sN[(16 * r + i) * FLDP];
+                    float acc0 = (col == 16 * r + i) ? 1.f : 0.f, acc1 = 0.f;
+#pragma unroll
+                    for (int j4 = 0; j4 < (i + 3) / 4; ++j4) {
+                        const f32x4 co = *reinterpret_cast<const f32x4*>(nrow + 16 * r + 4 * j4);
+                        const f32x4 cx = *reinterpret_cast<const f32x4*>(nrow + 16 * (1 - r) + 4 * j4);
+#pragma unroll
+                        for (int jj = 0; jj < 4; ++jj) {
+                            const int j = 4 * j4 + jj;
+                            if (j < i) { acc0 = fmaf(co[jj], x[j], acc0); acc1 = fmaf(cx[jj], y[j], acc1); }
+                        }
+                    }
+                    x[i] = acc0 + acc1;
+                    y[i] = xor32(x[i]);
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) sT[(16 * r + i) * FLDP + col] = x[i];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+#pragma unroll
+                for (int s2 = 0; s2 < 2; ++s2)
+                    tm[s][s2] = to_frag<T>(*reinterpret_cast<const f32x4*>(&sT[(16 * s + c) * FLDP + 16 * s2 + 4 * g]));
+            // for the other wave: the inverse's four blocks and A_ak as operand tiles (in A_ab's bytes, which are used up)
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s = 0; s < 2; ++s) st_pair2(sPub + s * PAIR, tm[s][0], tm[s][1]);
+            st_pair2(sPub + 2 * PAIR, aakf[0], aakf[1]);
+            if (CKPT) {
+                // What the checkpoint pass leaves in the workspace for chunk_grad ((I - A_ab)^-1 here, u and where needed w
+                // below) goes there from the consumers, which have no loads to wait for: a store issued here would stand
+                // behind the next chunk's loads in this wave's in-order memory counter.
+                T* tmw = reinterpret_cast<T*>(slot + L::TMB);
+#pragma unroll
+                for (int s = 0; s < 2; ++s) st_pair2(tmw + s * PAIR, transpose(tm[s][0], ident), transpose(tm[s][1], ident));
+            }
+            signal_set(f_inv, it + 1);
+        } else {
+            if (!wait_ge(f_inv, it + 1, f_abort)) { if (l == 0) *a.err = FUSED_ABORTED + 1; return; }
+#pragma unroll
+            for (int s = 0; s < 2; ++s) ld_pair(sPub + s * PAIR, tm[s][0], tm[s][1]);
+            ld_pair(sPub + 2 * PAIR, aakf[0], aakf[1]);
         }
-        __builtin_amdgcn_sched_barrier(0);
-        Frag<T> tm[2][2];
-#pragma unroll
-        for (int s = 0; s < 2; ++s)
-#pragma unroll
-            for (int s2 = 0; s2 < 2; ++s2)
-                tm[s][s2] = to_frag<T>(*reinterpret_cast<const f32x4*>(&sT[(16 * s + c) * FLDP + 16 * s2 + 4 * g]));
-        if (CKPT) {
-            // What the checkpoint pass leaves in the workspace for chunk_grad ((I - A_ab)^-1 here, u and where needed w
-            // below) goes there from the consumers, which have no loads to wait for: a store issued here would stand
-            // behind the next chunk's loads in this wave's in-order memory counter, and the wait for them would be a
-            // wait for it.
-            T* tmw = reinterpret_cast<T*>(slot + L::TMB);
-#pragma unroll
-            for (int s = 0; s < 2; ++s) st_pair2(tmw + s * PAIR, transpose(tm[s][0], ident), transpose(tm[s][1], ident));
-        }
-        // ---- w = Tm ag, in place of ag^T -------------------------------------------------------------------------------
-#pragma unroll
-        for (int kp = 0; kp < KT2; ++kp) {
+        // ---- w = Tm ag for the own channel tiles, in place of ag^T -------------------------------------------------------
+        {
             Frag<T> agT[2][2], fw[2][2];
-            ld_pair(sWW + (0 * KT2 + kp) * PAIR, agT[0][0], agT[0][1]);
-            ld_pair(sWW + (1 * KT2 + kp) * PAIR, agT[1][0], agT[1][1]);
+            ld_pair(sWW + (0 * KT2 + half) * PAIR, agT[0][0], agT[0][1]);
+            ld_pair(sWW + (1 * KT2 + half) * PAIR, agT[1][0], agT[1][1]);
 #pragma unroll
             for (int e = 0; e < 2; ++e)
 #pragma unroll
@@ -502,15 +591,15 @@ __device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem
                 }
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
-                if (!REV) st_pair2(sWW + (s * KT2 + kp) * PAIR, fw[s][0], fw[s][1]);
-                else st_pair2(sWW + (s * KT2 + kp) * PAIR, transpose(fw[s][0], ident), transpose(fw[s][1], ident));
+                if (!REV) st_pair2(sWW + (s * KT2 + half) * PAIR, fw[s][0], fw[s][1]);
+                else st_pair2(sWW + (s * KT2 + half) * PAIR, transpose(fw[s][0], ident), transpose(fw[s][1], ident));
             }
         }
-        // ---- phase D: u = Tm (A_ak v), transposed (prep.hip, phase D) ---------------------------------------------------
+        // ---- u = Tm (A_ak v) for the own value tiles, transposed (prep.hip, phase D) ------------------------------------
         if (!REV) {
 #pragma unroll
-            for (int vt = 0; vt < VT; ++vt) {
-                const Frag<T> mT[2] = {to_frag<T>(mm(vT[vt], aakf[0], zero4())), to_frag<T>(mm(vT[vt], aakf[1], zero4()))};
+            for (int j = 0; j < VH; ++j) {
+                const Frag<T> mT[2] = {to_frag<T>(mm(vT[j], aakf[0], zero4())), to_frag<T>(mm(vT[j], aakf[1], zero4()))};
                 Frag<T> fu[2];
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
@@ -518,14 +607,14 @@ __device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem
                     uT = mm(mT[1], tm[s][1], uT);
                     fu[s] = to_frag<T>(uT);
                 }
-                st_pair2(reinterpret_cast<T*>(slot + L::UT) + vt * PAIR, fu[0], fu[1]);
+                st_pair2(reinterpret_cast<T*>(slot + L::UT) + (vt0 + j) * PAIR, fu[0], fu[1]);
             }
         }
-        signal_set(&flags[pw], it + 1);
+        signal_add(f_ready);
     }
     // the last chunk's rows
     if (FWD && it > 0) {
-        if (!wait_ge(&flags[4 + pw], VT * it, &flags[8])) { if (l == 0) *a.err = FUSED_ABORTED + 1; return; }
+        if (!wait_ge(f_consumed, VT * it, f_abort)) { if (l == 0) *a.err = FUSED_ABORTED + 1; return; }
         copy_out(prev_cid);
     }
 }
@@ -582,7 +671,7 @@ __device__ __forceinline__ void fused_consumer_fwd(const FusedArgs<T>& a, char* 
 
     for (int t = 0; t < nst; ++t) {
         const int pp = t & (FNP - 1), it = t / FNP;
-        if (!wait_ge(&flags[pp], it + 1, &flags[8])) { if (l == 0) *a.err = FUSED_ABORTED + 2; return; }
+        if (!wait_ge(&flags[pp], 2 * (it + 1), &flags[8])) { if (l == 0) *a.err = FUSED_ABORTED + 2; return; }
         const char* slot = smem + pp * L::SLOT;
         const int cid = s0 + t;
         const int64_t chw = (int64_t)h * p.st.nch + cid;
@@ -802,7 +891,7 @@ __device__ __forceinline__ void fused_consumer_rev(const FusedArgs<T>& a, char* 
 
     for (int t = 0; t < nst; ++t) {
         const int pp = t & (FNP - 1), it = t / FNP;
-        if (!wait_ge(&flags[pp], it + 1, &flags[8])) { if (l == 0) *a.err = FUSED_ABORTED + 3; return; }
+        if (!wait_ge(&flags[pp], 2 * (it + 1), &flags[8])) { if (l == 0) *a.err = FUSED_ABORTED + 3; return; }
         const char* slot = smem + pp * L::SLOT;
         const int cid = s1 - 1 - t;
         const int64_t chw = (int64_t)h * p.st.nch + cid;
@@ -861,9 +950,9 @@ __device__ __forceinline__ void fused_consumer_rev(const FusedArgs<T>& a, char* 
 }
 
 // ---- the kernel ------------------------------------------------------------------------------------------------------
-// grid = (H, nseg, N); block = 64 (V/16 + FNP): waves 0 .. V/16-1 consume, the rest produce
+// grid = (H, nseg, N); block = 64 (V/16 + 2 FNP): waves 0 .. V/16-1 consume, the rest produce in pairs
 template <typename T, bool GKF32, int K, int V, int MODE, bool HD>
-__global__ __launch_bounds__(64 * (V / 16 + FNP)) void fused_kernel(FusedArgs<T> a) {
+__global__ __launch_bounds__(64 * (V / 16 + 2 * FNP)) void fused_kernel(FusedArgs<T> a) {
     typedef FusedLds<T, K, V, MODE> L;
     __shared__ __attribute__((aligned(16))) char smem[L::BYTES];
     const int h = blockIdx.x, seg = blockIdx.y;
@@ -874,13 +963,13 @@ __global__ __launch_bounds__(64 * (V / 16 + FNP)) void fused_kernel(FusedArgs<T>
     // an empty segment leaves nothing behind (whoever chains the segments skips it), except that the first one of an
     // empty sequence still passes the state through
     if (s1 <= s0 && seg > 0) return;
-    if (threadIdx.x < 16) reinterpret_cast<int*>(smem + L::FLAGS)[threadIdx.x] = 0;
+    if (threadIdx.x < 32) reinterpret_cast<int*>(smem + L::FLAGS)[threadIdx.x] = 0;
     __syncthreads();
     if (wv < V / 16) {
         if constexpr (MODE == FUSED_REV) fused_consumer_rev<T, K, V>(a, smem, n, h, seg, s0, s1, wv);
         else fused_consumer_fwd<T, K, V, MODE, MODE == FUSED_CKPT && (HD || GKF32)>(a, smem, n, h, seg, s0, s1, wv);
     } else {
-        fused_producer<T, GKF32, K, V, MODE, HD>(a, smem, n, h, seg, s0, s1, wv - V / 16);
+        fused_producer<T, GKF32, K, V, MODE, HD>(a, smem, n, h, seg, s0, s1, (wv - V / 16) >> 1, (wv - V / 16) & 1);
     }
 }
 

