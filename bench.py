@@ -46,7 +46,7 @@ def _args():
     return ap.parse_args()
 
 
-def interface_bytes(kernel, pass_, K, V, es, gs):
+def interface_bytes(kernel, pass_, K, V, es, gs, frac_seg=0.0):
     """Algorithmic HBM bytes of one kernel per (16-token chunk, head): every distinct input read once, every
     output written once (es = bytes per element of the inputs, gs = bytes per element of gk)."""
     W, UT, KGT, BGT, VTT, EGL = 32 * K * es, 32 * V * es, 16 * K * es, 32 * K * es, 16 * V * es, 4 * K
@@ -69,6 +69,18 @@ def interface_bytes(kernel, pass_, K, V, es, gs):
         outs = 2 * 16 * K * es + 16 * K * gs + 2 * 32 * K * es + 16 * V * es
         # (w itself is not read: the kernel rebuilds it from TM and a, for the plain operator with decays in the inputs' type)
         return inputs + 16 * V * es + TM + UT + HC + DHC + DVN + outs
+    # fused route: the scans' operands stay in LDS.  frac_seg = share of the chunks that lie in segments > 0 (their local
+    # output rows, fp32, and the 16 x K block G go through the workspace to the kernel that chains the segments)
+    if kernel == "fused_fwd":
+        return inputs + (1 - frac_seg) * 16 * V * es + frac_seg * (16 * V * 4 + 16 * K * es)
+    if kernel == "fixup":
+        return frac_seg * (16 * V * 4 + 16 * K * es + 16 * V * es)
+    if kernel == "fused_ckpt":
+        return inputs + 16 * V * es + HC + TM + UT
+    if kernel == "fused_sum":
+        return inputs
+    if kernel == "fused_rev":
+        return inputs - 16 * V * es + 16 * V * es + DHC + DVN          # q, k, gk, a, b and do in; dS checkpoint and dv_new out
     raise ValueError(kernel)
 
 
@@ -92,6 +104,19 @@ def algorithmic_bytes(kernel, pass_, K, V, es, gs):
         return C * (5 * K + 5 * V) * es + K * V * es
     if kernel == "scan_pair":
         return 2 * (C * (5 * K + 5 * V) * es + K * V * es)
+    # fused route: a kernel that prepares and scans is priced on the operator's inputs it must read and on what the
+    # algorithm makes it leave behind: the output rows (forward), one state checkpoint per chunk (checkpoint kernel; the
+    # reverse kernel also dv_new); the kernel that chains the segments has no compulsory bytes at all
+    if kernel == "fused_fwd":
+        return C * ((6 * K + 2 * V) * es + K * gs)
+    if kernel == "fused_ckpt":
+        return C * ((6 * K + 2 * V) * es + K * gs) + K * V * es
+    if kernel == "fused_rev":
+        return C * ((6 * K + V) * es + K * gs) + K * V * es + 2 * C * V * es
+    if kernel == "fused_sum":
+        return C * ((6 * K + V) * es + K * gs)
+    if kernel == "fixup":
+        return 0
     raise ValueError(kernel)
 
 
@@ -219,22 +244,31 @@ def time_steps(fn, steps, warmup):
 
 
 def stage_times(inp_dev, dims_kw, pass_, steps, outputs):
-    """Average duration (ms) of each kernel of one pass, events on the current stream around single-stage launches."""
+    """Average duration (ms) of each kernel of one pass, events on the current stream around single-stage launches
+    (hdla_chunk_stages).  Classic route: prep, scans, chunk_grad.  Fused route: the forward kernel and the kernel that
+    chains the segments (pass 0); checkpoint, reverse and chunk_grad kernels (pass 1), and under the name "summary" what a
+    backward pass runs first when the forward pass left no boundary record (not part of the default step)."""
     from hdla_hip import _lib
     lib = _lib.load()
     q, k, v, a, b, gk, h0, do, dht = inp_dev
     dims = _lib.make_dims(**dims_kw)
     ws = _lib.workspace(dims, pass_, q.device)
     P = _lib.ptr
-    names = {1: "prep", 2: "scan_fwd", 6: "scan_pair", 8: "chunk_grad"}
-    masks = [1, 2] if pass_ == 0 else [1, 6, 8]            # the library runs the two backward scans as one launch
+    fused = _lib.workspace_layout(dims, pass_)["ERR"] >= 0
+    if fused:
+        several = lib.hdla_boundary_bytes(ctypes.byref(dims)) > 0
+        names = {2: "fused_fwd", 16: "fixup"} if pass_ == 0 else {16: "summary", 2: "fused_ckpt", 4: "fused_rev", 8: "chunk_grad"}
+        masks = ([2, 16] if several else [2]) if pass_ == 0 else (([16] if several else []) + [2, 4, 8])
+    else:
+        names = {1: "prep", 2: "scan_fwd", 6: "scan_pair", 8: "chunk_grad"}
+        masks = [1, 2] if pass_ == 0 else [1, 6, 8]        # the library runs the two backward scans as one launch
     o, ht, dq, dk, dv, da, db, dgk, dh0 = outputs
     stream = _lib.current_stream(q.device)
     acc = {m: 0.0 for m in masks}
 
     def run(mask):
-        rc = lib.hdla_chunk_stages(ctypes.byref(dims), pass_, mask, P(q), P(k), P(v), P(a), P(b), P(gk), P(h0), P(o),
-                                   P(ht), P(do), P(dht), P(dq), P(dk), P(dv), P(da), P(db), P(dgk), P(dh0), P(ws),
+        rc = lib.hdla_chunk_stages(ctypes.byref(dims), pass_, mask | (1 if fused else 0), P(q), P(k), P(v), P(a), P(b), P(gk),
+                                   P(h0), P(o), P(ht), P(do), P(dht), P(dq), P(dk), P(dv), P(da), P(db), P(dgk), P(dh0), P(ws),
                                    ws.numel(), stream)
         _lib.check(rc, "hdla_chunk_stages")
 
@@ -255,24 +289,41 @@ def stage_times(inp_dev, dims_kw, pass_, steps, outputs):
     return {names[m]: acc[m] / steps for m in masks}
 
 
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline_train():
-    """The CPU oracle (chunk form of the reference's naive.py, fp32, chunk 16, torch on all host cores) on one
-    batch row of configuration 2: forward + autograd backward."""
+    """The CPU oracle (chunk form of the reference's naive.py, fp32, chunk 16, torch on all host cores), forward + autograd
+    backward: one warm-up run and three timed runs (the median is reported) on one batch row of configuration 2 -- every
+    (batch, head) is an independent recurrence, so tokens/s does not depend on the rows taken."""
     from hdla_hip.synthetic import make_config
     from oracle import hrdplr_oracle as O
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
     inp = make_config(2)
-    B_s = inp.q.shape[0]
-    t = [x[:B_s].bfloat16().float().requires_grad_() for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
-    h0 = inp.h0[:B_s].clone().requires_grad_()
-    t0 = time.perf_counter()
-    o, ht = O.chunk_naive(*t, 1.0, h0, chunk_size=16)
-    torch.autograd.grad([o, ht], t + [h0], [inp.do[:B_s], inp.dht[:B_s]])
-    dt = time.perf_counter() - t0
+    B_s = 1
     T = inp.q.shape[1]
-    return {"value": B_s * T / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": f"one run of the whole of configuration 2 (B=4, T=2048, H=16, K=V=64), fp32 chunk-form oracle fwd + autograd bwd, {dt:.1f} s"}
+
+    def run():
+        t = [x[:B_s].bfloat16().float().requires_grad_() for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+        h0 = inp.h0[:B_s].clone().requires_grad_()
+        t0 = time.perf_counter()
+        o, ht = O.chunk_naive(*t, 1.0, h0, chunk_size=16)
+        torch.autograd.grad([o, ht], t + [h0], [inp.do[:B_s], inp.dht[:B_s]])
+        return time.perf_counter() - t0
+    run()
+    times = sorted(run() for _ in range(3))
+    dt = times[1]
+    return {"value": B_s * T / dt, "unit": "tokens/s", "cores": cores, "cpu": cpu_model(), "kind": "port",
+            "sample": f"one batch row of configuration 2 (B=1 of 4, T=2048, H=16, K=V=64), fp32 chunk-form oracle fwd + autograd bwd: "
+                      f"1 warm-up + 3 timed runs, median {dt:.2f} s (min {times[0]:.2f}, max {times[2]:.2f})"}
 
 
 def cpu_baseline_decode():
@@ -287,7 +338,7 @@ def cpu_baseline_decode():
     with torch.no_grad():
         O.recurrence(*t, 1.0, inp.h0, dtype=torch.float32)
     dt = time.perf_counter() - t0
-    return {"value": B_s * steps / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
+    return {"value": B_s * steps / dt, "unit": "tokens/s", "cores": cores, "cpu": cpu_model(), "kind": "port",
             "sample": f"{steps} decode steps of {B_s} of the 256 sequences (H=32, K=V=128), fp32 token recurrence, {dt:.1f} s"}
 
 
@@ -675,6 +726,22 @@ def run_chunk_workload(wl, cfg, steps, warmup, dev, keep_variant=True):
             torch.autograd.grad([o, ht], leaves + [h0], [do, dht])
 
     sec = time_steps(step, steps, warmup)
+    # the same step on the other routes the library has for this shape (reported beside `value`, never as it): strictly
+    # the inputs kept between the passes (the fused route's default hands the states at the time-segment boundaries, 64 KiB
+    # per sequence, head and segment, from the forward to the backward pass; without them the backward pass re-derives
+    # them with one more pass over the inputs), and the classic launch plan (separate prep and scan kernels)
+    variants = {}
+    if keep_variant:
+        from hdla_hip import _lib as _l
+        probe = _l.make_dims(B, T, H, K, V, 2, N, dt, dt, 1.0, cu)
+        if _l.load().hdla_boundary_bytes(ctypes.byref(probe)) > 0 and wl != "fwd":
+            os.environ["HDLA_HIP_INPUTS_ONLY"] = "1"
+            variants["inputs_only"] = time_steps(step, steps, warmup)
+            del os.environ["HDLA_HIP_INPUTS_ONLY"]
+        if _l.workspace_layout(probe, 0)["ERR"] >= 0:
+            os.environ["HDLA_HIP_ROUTE"] = "classic"
+            variants["classic_route"] = time_steps(step, steps, warmup)
+            del os.environ["HDLA_HIP_ROUTE"]
     # the same step with keep_forward=True (an option, off by default: the forward pass's per-chunk intermediates stay
     # alive until the backward pass, which then does not recompute them); `value` is the default route
     sec_keep = time_steps(lambda: step(True), steps, warmup) if wl != "fwd" and keep_variant else None
@@ -692,11 +759,16 @@ def run_chunk_workload(wl, cfg, steps, warmup, dev, keep_variant=True):
         for name, ms in stage_times(raw, dims_kw, pass_, steps, outs).items():
             kern[f"{'fwd' if pass_ == 0 else 'bwd'}.{name}"] = ms
     nchunk_heads = H * sum(-(-int(l) // 16) for l in ([T] * B if cu is None else (cu[1:] - cu[:-1]).tolist()))
+    from hdla_hip import _lib as _l
+    probe = _l.make_dims(B, T, H, K, V, 2, N, dt, dt, 1.0, cu)
+    nseg = max(1, _l.load().hdla_boundary_bytes(ctypes.byref(probe)) // (N * H * K * V * 4))
+    frac_seg = (nseg - 1) / nseg                           # share of the chunks in time segments other than the first
+    summary_ms = kern.pop("bwd.summary", None)             # only a backward pass without a boundary record runs it
     klist = []
     for name, ms in kern.items():
         p_, kn = name.split(".")
         alg = algorithmic_bytes(kn, 0 if p_ == "fwd" else 1, K, V, 2, 2) * nchunk_heads
-        itf = interface_bytes(kn, 0 if p_ == "fwd" else 1, K, V, 2, 2) * nchunk_heads
+        itf = interface_bytes(kn, 0 if p_ == "fwd" else 1, K, V, 2, 2, frac_seg) * nchunk_heads
         klist.append({"kernel": name, "ms": ms, "bytes": alg, "GB/s": alg / (ms * 1e-3) / 1e9,
                       "frac_hbm": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                       "interface_bytes": itf, "frac_interface": itf / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
@@ -708,8 +780,19 @@ def run_chunk_workload(wl, cfg, steps, warmup, dev, keep_variant=True):
                 "instead of recomputing them (more memory held between the passes than the reference's inputs-only contract)",
         "ms_per_step": sec_keep * 1e3, "value": tokens / sec_keep,
         "whole_step_frac_hbm": ((21 * K + 5 * V) * 2) * H * tokens / sec_keep / 1e9 / HBM_PEAK_GBS}}
+    other = {}
+    if "inputs_only" in variants:
+        other["inputs_only"] = {
+            "what": "the same step with HDLA_HIP_INPUTS_ONLY=1: nothing but the inputs kept between the passes; the backward "
+                    "pass re-derives the states at the time-segment boundaries with one more pass (kernel time under summary_ms)",
+            "ms_per_step": variants["inputs_only"] * 1e3, "value": tokens / variants["inputs_only"], "summary_ms": summary_ms}
+    if "classic_route" in variants:
+        other["classic_route"] = {"what": "the same step with HDLA_HIP_ROUTE=classic: prep, scan and chunk_grad kernels with the "
+                                          "scans' operands passed through the workspace",
+                                  "ms_per_step": variants["classic_route"] * 1e3, "value": tokens / variants["classic_route"]}
     return dict(
-        **keep,
+        **keep, **other,
+        route="fused" if any("fused" in x["kernel"] for x in klist) else "classic", time_segments=nseg,
         value=tokens / sec, ms_per_step=sec * 1e3,
         config={"workload": {"train": "config 2: chunked fwd+bwd, B=4 T=2048 H=16 K=V=64, bf16 in, fp32 state, h0/do/dht",
                              "fwd": "config 1: chunked fwd, B=4 T=2048 H=16 K=V=64, bf16 in, fp32 state",

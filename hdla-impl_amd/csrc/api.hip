@@ -263,7 +263,8 @@ int run_chunk(const hdla_dims* d, int pass, const void* q, const void* k, const 
 int run_fused(const hdla_dims* d, bool fwd, const void* q, const void* k, const void* v, const void* a_, const void* b,
               const void* beta, const void* gk, const float* h0, void* o, float* ht, const void* d_o, const float* dht,
               void* dq, void* dk, void* dv, void* da, void* db, void* dbeta, void* dgk, float* dh0, void* boundary,
-              size_t boundary_bytes, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+              size_t boundary_bytes, void* workspace, size_t workspace_bytes, hipStream_t stream,
+              int stages = HDLA_STAGE_ALL) {
     typedef bf16 T;
     FusedLayout L;
     const int rc = make_fused_layout(d, fwd ? HDLA_PASS_FWD : HDLA_PASS_BWD, L);
@@ -298,7 +299,7 @@ int run_fused(const hdla_dims* d, bool fwd, const void* q, const void* k, const 
     f.rseg = reinterpret_cast<float*>(base + L.RSEG);
     f.err = reinterpret_cast<int*>(base + L.ERR);
     hipError_t e;
-    if (d->cu_seqlens) {
+    if (d->cu_seqlens && (stages & HDLA_STAGE_PREP)) {
         e = launch_chunk_table(d->cu_seqlens, d->N, d->T, L.nch, reinterpret_cast<int32_t*>(base + L.CHUNK_OFF),
                                reinterpret_cast<int32_t*>(base + L.CHUNK_SEQ), stream);
         if (e != hipSuccess) return (int)e;
@@ -306,31 +307,40 @@ int run_fused(const hdla_dims* d, bool fwd, const void* q, const void* k, const 
     if (fwd) {
         f.ol = reinterpret_cast<float*>(base + L.OL); f.gw = reinterpret_cast<T*>(base + L.GW);
         f.sin_out = static_cast<float*>(boundary);
-        e = launch_fused<T>(f, d->K, d->V, FUSED_FWD, stream);
-        if (e != hipSuccess) return (int)e;
-        if (L.nseg > 1) {
+        if (stages & HDLA_STAGE_SCAN_FWD) {
+            e = launch_fused<T>(f, d->K, d->V, FUSED_FWD, stream);
+            if (e != hipSuccess) return (int)e;
+        }
+        if (L.nseg > 1 && (stages & HDLA_STAGE_CHAIN)) {
             e = launch_fixup<T>(f, d->K, d->V, stream);
             if (e != hipSuccess) return (int)e;
         }
         return HDLA_OK;
     }
     if (L.nseg > 1 && !boundary) {
-        // inputs only: one pass for the segment records, chained into the states entering the segments
+        // inputs only: one pass for the segment records, chained into the states entering the segments (a caller that
+        // runs the stages one by one may leave this one out once the workspace holds them)
         f.sin_out = reinterpret_cast<float*>(base + L.SIN);
         f.gw = nullptr;
-        e = launch_fused<T>(f, d->K, d->V, FUSED_SUM, stream);
-        if (e != hipSuccess) return (int)e;
-        e = launch_fixup<T>(f, d->K, d->V, stream);
-        if (e != hipSuccess) return (int)e;
+        if (stages & HDLA_STAGE_CHAIN) {
+            e = launch_fused<T>(f, d->K, d->V, FUSED_SUM, stream);
+            if (e != hipSuccess) return (int)e;
+            e = launch_fixup<T>(f, d->K, d->V, stream);
+            if (e != hipSuccess) return (int)e;
+        }
         f.sin = f.sin_out;
     } else {
         f.sin = static_cast<const float*>(boundary);
     }
-    e = launch_fused<T>(f, d->K, d->V, FUSED_CKPT, stream);
-    if (e != hipSuccess) return (int)e;
-    e = launch_fused<T>(f, d->K, d->V, FUSED_REV, stream);
-    if (e != hipSuccess) return (int)e;
-    if (L.nch > 0) {
+    if (stages & HDLA_STAGE_SCAN_FWD) {
+        e = launch_fused<T>(f, d->K, d->V, FUSED_CKPT, stream);
+        if (e != hipSuccess) return (int)e;
+    }
+    if (stages & HDLA_STAGE_SCAN_BWD) {
+        e = launch_fused<T>(f, d->K, d->V, FUSED_REV, stream);
+        if (e != hipSuccess) return (int)e;
+    }
+    if (L.nch > 0 && (stages & HDLA_STAGE_CHUNK_GRAD)) {
         e = launch_chunk_grad<T>(a, d->K, d->V, stream);
         if (e != hipSuccess) return (int)e;
     }
@@ -599,6 +609,12 @@ int hdla_chunk_stages(const hdla_dims* dims, int pass, int stages, const void* q
     if (!q || !k || !v || !a || !b || !gk) return HDLA_ERR_NULL;
     if (pass == 0 ? !o : (!d_o || !dq || !dk || !dv || !da || !db || !dgk)) return HDLA_ERR_NULL;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    bool fused;
+    const int rr = pick_route(dims, fused);
+    if (rr) return rr;
+    if (fused)
+        return run_fused(dims, pass == 0, q, k, v, a, b, nullptr, gk, h0, o, ht, d_o, dht, dq, dk, dv, da, db, nullptr, dgk, dh0,
+                         nullptr, 0, workspace, workspace_bytes, s, stages);
     if (dims->in_dtype == HDLA_BF16)
         return run_chunk<bf16>(dims, pass, q, k, v, a, b, gk, h0, o, ht, d_o, dht, dq, dk, dv, da, db, dgk, dh0,
                                workspace, workspace_bytes, s, stages);

@@ -478,13 +478,13 @@ __device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem
 #pragma unroll
             for (int j = 0; j < VH; ++j) {
                 vT[j] = transpose(sel(nv[j], rowok), ident);
-                st_tile(reinterpret_cast<T*>(slot + L::VTT) + (vt0 + j) * TILE, vT[j]);
+                st_frag(reinterpret_cast<T*>(slot + L::VTT) + (vt0 + j) * TILE + 4 * l, vT[j]);
             }
         }
         if (REV || CKPT) {
             // rows past the end of a ragged chunk were taken as zeros
 #pragma unroll
-            for (int j = 0; j < VH; ++j) st_tile(reinterpret_cast<T*>(slot + L::DOT) + (vt0 + j) * TILE, transpose(sel(ndo[j], rowok), ident));
+            for (int j = 0; j < VH; ++j) st_frag(reinterpret_cast<T*>(slot + L::DOT) + (vt0 + j) * TILE + 4 * l, transpose(sel(ndo[j], rowok), ident));
         }
 
         // ---- the lead: whole score tiles, (I - A_ab)^-1 by forward substitution (prep.hip, phase B) ---------------------
@@ -510,7 +510,7 @@ __device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem
                 if (!tle) { aqbT[0][i] = 0.f; aqbT[1][i] = 0.f; }
             }
             if (!REV) {
-                if (FWD) st_tile(reinterpret_cast<T*>(slot + BF.AQK), to_frag<T>(aqk));
+                if (FWD) st_frag(reinterpret_cast<T*>(slot + BF.AQK) + 4 * l, to_frag<T>(aqk));
                 st_pair2(reinterpret_cast<T*>(slot + BF.AQB), to_frag<T>(aqb[0]), to_frag<T>(aqb[1]));
             } else {
                 st_pair2(reinterpret_cast<T*>(slot + SB.AQBT), to_frag<T>(aqbT[0]), to_frag<T>(aqbT[1]));
@@ -976,108 +976,123 @@ __global__ __launch_bounds__(64 * (V / 16 + 2 * FNP)) void fused_kernel(FusedArg
 // ---- forward pass, second kernel: the true entering states, and their part of the output ----------------------------
 // grid = (H, nseg, N), 256 threads.  blockIdx.y = s in 1 .. nseg-1: segment s (chain the records of segments 0 .. s-1
 // into S_in(s), keep it as the boundary record, add G S_in(s) to the segment's local outputs); blockIdx.y = 0: the
-// final state (all segments chained).  Every wave chains for itself (a few dozen products), so there is no exchange.
+// final state (all segments chained).  Wave j chains column block j of the state (the blocks are independent), the
+// waves exchange their blocks through LDS, and each then takes every fourth chunk of the segment, four chunks' loads in
+// flight at a time.
 template <typename T, int K, int V>
 __global__ __launch_bounds__(256) void fixup_kernel(FusedArgs<T> a) {
-    constexpr int KT = K / 16, VT = V / 16;
+    constexpr int KT = K / 16, VT = V / 16, NB = 4;
+    static_assert(VT == 4, "one column block per wave");
     constexpr int OROW = V * (int)sizeof(T) + 16;
     __shared__ __attribute__((aligned(16))) char stage[4][CH * OROW];
+    __shared__ __attribute__((aligned(16))) T sS[VT * KT * TILE];          // S_in as operand tiles [vt][kt]
     const ChunkArgs<T>& p = a.c;
     const int h = blockIdx.x;
     const int n = p.st.cu ? p.st.order[blockIdx.z] : (int)blockIdx.z;
     const int target = blockIdx.y == 0 ? a.nseg : (int)blockIdx.y;       // chain segments 0 .. target-1
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int l = lane_id(), g = l >> 4, c = l & 15;
-    const int H = p.H;
-    int s0, s1;
+    const int H = p.H, vt = wv;
+    int s0 = 0, s1 = 0;
     if (target < a.nseg) {
         seg_range(p.st, n, a.nseg, target, s0, s1);
         if (s1 <= s0) return;
     } else if (!p.ht) return;
     const int64_t rec0 = ((int64_t)n * H + h) * a.nseg;
+    const int64_t soff = ((int64_t)n * H + h) * K * V + 16 * vt + c;
 
-    // S[vt][kt]: lane (g,c) reg i = S[16kt + 4g + i][16vt + c]
-    f32x4 S[VT][KT];
-#pragma unroll
-    for (int vt = 0; vt < VT; ++vt)
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt) {
-            S[vt][kt] = zero4();
-            if (p.h0) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    S[vt][kt][i] = p.h0[((int64_t)n * H + h) * K * V + (int64_t)(16 * kt + 4 * g + i) * V + 16 * vt + c];
-            }
-        }
-    for (int s = 0; s < target; ++s) {
-        int q0, q1;
-        seg_range(p.st, n, a.nseg, s, q0, q1);
-        if (q1 <= q0) continue;
-        const float* sloc = a.sloc + (rec0 + s) * (K * V);
-        if (s == 0) {
-#pragma unroll
-            for (int vt = 0; vt < VT; ++vt)
-#pragma unroll
-                for (int kt = 0; kt < KT; ++kt) S[vt][kt] = *reinterpret_cast<const f32x4*>(sloc + (vt * KT + kt) * TILE + 4 * l);
-        } else {
-#pragma unroll
-            for (int vt = 0; vt < VT; ++vt) chain_step<T, KT>(S[vt], a.mseg + (rec0 + s) * (K * K), sloc + vt * KT * TILE, TILE, true);
-        }
-    }
-    if (target == a.nseg) {
-        if (wv == 0) {
-#pragma unroll
-            for (int vt = 0; vt < VT; ++vt)
-#pragma unroll
-                for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        p.ht[((int64_t)n * H + h) * K * V + (int64_t)(16 * kt + 4 * g + i) * V + 16 * vt + c] = S[vt][kt][i];
-        }
-        return;
-    }
-    if (wv == 0 && a.sin_out) {
-        float* so = a.sin_out + (rec0 + target) * (K * V);
-#pragma unroll
-        for (int vt = 0; vt < VT; ++vt)
-#pragma unroll
-            for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<f32x4*>(so + (vt * KT + kt) * TILE + 4 * l) = S[vt][kt];
-    }
-    if (!a.gw) return;                                    // chaining only (the backward pass re-deriving the states)
-    Frag<T> Sb[VT][KT];
-#pragma unroll
-    for (int vt = 0; vt < VT; ++vt)
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt) Sb[vt][kt] = to_frag<T>(S[vt][kt]);
+    // the chunks' operands are requested before the chain, whose loads are dependent round trips
     int c0, c1;
     seq_chunks(p.st, n, c0, c1);
     int64_t bos, eos;
     seq_bounds(p.st, n, bos, eos);
+    Frag<T> G[NB][KT];
+    f32x4 OLr[NB][VT];
+    auto request = [&](int first) __attribute__((always_inline)) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const int cid = min(first + 4 * b, s1 - 1);   // past the end: the last chunk again, never used
+            const int64_t chw = (int64_t)h * p.st.nch + cid;
+            const T* gw = a.gw + chw * (CH * K) + c * K + 4 * g;
+            const float* ol = a.ol + chw * (CH * V) + c * V + 4 * g;
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) G[b][kt] = ld_frag(gw + 16 * kt);
+#pragma unroll
+            for (int j = 0; j < VT; ++j) OLr[b][j] = *reinterpret_cast<const f32x4*>(ol + 16 * j);
+        }
+    };
+    const bool outputs = target < a.nseg && a.gw != nullptr;
+    if (outputs) request(s0 + wv);
+
+    // S[kt]: lane (g,c) reg i = S[16kt + 4g + i][16vt + c]
+    f32x4 S[KT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+        S[kt] = zero4();
+        if (p.h0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) S[kt][i] = p.h0[soff + (int64_t)(16 * kt + 4 * g + i) * V];
+        }
+    }
+    for (int s = 0; s < target; ++s) {
+        int q0, q1;
+        seg_range(p.st, n, a.nseg, s, q0, q1);
+        if (q1 <= q0) continue;
+        const float* sloc = a.sloc + (rec0 + s) * (K * V) + vt * KT * TILE;
+        if (s == 0) {
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) S[kt] = *reinterpret_cast<const f32x4*>(sloc + kt * TILE + 4 * l);
+        } else {
+            chain_step<T, KT>(S, a.mseg + (rec0 + s) * (K * K), sloc, TILE, true);
+        }
+    }
+    if (target == a.nseg) {
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) p.ht[soff + (int64_t)(16 * kt + 4 * g + i) * V] = S[kt][i];
+        return;
+    }
+    if (a.sin_out) {
+        float* so = a.sin_out + (rec0 + target) * (K * V) + vt * KT * TILE;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<f32x4*>(so + kt * TILE + 4 * l) = S[kt];
+    }
+    if (!a.gw) return;                                    // chaining only (the backward pass re-deriving the states)
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) st_tile(sS + (vt * KT + kt) * TILE, to_frag<T>(S[kt]));
+    __syncthreads();
+    Frag<T> Sb[VT][KT];
+#pragma unroll
+    for (int j = 0; j < VT; ++j)
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) Sb[j][kt] = ld_tile(sS + (j * KT + kt) * TILE);
     char* const st = stage[wv];
-    for (int cid = s0 + wv; cid < s1; cid += 4) {
-        const int64_t chw = (int64_t)h * p.st.nch + cid;
-        const int64_t tok0 = bos + (int64_t)(cid - c0) * CH;
-        const int len = (int)min((int64_t)CH, eos - tok0);
-        const T* gw = a.gw + chw * (CH * K) + c * K + 4 * g;
-        const float* ol = a.ol + chw * (CH * V) + c * V + 4 * g;
-        Frag<T> G[KT];
+    for (int first = s0 + wv; first < s1; first += 4 * NB) {
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) G[kt] = ld_frag(gw + 16 * kt);
+        for (int b = 0; b < NB; ++b) {
+            const int cid = first + 4 * b;
+            if (cid < s1) {
+                const int64_t tok0 = bos + (int64_t)(cid - c0) * CH;
+                const int len = (int)min((int64_t)CH, eos - tok0);
 #pragma unroll
-        for (int vt = 0; vt < VT; ++vt) {
-            f32x4 o = *reinterpret_cast<const f32x4*>(ol + 16 * vt);
+                for (int j = 0; j < VT; ++j) {
+                    f32x4 o = OLr[b][j];
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt) o = mm(G[kt], Sb[vt][kt], o);
-            st_frag(reinterpret_cast<T*>(st + c * OROW) + 16 * vt + 4 * g, to_frag<T>(o));
+                    for (int kt = 0; kt < KT; ++kt) o = mm(G[b][kt], Sb[j][kt], o);
+                    st_frag(reinterpret_cast<T*>(st + c * OROW) + 16 * j + 4 * g, to_frag<T>(o));
+                }
+                // whole rows, 16 bytes a lane (the wave's own staging area: LDS accesses of one wave complete in order)
+                constexpr int LPR = V * (int)sizeof(T) / 16, RPI = 64 / LPR;
+#pragma unroll
+                for (int r0 = 0; r0 < CH; r0 += RPI) {
+                    const int r = r0 + l / LPR, e = (l % LPR) * 16;
+                    const i32x4 x = *reinterpret_cast<const i32x4*>(st + r * OROW + e);
+                    if (r < len) *reinterpret_cast<i32x4*>(reinterpret_cast<char*>(p.o + ((tok0 + r) * H + h) * V) + e) = x;
+                }
+            }
         }
-        // whole rows, 16 bytes a lane (the wave's own staging area: LDS accesses of one wave complete in order)
-        constexpr int LPR = V * (int)sizeof(T) / 16, RPI = 64 / LPR;
-#pragma unroll
-        for (int r0 = 0; r0 < CH; r0 += RPI) {
-            const int r = r0 + l / LPR, e = (l % LPR) * 16;
-            const i32x4 x = *reinterpret_cast<const i32x4*>(st + r * OROW + e);
-            if (r < len) *reinterpret_cast<i32x4*>(reinterpret_cast<char*>(p.o + ((tok0 + r) * H + h) * V) + e) = x;
-        }
+        if (first + 4 * NB < s1) request(first + 4 * NB);
     }
 }
 

@@ -201,11 +201,16 @@ int hdla_chunk_bwd_kept(const hdla_dims* dims, const void* q, const void* k, con
  * that a caller can bracket each kernel with events on `stream`.  A stage reads what the earlier stages left
  * in the workspace.  Unused tensor arguments of the other pass may be NULL. */
 enum {
-    HDLA_STAGE_PREP = 1,        /* chunk table (with cu_seqlens) + prep kernel */
-    HDLA_STAGE_SCAN_FWD = 2,    /* forward state scan (writes o in pass 0; h and v_new in pass 1) */
+    HDLA_STAGE_PREP = 1,        /* chunk table (with cu_seqlens) + prep kernel (fused route: the table only) */
+    HDLA_STAGE_SCAN_FWD = 2,    /* forward state scan (writes o in pass 0; state checkpoints in pass 1); on the fused route
+                                 * the kernel that prepares and scans (forward kernel in pass 0, checkpoint kernel in pass 1) */
     HDLA_STAGE_SCAN_BWD = 4,    /* reverse state-gradient scan (pass 1 only) */
     HDLA_STAGE_CHUNK_GRAD = 8,  /* per-chunk gradient assembly (pass 1 only) */
-    HDLA_STAGE_ALL = 15
+    HDLA_STAGE_CHAIN = 16,      /* fused route with several segments only.  Pass 0: the kernel that chains the segments and
+                                 * completes the outputs.  Pass 1: what a backward pass without a boundary record runs first
+                                 * (summary kernel + chaining); it leaves the states entering the segments in the workspace,
+                                 * where later calls without this stage find them */
+    HDLA_STAGE_ALL = 31
 };
 int hdla_chunk_stages(const hdla_dims* dims, int pass, int stages, const void* q, const void* k, const void* v,
                       const void* a, const void* b, const void* gk, const float* h0, void* o, float* ht,

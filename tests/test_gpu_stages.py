@@ -22,7 +22,23 @@ TOL = {torch.float32: 5e-6, torch.bfloat16: 1e-2}
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("B,T,H,K,V", [(2, 40, 2, 64, 64), (1, 64, 2, 128, 128), (1, 35, 2, 128, 64), (1, 20, 2, 64, 128)])
-def test_workspace_buffers_backward_pass(B, T, H, K, V, dtype):
+def test_workspace_buffers_backward_pass(B, T, H, K, V, dtype, monkeypatch):
+    monkeypatch.setenv("HDLA_HIP_ROUTE", "classic")       # the buffers below are those of the four-kernel launch plan
+    _backward_buffers(B, T, H, K, V, dtype, None)
+
+
+@pytest.mark.parametrize("segments", [1, 2, 3])
+@pytest.mark.parametrize("B,T,H", [(2, 40, 2), (1, 150, 3)])
+def test_workspace_buffers_backward_pass_fused_route(B, T, H, segments, monkeypatch):
+    """What the fused kernels leave for chunk_grad: u, (I - A_ab)^-1, the states and state gradients entering the chunks
+    and dv_new, in the same tile formats as the classic route (with several time segments the states are the true ones:
+    the checkpoint kernel starts every segment from the chained state)."""
+    monkeypatch.setenv("HDLA_HIP_ROUTE", "fused")
+    monkeypatch.setenv("HDLA_HIP_SEGMENTS", str(segments))
+    _backward_buffers(B, T, H, 64, 64, torch.bfloat16, ("UT", "TM", "HC", "DHC", "DVN"))
+
+
+def _backward_buffers(B, T, H, K, V, dtype, only):
     scale = 0.7
     inp = make_inputs(11, B, T, H, K, V, gk_div=1.0)
     q, k, v, a, b, gk, do = (x.to(dtype).double() for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk, inp.do))
@@ -56,20 +72,20 @@ def test_workspace_buffers_backward_pass(B, T, H, K, V, dtype):
         return t.permute(0, 1, 3, 5, 2, 4).reshape(H, nch, 2, 16, V)
 
     got = {
-        "W": (G.cat_tiles(G.pair_tiles(ws, L["W"], dtype, H, nch, 2, KT, stride=SA), 3), bh(p["w"])),
-        "UT": (G.cat_tiles(G.pair_tiles(ws, L["UT"], dtype, H, nch, VT, 2).transpose(2, 3), 3, transpose=True), bh(p["u"])),
-        "KGT": (G.cat_tiles(G.pair_tiles(ws, L["KGT"], dtype, H, nch, KT, stride=SA), 2, transpose=True), bh(p["kg"])),
-        "BGT": (G.cat_tiles(G.pair_tiles(ws, L["BGT"], dtype, H, nch, 2, KT, stride=SA), 3, transpose=True), bh(p["bg"])),
-        "VTT": (G.cat_tiles(G.tiles(ws, L["VTT"], dtype, H, nch, VT), 2, transpose=True), bh(p["v"])),
-        "EGL": (G.rows(ws, L["EGL"], torch.float32, H, nch, K, stride=SA), bh(torch.exp(p["gl"]))[..., 0, :]),
-        "AQBT": (G.pair_tiles(ws, L["AQBT"], dtype, H, nch, 2, stride=SB), bh(p["Aqb"]).transpose(-1, -2)),
-        "QGT": (G.cat_tiles(G.pair_tiles(ws, L["QGT"], dtype, H, nch, KT, stride=SB), 2, transpose=True), bh(p["qg"])),
-        "TM": (G.pair_tiles(ws, L["TM"], dtype, H, nch, 2, 2), bh(p["Tm"]).transpose(-1, -2)),   # tiles hold the blocks transposed
-        "HC": (state(L["HC"]), bh(f["h"])),
-        "DHC": (state(L["DHC"]), bh(r["dh"])),
-        "DVN": (vnew(L["DVN"]), bh(r["dvn"])),
+        "W": lambda: (G.cat_tiles(G.pair_tiles(ws, L["W"], dtype, H, nch, 2, KT, stride=SA), 3), bh(p["w"])),
+        "UT": lambda: (G.cat_tiles(G.pair_tiles(ws, L["UT"], dtype, H, nch, VT, 2).transpose(2, 3), 3, transpose=True), bh(p["u"])),
+        "KGT": lambda: (G.cat_tiles(G.pair_tiles(ws, L["KGT"], dtype, H, nch, KT, stride=SA), 2, transpose=True), bh(p["kg"])),
+        "BGT": lambda: (G.cat_tiles(G.pair_tiles(ws, L["BGT"], dtype, H, nch, 2, KT, stride=SA), 3, transpose=True), bh(p["bg"])),
+        "VTT": lambda: (G.cat_tiles(G.tiles(ws, L["VTT"], dtype, H, nch, VT), 2, transpose=True), bh(p["v"])),
+        "EGL": lambda: (G.rows(ws, L["EGL"], torch.float32, H, nch, K, stride=SA), bh(torch.exp(p["gl"]))[..., 0, :]),
+        "AQBT": lambda: (G.pair_tiles(ws, L["AQBT"], dtype, H, nch, 2, stride=SB), bh(p["Aqb"]).transpose(-1, -2)),
+        "QGT": lambda: (G.cat_tiles(G.pair_tiles(ws, L["QGT"], dtype, H, nch, KT, stride=SB), 2, transpose=True), bh(p["qg"])),
+        "TM": lambda: (G.pair_tiles(ws, L["TM"], dtype, H, nch, 2, 2), bh(p["Tm"]).transpose(-1, -2)),   # tiles hold the blocks transposed
+        "HC": lambda: (state(L["HC"]), bh(f["h"])),
+        "DHC": lambda: (state(L["DHC"]), bh(r["dh"])),
+        "DVN": lambda: (vnew(L["DVN"]), bh(r["dvn"])),
     }
-    errs = {n: O.rel_l2(x, y) for n, (x, y) in got.items()}
+    errs = {n: O.rel_l2(*xy()) for n, xy in got.items() if only is None or n in only}
     print(dtype, {k: f"{v:.1e}" for k, v in errs.items()}, flush=True)
     assert all(e <= TOL[dtype] for e in errs.values()), errs
 
@@ -83,7 +99,7 @@ def test_workspace_buffers_forward_pass(K, V, dtype):
     _, _, p, f = CS.forward(q, k, v, a, b, gk, scale, inp.h0.double())
     d = lambda x: x.to(dtype).to(DEV).contiguous()
     lib = _lib.load()
-    dims = _lib.make_dims(B, T, H, K, V, 2, B, dtype, dtype, scale, None)
+    dims = _lib.make_dims(B, T, H, K, V, 2, B, dtype, dtype, scale, None, route=_lib.ROUTE_CLASSIC)
     ws = _lib.workspace(dims, 0, DEV)
     t = [d(x) for x in (q, k, v, a, b, gk)] + [inp.h0.float().to(DEV).contiguous()]
     o = torch.empty_like(t[2])

@@ -58,7 +58,7 @@ def test_two_calls_in_a_row_match_the_workspace_entry_point(dtype):
 
 def test_size_limit_and_argument_errors():
     lib = _lib.load()
-    dims, t, h0, _ = _case(33, 4, 2048, 16, 64, 64, torch.bfloat16)      # 168 MB of workspace: beyond the array
+    dims, t, h0, _ = _case(33, 8, 2048, 16, 64, 64, torch.bfloat16)      # 117 MB of workspace or more: beyond the array
     assert lib.hdla_workspace_bytes(ctypes.byref(dims), 0) > STATIC_BYTES
     rc, _, _ = _call(True, dims, t, h0, with_ws=False)
     assert rc == -8 and b"HDLA_STATIC_WORKSPACE_BYTES" in lib.hdla_strerror(rc)
