@@ -217,6 +217,16 @@ struct ChunkPos {
     int n;         // sequence
 };
 
+// A value that is the same on every lane of the wave, moved to scalar registers.  What is read from a table arrives in
+// vector registers even when the index is uniform; addresses formed from it would then be 64-bit vector arithmetic
+// for every access, where a scalar base and a 32-bit lane offset do.
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ int64_t uniform(int64_t x) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)x);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)x >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
 // Token rows [bos, eos) of packed sequence n, forced into 0 <= bos <= eos <= total: the table comes from the caller
 // and is not validated on the device, and no value in it may take an access outside the tensors.
 __device__ __forceinline__ void packed_bounds(const int64_t* cu, int n, int64_t total, int64_t& bos, int64_t& eos) {
@@ -224,6 +234,7 @@ __device__ __forceinline__ void packed_bounds(const int64_t* cu, int n, int64_t 
     eos = min(max(cu[n + 1], bos), total);
 }
 
+// (cid: the same on every lane)
 __device__ __forceinline__ bool locate_chunk(const SeqTab& st, int cid, ChunkPos& cp) {
     if (st.cu == nullptr) {
         if (cid >= st.N * st.NT) return false;
@@ -233,26 +244,30 @@ __device__ __forceinline__ bool locate_chunk(const SeqTab& st, int cid, ChunkPos
         cp.len = min(CH, st.T - ic * CH);
         return true;
     }
-    if (cid >= st.chunk_off[st.N]) return false;
-    cp.n = st.chunk_seq[cid];
-    const int ic = cid - st.chunk_off[cp.n];
+    if (cid >= uniform(st.chunk_off[st.N])) return false;
+    cp.n = uniform(st.chunk_seq[cid]);
+    const int ic = cid - uniform(st.chunk_off[cp.n]);
     int64_t bos, eos;
     packed_bounds(st.cu, cp.n, st.T, bos, eos);
-    cp.tok0 = bos + (int64_t)ic * CH;
-    cp.len = (int)min((int64_t)CH, eos - cp.tok0);
+    cp.tok0 = uniform(bos) + (int64_t)ic * CH;
+    cp.len = (int)min((int64_t)CH, uniform(eos) - cp.tok0);
     return cp.len > 0;
 }
 
-// chunk range [c0, c1) of sequence n
+// chunk range [c0, c1) of sequence n (n: the same on every lane)
 __device__ __forceinline__ void seq_chunks(const SeqTab& st, int n, int& c0, int& c1) {
     if (st.cu == nullptr) { c0 = n * st.NT; c1 = c0 + st.NT; }
-    else { c0 = st.chunk_off[n]; c1 = st.chunk_off[n + 1]; }
+    else { c0 = uniform(st.chunk_off[n]); c1 = uniform(st.chunk_off[n + 1]); }
 }
 
-// token rows [bos, eos) of sequence n on the flattened axis
+// token rows [bos, eos) of sequence n on the flattened axis (n: the same on every lane)
 __device__ __forceinline__ void seq_bounds(const SeqTab& st, int n, int64_t& bos, int64_t& eos) {
     if (st.cu == nullptr) { bos = (int64_t)n * st.T; eos = bos + st.T; }
-    else packed_bounds(st.cu, n, st.T, bos, eos);
+    else {
+        packed_bounds(st.cu, n, st.T, bos, eos);
+        bos = uniform(bos);
+        eos = uniform(eos);
+    }
 }
 
 // ---- per-chunk decay quantities in fragment layout ---------------------------------------------------------
