@@ -289,6 +289,41 @@ def stage_times(inp_dev, dims_kw, pass_, steps, outputs):
     return {names[m]: acc[m] / steps for m in masks}
 
 
+def chunk_table_times(dev, steps=20):
+    """Average duration (microseconds) of the kernel that turns cu_seqlens into the chunk table of a packed batch, for 4,
+    2048 (the most whose start order is ranked) and 65535 (the most the library takes) sequences of 16 tokens, one head:
+    events around launches of that kernel alone (on the fused route stage 1 of hdla_chunk_stages is nothing else)."""
+    from hdla_hip import _lib
+    lib = _lib.load()
+    out = {}
+    for N in (4, 2048, 65535):
+        T, H, K, V = 16 * N, 1, 64, 64
+        cu = (16 * torch.arange(N + 1, dtype=torch.int64)).to(dev)
+        dims = _lib.make_dims(1, T, H, K, V, 2, N, torch.bfloat16, torch.bfloat16, 1.0, cu, route=_lib.ROUTE_FUSED)
+        ws = _lib.workspace(dims, 0, dev)
+        t = [torch.empty(1, T * r, H, K, dtype=torch.bfloat16, device=dev) for r in (1, 1, 1, 2, 2, 1)]
+        o = torch.empty(1, T, H, V, dtype=torch.bfloat16, device=dev)
+        P, stream = _lib.ptr, _lib.current_stream(dev)
+
+        def run():
+            rc = lib.hdla_chunk_stages(ctypes.byref(dims), 0, 1, *[P(x) for x in t], None, P(o), None, *([None] * 9), P(ws),
+                                       ws.numel(), stream)
+            _lib.check(rc, "hdla_chunk_stages")
+        run()
+        torch.cuda.synchronize()
+        tot = 0.0
+        for _ in range(steps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            run()
+            e1.record()
+            torch.cuda.synchronize()
+            tot += e0.elapsed_time(e1)
+        out[f"{N} sequences"] = round(tot / steps * 1e3, 1)
+        del t, o, ws
+    return out
+
+
 def cpu_model():
     try:
         for line in open("/proc/cpuinfo"):
@@ -699,6 +734,7 @@ def main():
                                     "achieved_GB/s": r["roofline"]["achieved"], "traffic": r["roofline"]["traffic"],
                                     "ms_per_launch": r["roofline"]["ms_per_launch"]}
         res["other_configs"] = others
+        res["chunk_table_us"] = chunk_table_times(dev)
     if not args.no_cpu_baseline and wl == "train":
         res["cpu_baseline"] = cpu_baseline_train()
     print(json.dumps(res))

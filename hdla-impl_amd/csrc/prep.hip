@@ -332,45 +332,80 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
 
 // ---- chunk table for packed variable-length batches ----------------------------------------------------------
 constexpr int ORDER_MAX_N = 2048;      // beyond this many sequences they are taken as they come (ranking is quadratic)
-__global__ void build_chunk_table_kernel(const int64_t* cu, int N, int T, int nch, int32_t* chunk_off, int32_t* chunk_seq) {
-    // one workgroup; N is small (number of packed sequences)
-    __shared__ int total;
-    if (threadIdx.x == 0) {
-        int64_t acc = 0;
-        for (int n = 0; n < N; ++n) {
-            // never beyond the slots the workspace has (cannot happen for a non-decreasing table that ends at T)
-            chunk_off[n] = (int)min(acc, (int64_t)nch);
-            int64_t bos, eos;
-            packed_bounds(cu, n, T, bos, eos);
-            acc += (eos - bos + CH - 1) / CH;
-        }
-        total = (int)min(acc, (int64_t)nch);
-        chunk_off[N] = total;
-    }
-    __syncthreads();
-    for (int cid = threadIdx.x; cid < total; cid += blockDim.x) {
-        int lo = 0, hi = N - 1;   // last n with chunk_off[n] <= cid
-        while (lo < hi) {
-            const int mid = (lo + hi + 1) >> 1;
-            if (chunk_off[mid] <= cid) lo = mid; else hi = mid - 1;
-        }
-        chunk_seq[cid] = lo;
-    }
-    // order[r] = the sequence with the r-th most chunks (ties by index): the scans start their workgroups in this
-    // order, so that when there are more workgroups than compute units the long sequences are not the ones that wait
+constexpr int TABLE_THREADS = 256;
+// Workgroup 0 builds the table; with at most ORDER_MAX_N sequences, workgroups 1 .. ceil(N / 256) rank the sequences by
+// their chunk counts, one sequence a thread (they form the counts from cu themselves, so they wait for nobody).
+__global__ __launch_bounds__(TABLE_THREADS) void build_chunk_table_kernel(const int64_t* cu, int N, int T, int nch, int32_t* chunk_off,
+                                                                          int32_t* chunk_seq) {
+    constexpr int LONG_SEQ = 64, LONG_LIST = 512;
+    __shared__ long long strip[2][TABLE_THREADS];
+    __shared__ __attribute__((aligned(16))) int32_t len[ORDER_MAX_N];
+    __shared__ int n_long, long_seq[LONG_LIST], long_c0[LONG_LIST], long_c1[LONG_LIST];
+    const int t = threadIdx.x;
+    auto chunks_of = [&](int n) {
+        int64_t bos, eos;
+        packed_bounds(cu, n, T, bos, eos);
+        return (long long)((eos - bos + CH - 1) / CH);
+    };
     int32_t* order = chunk_off + N + 1;
-    for (int n = threadIdx.x; n < N; n += blockDim.x) {
-        int r = n;
-        if (N <= ORDER_MAX_N) {
-            const int len = chunk_off[n + 1] - chunk_off[n];
-            r = 0;
-            for (int m = 0; m < N; ++m) {
-                const int lm = chunk_off[m + 1] - chunk_off[m];
-                r += (lm > len || (lm == len && m < n)) ? 1 : 0;
-            }
+    if (blockIdx.x > 0) {
+        // order[r] = the sequence with the r-th most chunks (ties by index): the scans start their workgroups in this
+        // order, so that when there are more workgroups than compute units the long sequences are not the ones that
+        // wait.  All counts go to LDS (entries past N hold -1 and rank behind everything); a thread reads them four at
+        // a time against its own.
+        typedef int i32x4 __attribute__((ext_vector_type(4)));
+        for (int n = t; n < ORDER_MAX_N; n += TABLE_THREADS) len[n] = n < N ? (int)min(chunks_of(n), (long long)0x7fffffff) : -1;
+        __syncthreads();
+        const int n = ((int)blockIdx.x - 1) * TABLE_THREADS + t;
+        if (n >= N) return;
+        const int mine = len[n];
+        int r = 0;
+        for (int m = 0; m < N; m += 4) {
+            const i32x4 lm = *reinterpret_cast<const i32x4*>(&len[m]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) r += (lm[j] > mine || (lm[j] == mine && m + j < n)) ? 1 : 0;
         }
         order[r] = n;
+        return;
     }
+    // chunk_off = exclusive prefix sum of the sequences' chunk counts: every thread sums a strip of consecutive
+    // sequences, the strip sums are scanned in LDS, and the strips are walked a second time.
+    const int per = (N + TABLE_THREADS - 1) / TABLE_THREADS;
+    const int n0 = min(t * per, N), n1 = min(n0 + per, N);
+    long long own = 0;
+#pragma unroll 8
+    for (int n = n0; n < n1; ++n) own += chunks_of(n);
+    strip[0][t] = own;
+    if (t == 0) n_long = 0;
+    __syncthreads();
+    int cur = 0;
+    for (int d = 1; d < TABLE_THREADS; d <<= 1) {         // inclusive scan, one doubling step per round
+        strip[cur ^ 1][t] = strip[cur][t] + (t >= d ? strip[cur][t - d] : 0);
+        cur ^= 1;
+        __syncthreads();
+    }
+    // chunk_off, and chunk_seq: a thread writes the entries of its own strip's sequences; sequences of more than
+    // LONG_SEQ chunks are put on a list and written by the whole workgroup afterwards (a thread that finds the list
+    // full writes its own).  Offsets never go beyond the slots the workspace has (cannot happen for a non-decreasing
+    // table that ends at T).
+    long long acc = strip[cur][t] - own;
+    for (int n = n0; n < n1; ++n) {
+        const long long nx = acc + chunks_of(n);
+        const int c0 = (int)min(acc, (long long)nch), c1 = (int)min(nx, (long long)nch);
+        acc = nx;
+        chunk_off[n] = c0;
+        int slot = LONG_LIST;
+        if (c1 - c0 > LONG_SEQ) slot = atomicAdd(&n_long, 1);
+        if (slot < LONG_LIST) { long_seq[slot] = n; long_c0[slot] = c0; long_c1[slot] = c1; }
+        else for (int cid = c0; cid < c1; ++cid) chunk_seq[cid] = n;
+    }
+    if (t == 0) chunk_off[N] = (int)min(strip[cur][TABLE_THREADS - 1], (long long)nch);
+    __syncthreads();
+    const int nl = min(n_long, LONG_LIST);
+    for (int i = 0; i < nl; ++i)
+        for (int cid = long_c0[i] + t; cid < long_c1[i]; cid += TABLE_THREADS) chunk_seq[cid] = long_seq[i];
+    if (N > ORDER_MAX_N)                                  // too many to rank: as they come
+        for (int n = t; n < N; n += TABLE_THREADS) order[n] = n;
 }
 
 template <typename T, int K, int V, bool HD>
@@ -409,7 +444,8 @@ template hipError_t launch_prep<bf16>(const ChunkArgs<bf16>&, int, int, int, hip
 template hipError_t launch_prep<float>(const ChunkArgs<float>&, int, int, int, hipStream_t);
 
 hipError_t launch_chunk_table(const int64_t* cu, int N, int T, int nch, int32_t* chunk_off, int32_t* chunk_seq, hipStream_t stream) {
-    hipLaunchKernelGGL(build_chunk_table_kernel, dim3(1), dim3(256), 0, stream, cu, N, T, nch, chunk_off, chunk_seq);
+    const int rankers = N <= ORDER_MAX_N ? (N + TABLE_THREADS - 1) / TABLE_THREADS : 0;
+    hipLaunchKernelGGL(build_chunk_table_kernel, dim3(1 + rankers), dim3(TABLE_THREADS), 0, stream, cu, N, T, nch, chunk_off, chunk_seq);
     return hipGetLastError();
 }
 

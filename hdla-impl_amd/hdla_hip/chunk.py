@@ -39,7 +39,12 @@ def _native_dim(d: int, sizes=_NATIVE_D) -> int:
     for n in sizes:
         if d <= n:
             return n
-    raise ValueError(f"head dimension {d} is not supported (maximum {sizes[-1]})")
+    hint = ""
+    if sizes[-1] < 256:
+        hint = ("; the chunked operators hold a head's state tile by tile in registers and stop there: for head dimensions "
+                "up to 256 use the token-serial operators fused_recurrent_dplr_delta_rule / "
+                "fused_recurrent_hdla_delta_rule (forward only)")
+    raise ValueError(f"head dimension {d} is not supported (maximum {sizes[-1]}){hint}")
 
 
 def _pad_last(x: Optional[torch.Tensor], d: int) -> Optional[torch.Tensor]:
@@ -257,6 +262,7 @@ def chunk_hrdplr_delta_rule(
                          f"got {tuple(a.shape)} and {tuple(b.shape)}")
     if int(chunk_size) < 1:
         raise ValueError("chunk_size must be positive")
+    _native_dim(K), _native_dim(V)                   # raises for head dimensions beyond the chunked kernels' 128
     if cu_seqlens is not None:
         if B != 1:
             raise ValueError(f"The batch size is expected to be 1 rather than {B} when using `cu_seqlens`."

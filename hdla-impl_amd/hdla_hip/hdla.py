@@ -121,6 +121,7 @@ def chunk_hdla_delta_rule(
         raise ValueError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)} log_f {tuple(log_f.shape)}")
     if beta.shape not in ((B, T, H, 1), (B, T, H)):
         raise ValueError(f"beta must be [B, T, H, 1] or [B, T, H], got {tuple(beta.shape)}")
+    _native_dim(K), _native_dim(V)                   # raises for head dimensions beyond the chunked kernels' 128
     if cu_seqlens is not None:
         if B != 1:
             raise ValueError(f"The batch size is expected to be 1 rather than {B} when using `cu_seqlens`."

@@ -154,6 +154,23 @@ def test_strong_decay_stays_finite_and_within_tolerance(dtype, B, T, H, K, V):
     _compare(_gpu(inp2, dtype, 1.0, cu=cu), _oracle(inp2, dtype, 1.0, cu=cu), dtype, what=f"strong decay, packed {dtype}")
 
 
+def test_config0_against_the_golden_fixture():
+    """Benchmark configuration 0 (B1 T256 H2 K=V=64, fp32, no initial state), the one case the reference itself can
+    run on a CPU: the chunked and the token-serial kernels against the committed fixture tests/golden/config0.npz
+    (every eighth output row and the final state of the float64 recurrence), relative L2 error <= 1e-5."""
+    import os
+    import numpy as np
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "config0.npz"))
+    inp = make_config(0)
+    t = [x.float().to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    want_o, want_h = torch.from_numpy(gold["o_every8"]), torch.from_numpy(gold["final_state"])
+    for name, fn in (("chunked", chunk_hrdplr_delta_rule), ("token-serial", fused_recurrent_dplr_delta_rule)):
+        o, ht = fn(*t, 2, scale=1.0, initial_state=None, output_final_state=True)
+        e_o, e_h = O.rel_l2(o[:, ::8], want_o), O.rel_l2(ht, want_h)
+        print(f"config 0, {name}: o {e_o:.2e} final state {e_h:.2e}", flush=True)
+        assert e_o <= 1e-5 and e_h <= 1e-5, name
+
+
 def test_reference_integrated_test_shape_fp32():
     """Shape and distributions of the reference's end-to-end test (test_integrated.py:9-42): B2 H4 T256 K128 V64
     fp32, scale 1, gk = logsigmoid(randn), random initial state, random do / dht."""

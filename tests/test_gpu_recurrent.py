@@ -94,6 +94,44 @@ def test_decode_steps_config4_full_size_batch_subset():
     assert e_o <= 5e-3 and e_s <= 1e-5
 
 
+def test_decode_config4_full_size_all_1024_carried_steps():
+    """Configuration 4 exactly as it is timed: B256 H32 K=V=128, bf16 inputs, 1024 single-token calls carrying the fp32
+    state.  The inputs are drawn on the GPU in blocks of 64 steps (the whole run's inputs would be 40 GB on the host);
+    the CPU oracle runs all 1024 tokens for two of the 256 sequences."""
+    import torch.nn.functional as F
+    B, H, K, V, steps, blk = 256, 32, 128, 128, 1024, 64
+    sel = [3, 200]
+    g = torch.Generator(device=DEV).manual_seed(4004)
+    rn = lambda *s: torch.randn(*s, generator=g, device=DEV, dtype=torch.float32)
+    S = rn(B, H, K, V) * 0.1
+    S0 = S[sel].cpu()
+    kept = {n: [] for n in ("q", "k", "v", "a", "b", "gk")}
+    outs = []
+    for j in range(steps // blk):
+        q, k, v = F.normalize(rn(B, blk, H, K), dim=-1), F.normalize(rn(B, blk, H, K), dim=-1), rn(B, blk, H, V)
+        b_r = [F.normalize(rn(B, blk, H, K), dim=-1) for _ in range(2)]
+        a_r = [-2.0 * torch.rand(B, blk, H, 1, generator=g, device=DEV) * bb for bb in b_r]
+        a = torch.stack(a_r, dim=2).reshape(B, 2 * blk, H, K)
+        b = torch.stack(b_r, dim=2).reshape(B, 2 * blk, H, K)
+        gk = F.logsigmoid(rn(B, blk, H, K)) / 16
+        t = dict(q=q.bfloat16(), k=k.bfloat16(), v=v.bfloat16(), a=a.bfloat16(), b=b.bfloat16(), gk=gk.bfloat16())
+        for n in kept:
+            kept[n].append(t[n][sel].cpu())
+        for i in range(blk):
+            o, S = fused_recurrent_dplr_delta_rule(t["q"][:, i:i + 1], t["k"][:, i:i + 1], t["v"][:, i:i + 1],
+                                                   t["a"][:, 2 * i:2 * i + 2], t["b"][:, 2 * i:2 * i + 2], t["gk"][:, i:i + 1],
+                                                   2, scale=1.0, initial_state=S, output_final_state=True)
+            outs.append(o[sel])
+        del q, k, v, a, b, gk, t
+    o = torch.cat(outs, 1)
+    assert torch.isfinite(S).all()
+    ref = [torch.cat(kept[n], 1) for n in ("q", "k", "v", "a", "b", "gk")]
+    o_r, S_r = O.recurrence(*ref, 1.0, S0)
+    e_o, e_s = O.rel_l2(o, o_r), O.rel_l2(S[sel], S_r)
+    print(f"cfg4 full size, 1024 carried steps: o {e_o:.2e} state {e_s:.2e}", flush=True)
+    assert e_o <= 5e-3 and e_s <= 1e-5
+
+
 def test_rank_one_and_padded_dims():
     inp = make_inputs(33, 2, 12, 2, 96, 48, R=1)
     t = [x.float().to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
@@ -123,6 +161,18 @@ def test_head_sizes_up_to_256(dtype, tol, K, V):
     a, b = O.parameterize_a_b(beta.to(dtype).double(), k.double(), lf.double())
     o2_r, h2_r = O.recurrence(q, k, v, a.to(dtype), b.to(dtype), lf, 1.0, inp.h0[:1])
     assert O.rel_l2(o2, o2_r) <= tol and O.rel_l2(h2, h2_r) <= min(tol, 1e-5)
+
+
+def test_chunked_operator_refuses_what_only_the_token_serial_one_takes():
+    """Head dimensions above 128: the chunked operator raises a ValueError that names the token-serial operator, and
+    that operator runs the same inputs (checked against the float64 recurrence)."""
+    inp = make_inputs(77, 1, 24, 2, 256, 192)
+    t = [x.bfloat16().to(DEV) for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)]
+    with pytest.raises(ValueError, match="fused_recurrent_dplr_delta_rule"):
+        chunk_hrdplr_delta_rule(*t, 2, scale=1.0, initial_state=inp.h0.to(DEV), output_final_state=True)
+    o, ht = fused_recurrent_dplr_delta_rule(*t, 2, scale=1.0, initial_state=inp.h0.to(DEV), output_final_state=True)
+    o_r, ht_r = O.recurrence(*[x.bfloat16() for x in (inp.q, inp.k, inp.v, inp.a, inp.b, inp.gk)], 1.0, inp.h0)
+    assert O.rel_l2(o, o_r) <= 5e-3 and O.rel_l2(ht, ht_r) <= 5e-3
 
 
 def test_backward_raises():

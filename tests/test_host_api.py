@@ -288,6 +288,20 @@ def test_python_entry_points_validate_like_the_reference():
         chunk_hrdplr_delta_rule(q, k, v, torch.cat([a, a[:, :32]], 1), torch.cat([b, b[:, :32]], 1), gk, 3)
 
 
+def test_chunked_operators_name_the_token_serial_ones_for_head_dimensions_beyond_128():
+    from hdla_hip import chunk_hdla_delta_rule
+    x = make_inputs(4, 1, 16, 1, 256, 64)
+    t = [y.bfloat16() for y in (x.q, x.k, x.v, x.a, x.b, x.gk)]
+    with pytest.raises(ValueError, match="maximum 128.*fused_recurrent_dplr_delta_rule"):
+        chunk_hrdplr_delta_rule(*t, 2)
+    with pytest.raises(ValueError, match="maximum 128"):
+        chunk_hdla_delta_rule(t[0], t[1], t[2], torch.ones(1, 16, 1, 1).bfloat16(), t[5])
+    x = make_inputs(4, 1, 16, 1, 64, 200)
+    t = [y.bfloat16() for y in (x.q, x.k, x.v, x.a, x.b, x.gk)]
+    with pytest.raises(ValueError, match="head dimension 200 is not supported.*fused_recurrent_hdla_delta_rule"):
+        chunk_hrdplr_delta_rule(*t, 2)
+
+
 def test_no_cpu_fallback():
     (q, k, v, a, b, gk), _ = _cpu_args()
     with pytest.raises(_lib.HdlaError, match="GPU only"):
