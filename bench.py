@@ -156,10 +156,18 @@ def measured_traffic(workload, kernel_key, K, V):
     except (OSError, ValueError):
         return None
     pass_, name = kernel_key.split(".") if "." in kernel_key else ("", kernel_key)
+    fused_mode = {"fused_fwd": "0", "summary": "1", "fused_ckpt": "2", "fused_rev": "3"}.get(name)
     for k, rec in table.items():
+        targs = [a.strip() for a in k[k.index("<") + 1:k.rindex(">")].split(",")] if "<" in k else []
+        if fused_mode is not None or name == "fixup":
+            # fused_kernel<T, GKF32, K, V, MODE (0 forward, 1 summary, 2 checkpoint, 3 reverse), HD>, fixup_kernel<T, K, V>
+            if name == "fixup" and k.startswith("fixup_kernel<") and targs[1:3] == [str(K), str(V)]:
+                return rec["hbm_bytes_per_launch"]
+            if fused_mode is not None and k.startswith("fused_kernel<") and targs[2:] == [str(K), str(V), fused_mode, "false"]:
+                return rec["hbm_bytes_per_launch"]
+            continue
         if not k.startswith(name + "_kernel<"):
             continue
-        targs = [a.strip() for a in k[k.index("<") + 1:k.rindex(">")].split(",")]
         # prep<T, GKF32, K, V, MODE (0 forward, 1 backward, 2 kept forward), HD>, scan_fwd<T, K, V, NWC, WRITE_O>, scan_pair<T, K, V, NWC>,
         # chunk_grad<T, GKF32, K, V, HD>, recurrent<T, K, V, BV, HD>
         kv = targs[2:4] if name in ("prep", "chunk_grad") else targs[1:3]
@@ -807,7 +815,8 @@ def run_chunk_workload(wl, cfg, steps, warmup, dev, keep_variant=True):
         itf = interface_bytes(kn, 0 if p_ == "fwd" else 1, K, V, 2, 2, frac_seg) * nchunk_heads
         klist.append({"kernel": name, "ms": ms, "bytes": alg, "GB/s": alg / (ms * 1e-3) / 1e9,
                       "frac_hbm": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                      "interface_bytes": itf, "frac_interface": itf / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
+                      "interface_bytes": itf, "frac_interface": itf / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                      "traffic": measured_traffic(wl, name, K, V)})
     dom = max(klist, key=lambda x: x["ms"])
     per_tok_head = ((7 * K + 2 * V) * 2) if wl == "fwd" else ((21 * K + 5 * V) * 2)   # compulsory bytes per (token, head)
     whole = per_tok_head * H * tokens

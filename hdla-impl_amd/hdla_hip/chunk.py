@@ -114,12 +114,14 @@ def chunk_hrdplr_bwd_kept(q, k, v, a, b, gk, scale, initial_state, do, dht, kept
     with torch.cuda.device(q.device):
         dims = _dims(q, v, gk, scale, cu_seqlens, N)
         ws = _lib.workspace(dims, _lib.PASS_BWD_KEPT, q.device)
-        dq, dk, dv, dgk = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.empty_like(gk)
+        # rows outside every sequence of a packed batch stay unwritten: they must not carry garbage upstream
+        new = torch.zeros_like if cu_seqlens is not None else torch.empty_like
+        dq, dk, dv, dgk = new(q), new(k), new(v), new(gk)
         da = db = dbeta = None
         if beta is None:
-            da, db = torch.empty_like(a), torch.empty_like(b)
+            da, db = new(a), new(b)
         else:
-            dbeta = torch.empty_like(beta)
+            dbeta = new(beta)
         dh0 = torch.empty(N, H, K, V, dtype=torch.float32, device=q.device) if want_dh0 else None
         rc = lib.hdla_chunk_bwd_kept(ctypes.byref(dims), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(a), _lib.ptr(b),
                                      _lib.ptr(beta), _lib.ptr(gk), _lib.ptr(initial_state), _lib.ptr(do), _lib.ptr(dht),

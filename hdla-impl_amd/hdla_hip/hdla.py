@@ -221,7 +221,7 @@ def fused_recurrent_hdla_delta_rule(
         dims = _dims(q, v, gk, scale, cu_seqlens, N)
         h0 = None if h0 is None else h0.contiguous()
         ht = torch.empty(N, H, Kn, Vn, dtype=torch.float32, device=q.device) if output_final_state else None
-        o = torch.empty_like(v)
+        o = torch.zeros_like(v) if cu_seqlens is not None else torch.empty_like(v)     # rows of no sequence stay zero
         rc = lib.hdla_param_recurrent_fwd(ctypes.byref(dims), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(beta),
                                           _lib.ptr(gk), int(bool(reverse)), _lib.ptr(h0), _lib.ptr(o), _lib.ptr(ht),
                                           _lib.current_stream(q.device))

@@ -35,7 +35,7 @@ def fused_recurrent_dplr_delta_rule_fwd(q, k, v, a, b, gk, rank_ab, scale=1.0, i
         dims = _lib.make_dims(B, T, H, K, V, 2, N, q.dtype, gk.dtype, scale, cu_seqlens)
         h0 = None if initial_state is None else initial_state.to(torch.float32).contiguous()
         ht = q.new_empty(N, H, K, V, dtype=torch.float32) if output_final_state else None
-        o = torch.empty_like(v)
+        o = torch.zeros_like(v) if cu_seqlens is not None else torch.empty_like(v)     # rows of no sequence stay zero
         rc = lib.hdla_recurrent_fwd(ctypes.byref(dims), _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(a), _lib.ptr(b),
                                     _lib.ptr(gk), int(bool(reverse)), _lib.ptr(h0), _lib.ptr(o), _lib.ptr(ht),
                                     _lib.current_stream(q.device))
