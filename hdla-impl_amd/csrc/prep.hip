@@ -64,7 +64,6 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
     f32x4 gi[KTW], ge[KTW];
     f32x4 aqk = zero4(), aqb[2] = {zero4(), zero4()}, aak[2] = {zero4(), zero4()};
     f32x4 aab[2][2] = {{zero4(), zero4()}, {zero4(), zero4()}};
-    f32x4 aqbT[2] = {zero4(), zero4()};
     // the inputs of the chunk stay in registers (as loaded) for the second use in phase C: the working set of the
     // resident waves is larger than the L2, so a second load would come from HBM again
     Frag<T> rq[KTW], rk[KTW], ra[2][KTW], rb[2][KTW];       // own channel tiles; index kt below is local, kt0 + kt global
@@ -127,7 +126,6 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
         for (int s = 0; s < 2; ++s) {
             aqb[s] = mm3(qh, bh[s], aqb[s]);
             aak[s] = mm3(ah[s], kh, aak[s]);
-            if (BWD) aqbT[s] = mm3(bh[s], qh, aqbT[s]);
 #pragma unroll
             for (int r = 0; r < 2; ++r) aab[r][s] = mm3(ah[r], bh[s], aab[r][s]);
         }
@@ -145,7 +143,7 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
         aqk = zero4();
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            aqb[s] = zero4(); aak[s] = zero4(); aqbT[s] = zero4(); aab[0][s] = zero4(); aab[1][s] = zero4();
+            aqb[s] = zero4(); aak[s] = zero4(); aab[0][s] = zero4(); aab[1][s] = zero4();
         }
 #pragma unroll 1
         for (int ps = 0; ps < DecayPass::COUNT; ++ps) {
@@ -168,7 +166,6 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
                 for (int s = 0; s < 2; ++s) {
                     split(to_f32(rb[s][kt]) * ek, bh[s]);
                     aqb[s] = mm3(qh, bh[s], aqb[s]);
-                    if (BWD) aqbT[s] = mm3(bh[s], qh, aqbT[s]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
 #pragma unroll
@@ -186,7 +183,7 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
     if (NWP > 1) {
         // sums over all channels: every wave leaves its parts in LDS and adds the others'
         f32x4* const tiles[9] = {&aak[0], &aak[1], &aab[0][0], &aab[0][1], &aab[1][0], &aab[1][1],
-                                 BWD ? &aqbT[0] : &aqb[0], BWD ? &aqbT[1] : &aqb[1], &aqk};
+                                 &aqb[0], &aqb[1], &aqk};
 #pragma unroll
         for (int i = 0; i < NPART; ++i) *reinterpret_cast<f32x4*>(&sPart[((w * NPART + i) * 64 + l) * 4]) = *tiles[i];
         __syncthreads();
@@ -206,19 +203,18 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int j = 4 * g + i;
-        const bool le = j <= c, lt = j < c, tle = c <= j;
+        const bool le = j <= c, lt = j < c;
         if (!le) { aqk[i] = 0.f; aqb[0][i] = 0.f; aqb[1][i] = 0.f; }
         if (!lt) { aak[0][i] = 0.f; aak[1][i] = 0.f; aab[0][0][i] = 0.f; aab[0][1][i] = 0.f; aab[1][0][i] = 0.f; aab[1][1][i] = 0.f; }
-        if (!tle) { aqbT[0][i] = 0.f; aqbT[1][i] = 0.f; }
     }
     if (w == 0) {
         if (!BWD) {
             st_tile(p.ws.AQK + chw * SAS, to_frag<T>(aqk));
             st_pair2(p.ws.AQB + chw * SAS, to_frag<T>(aqb[0]), to_frag<T>(aqb[1]));
         }
-        if (BWD) st_pair2(p.ws.AQBT + chw * SBS, to_frag<T>(aqbT[0]), to_frag<T>(aqbT[1]));
-        else if (WB) {
-            // both orientations wanted: the second is the first turned (a product with the identity: exact)
+        if (BWD || WB) {
+            // the other orientation is the rounded tile turned (a product with the identity: exact), in every mode, so
+            // that a backward pass finds the same bytes whether it recomputes them or reads what a forward pass kept
             const Frag<T> id = ident_frag<T>();
             st_pair2(p.ws.AQBT + chw * SBS, transpose(to_frag<T>(aqb[0]), id), transpose(to_frag<T>(aqb[1]), id));
         }
