@@ -36,7 +36,8 @@ int check_dims(const hdla_dims* d, int max_dim = 128) {
 }
 
 // ---- the fused route (fused_impl.cuh) ----------------------------------------------------------------------------
-constexpr int FUSED_MAX_SEGMENTS = 8;        // the segments are chained serially by every workgroup that needs them
+constexpr int FUSED_MAX_SEGMENTS = 64;       // the segments are chained serially by every workgroup that needs them: about a
+                                             // microsecond a segment, against 2.5 for every chunk a segment is shorter
 constexpr int FUSED_MIN_SEGMENT_CHUNKS = 8;  // a segment pays for its transition matrix: not worth it for a few chunks
 constexpr int FUSED_TARGET_WORKGROUPS = 256; // one workgroup per compute unit
 

@@ -80,7 +80,7 @@ typedef struct hdla_dims {
     float scale;               /* applied to q (HRDPLR/hrdplr.py:302) */
     const int64_t* cu_seqlens; /* DEVICE int64[N+1] cumulative sequence starts on the T axis, or NULL */
     int32_t route;             /* HDLA_ROUTE_*; 0 = the library chooses */
-    int32_t segments;          /* fused route: time segments per sequence (at most 8); 0 = the library chooses */
+    int32_t segments;          /* fused route: time segments per sequence (at most 64); 0 = the library chooses */
 } hdla_dims;
 
 /* Byte offsets of the named intermediates inside the workspace (0 = not part of this pass); for tests and

@@ -98,6 +98,23 @@ def test_forward_segments_against_classic_route_and_recurrence(B, T, H, segments
     assert r_o <= 5e-3 and r_h <= 5e-3
 
 
+@pytest.mark.parametrize("segments", [16, 37, 64])
+def test_many_segments_forward_and_backward(segments):
+    """Long sequences of few heads are cut into up to 64 segments (here: 2 x 3 (sequence, head) pairs, 125 chunks, so
+    that 64 segments hold one or two chunks each): both passes against the classic route, with the boundary record and
+    without."""
+    x = _dev(make_inputs(27, 2, 2000, 3, 64, 64, gk_div=8.0))
+    o_c, ht_c, _ = forward(x, _lib.ROUTE_CLASSIC, 0)
+    o_f, ht_f, bnd = forward(x, _lib.ROUTE_FUSED, segments, boundary=True)
+    assert O.rel_l2(o_f, o_c) <= 3e-3 and O.rel_l2(ht_f, ht_c) <= 3e-3
+    g_c = backward(x, _lib.ROUTE_CLASSIC, 0)
+    for b in (bnd, None):
+        g_f = backward(x, _lib.ROUTE_FUSED, segments, bnd=b)
+        errs = {n: O.rel_l2(g_f[n], g_c[n]) for n in g_c}
+        print(f"segments {segments} kept {b is not None}:", {k: f"{v:.1e}" for k, v in errs.items()}, flush=True)
+        assert all(e <= 6e-3 for e in errs.values()), errs
+
+
 def test_forward_packed_sequences_and_no_initial_state():
     cu = torch.tensor([0, 37, 37, 500, 516, 1200], dtype=torch.int64)
     inp = make_inputs(23, 1, 1200, 2, 64, 64, gk_div=4.0, n_states=5)

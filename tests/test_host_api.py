@@ -95,7 +95,7 @@ def test_routes_workspaces_and_boundary_records():
     # boundary record: one fp32 K x V state per (sequence, head, segment); none for one segment or the classic route
     assert B(classic) == 0 and B(_dims(segments=1)) == 0
     assert B(_dims(segments=4)) == 2 * 2 * 4 * 64 * 64 * 4
-    assert B(_dims(segments=100)) == 2 * 2 * 8 * 64 * 64 * 4                     # capped
+    assert B(_dims(segments=100)) == 2 * 2 * 64 * 64 * 64 * 4                    # capped at 64 segments
     # chosen by the library: enough segments to give every compute unit a workgroup, never segments of a few chunks
     assert B(_dims(B=4, N=4, T=2048, H=16)) == 4 * 16 * 4 * 64 * 64 * 4
     assert B(_dims(B=64, N=64, T=2048, H=16)) == 0 and B(_dims(T=64)) == 0
