@@ -5,8 +5,9 @@
 //
 // Work division.  A workgroup owns one (sequence, head, time segment): the chunks of a sequence are cut into `nseg`
 // consecutive segments so that few (sequence, head) pairs still fill the device.  It has
-//   * FNP = 4 producer waves.  Producer p prepares the chunks p, p+4, ... of the segment, each entirely by itself (one
-//     wave holds all 64 channels), and leaves the operands in LDS slot p;
+//   * FNP = 4 pairs of producer waves.  Pair p prepares the chunks p, p+4, ... of the segment and leaves the operands in
+//     LDS slot p.  The two waves of a pair take two of the four channel tiles and half of the value tiles each; one of
+//     them (the pair's lead) also adds up the two waves' parts of the score tiles and solves for (I - A_ab)^-1;
 //   * V/16 consumer waves.  Consumer j owns column block j of the fp32 state for the whole segment, in registers, and
 //     walks the chunks in order, exactly as the stand-alone scan kernels do.
 // A segment other than the first does not know the state that enters it.  The state leaving a chunk is affine in the
@@ -21,7 +22,8 @@
 //                   chain themselves before they start.
 //
 // Synchronisation.  Producers and consumers run at their own pace; a slot is handed over through two counters in LDS
-// that only ever grow: ready[p] (chunks producer p has completed) and consumed[p] (consumer-steps finished on slot p).
+// that only ever grow: ready[p] (+1 per wave of pair p and chunk completed) and consumed[p] (consumer-steps finished on
+// slot p); the waves of a pair hand each other the parts and the inverse the same way (part[p], inv[p]).
 // Waiting is polling with s_sleep; every wait is bounded (FUSED_SPIN_LIMIT polls), and a wave that runs into the bound
 // raises an abort flag that ends every other wave's waits as well and is reported through FusedArgs::err, so the grid
 // always drains.  There are no workgroup barriers after the first.
@@ -525,15 +527,22 @@ __device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem
                 for (int s = 0; s < 2; ++s)
                     *reinterpret_cast<f32x4*>(&sN[(16 * r + c) * FLDP + 16 * s + 4 * g]) = aab[r][s];
             __builtin_amdgcn_sched_barrier(0);
+            // The system in token halves, L = tokens 0..7 and H = 8..15 (both ranks: 16 rows each):
+            //   (I - A)^-1 = [[T_LL, 0], [T_HL, T_HH]],  T_LL = (I - A_LL)^-1,  T_HH = (I - A_HH)^-1,  T_HL = T_HH A_HL T_LL.
+            // The two diagonal blocks are independent eight-step substitutions that run side by side on the lanes (a
+            // quarter of the dependent multiply-adds of one sixteen-step substitution); the block below the diagonal is
+            // two 16 x 16 x 16 products, in split operands like the score products (the error of fp32 products).
             {
                 int lb = l;                               // formed afresh per chunk (see copy_out)
                 asm volatile("" : "+v"(lb));
-                const int r = lb >> 5, col = lb & 31;
-                float x[16], y[16];
+                // lane: rank of the rows r, token half hf, column (rank sc, token jc of the same half)
+                const int r = lb >> 5, hf = (lb >> 4) & 1, sc = (lb >> 3) & 1, jc = lb & 7;
+                const int col = 16 * sc + 8 * hf + jc;
+                float x[8], y[8];
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const float* nrow = &sN[(16 * r + i) * FLDP];
-                    float acc0 = (col == 16 * r + i) ? 1.f : 0.f, acc1 = 0.f;
+                for (int i = 0; i < 8; ++i) {
+                    const float* nrow = &sN[(16 * r + 8 * hf + i) * FLDP + 8 * hf];
+                    float acc0 = (sc == r && jc == i) ? 1.f : 0.f, acc1 = 0.f;
 #pragma unroll
                     for (int j4 = 0; j4 < (i + 3) / 4; ++j4) {
                         const f32x4 co = *reinterpret_cast<const f32x4*>(nrow + 16 * r + 4 * j4);
@@ -548,7 +557,29 @@ __device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem
                     y[i] = xor32(x[i]);
                 }
 #pragma unroll
-                for (int i = 0; i < 16; ++i) sT[(16 * r + i) * FLDP + col] = x[i];
+                for (int i = 0; i < 8; ++i) {
+                    sT[(16 * r + 8 * hf + i) * FLDP + col] = x[i];
+                    // the block above the diagonal (rows of L, columns of H) is zero: the lanes of L write it
+                    if (hf == 0) sT[(16 * r + i) * FLDP + col + 8] = 0.f;
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            {
+                // 16 x 16 matrices in (rank, token of the half) order: row c = 8 rank + token, inner 4g .. 4g+3 likewise
+                const int rr = c >> 3, ii = c & 7, ss = g >> 1, j0 = 4 * (g & 1);
+                const f32x4 ahl = *reinterpret_cast<const f32x4*>(&sN[(16 * rr + 8 + ii) * FLDP + 16 * ss + j0]);
+                const f32x4 thh = *reinterpret_cast<const f32x4*>(&sT[(16 * rr + 8 + ii) * FLDP + 16 * ss + 8 + j0]);
+                f32x4 tllT;                               // T_LL^T: row c is column c of T_LL
+#pragma unroll
+                for (int e = 0; e < 4; ++e) tllT[e] = sT[(16 * ss + j0 + e) * FLDP + 16 * rr + ii];
+                Split<T> pa, pb;
+                split(tllT, pa);
+                split(ahl, pb);
+                const f32x4 xT = mm3(pa, pb, zero4());    // (A_HL T_LL)^T = T_LL^T A_HL^T
+                split(thh, pa);
+                split(xT, pb);
+                const f32x4 thl = mm3(pa, pb, zero4());   // T_HH (A_HL T_LL)
+                *reinterpret_cast<f32x4*>(&sT[(16 * rr + 8 + ii) * FLDP + 16 * ss + j0]) = thl;
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
