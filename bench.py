@@ -67,8 +67,9 @@ def interface_bytes(kernel, pass_, K, V, es, gs, frac_seg=0.0):
         return interface_bytes("scan_fwd", 1, K, V, es, gs) + interface_bytes("scan_bwd", 1, K, V, es, gs) - (W + BGT + EGL)
     if kernel == "chunk_grad":
         outs = 2 * 16 * K * es + 16 * K * gs + 2 * 32 * K * es + 16 * V * es
-        # (w itself is not read: the kernel rebuilds it from TM and a, for the plain operator with decays in the inputs' type)
-        return inputs + 16 * V * es + TM + UT + HC + DHC + DVN + outs
+        # (w and u themselves are not read: the kernel rebuilds them from TM, a and v, for the plain operator with decays in
+        # the inputs' type)
+        return inputs + 16 * V * es + TM + HC + DHC + DVN + outs
     # fused route: the scans' operands stay in LDS.  frac_seg = share of the chunks that lie in segments > 0 (their local
     # output rows, fp32, and the 16 x K block G go through the workspace to the kernel that chains the segments)
     if kernel == "fused_fwd":
@@ -76,7 +77,7 @@ def interface_bytes(kernel, pass_, K, V, es, gs, frac_seg=0.0):
     if kernel == "fixup":
         return frac_seg * (16 * V * 4 + 16 * K * es + 16 * V * es)
     if kernel == "fused_ckpt":
-        return inputs + 16 * V * es + HC + TM + UT
+        return inputs + 16 * V * es + HC + TM
     if kernel == "fused_sum":
         return inputs
     if kernel == "fused_rev":

@@ -755,9 +755,9 @@ __device__ __forceinline__ void fused_consumer_fwd(const FusedArgs<T>& a, char* 
             T* hc = p.ws.HC + chw * (K * V) + vt * PAIR;
 #pragma unroll
             for (int kp = 0; kp < KT2; ++kp) st_pair2(hc + kp * (VT * PAIR), sb[2 * kp], sb[2 * kp + 1]);
-            // the producer's results that chunk_grad reads: this wave's tiles of u, and between the waves the two tile
-            // pairs of (I - A_ab)^-1 and (where wanted) the 2 KT/2 pairs of w
-            st_pair2(p.ws.UT + (chw * VT + vt) * PAIR, ut[0], ut[1]);
+            // the producer's results that chunk_grad reads: between the waves the two tile pairs of (I - A_ab)^-1 and,
+            // where chunk_grad does not rebuild them, this wave's tiles of u and the 2 KT/2 pairs of w
+            if (W_GLOBAL) st_pair2(p.ws.UT + (chw * VT + vt) * PAIR, ut[0], ut[1]);
             if (wv < 2) {
                 Frag<T> t0, t1;
                 ld_pair(reinterpret_cast<const T*>(slot + L::TMB) + wv * PAIR, t0, t1);

@@ -30,12 +30,12 @@ def test_workspace_buffers_backward_pass(B, T, H, K, V, dtype, monkeypatch):
 @pytest.mark.parametrize("segments", [1, 2, 3])
 @pytest.mark.parametrize("B,T,H", [(2, 40, 2), (1, 150, 3)])
 def test_workspace_buffers_backward_pass_fused_route(B, T, H, segments, monkeypatch):
-    """What the fused kernels leave for chunk_grad: u, (I - A_ab)^-1, the states and state gradients entering the chunks
-    and dv_new, in the same tile formats as the classic route (with several time segments the states are the true ones:
-    the checkpoint kernel starts every segment from the chained state)."""
+    """What the fused kernels leave for chunk_grad: (I - A_ab)^-1, the states and state gradients entering the chunks and
+    dv_new, in the same tile formats as the classic route (with several time segments the states are the true ones: the
+    checkpoint kernel starts every segment from the chained state).  u is not among them: chunk_grad rebuilds it."""
     monkeypatch.setenv("HDLA_HIP_ROUTE", "fused")
     monkeypatch.setenv("HDLA_HIP_SEGMENTS", str(segments))
-    _backward_buffers(B, T, H, 64, 64, torch.bfloat16, ("UT", "TM", "HC", "DHC", "DVN"))
+    _backward_buffers(B, T, H, 64, 64, torch.bfloat16, ("TM", "HC", "DHC", "DVN"))
 
 
 def _backward_buffers(B, T, H, K, V, dtype, only):
