@@ -226,17 +226,22 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
             *reinterpret_cast<f32x4*>(&sN[(16 * r + c) * LDP + 16 * s + 4 * g]) = aab[r][s];
     __syncthreads();
 
-    // ---- phase B: (I - A_ab)^-1 by forward substitution over tokens, in registers -----------------------------
-    // Lane (r, col) builds column `col` of the rows (r, i), i = 0..15, one token per step; the entries of the
-    // other rank's rows come from the lane 32 positions away.  The coefficients N[(r,i)][*] are uniform per
-    // half-wave (LDS broadcast reads, off the dependency chain); entries with j >= i are zero by the mask.
+    // ---- phase B: (I - A_ab)^-1 -----------------------------------------------------------------------------------
+    // In token halves, L = tokens 0..7 and H = 8..15 (both ranks: 16 rows each):
+    //   (I - A)^-1 = [[T_LL, 0], [T_HL, T_HH]],  T_LL = (I - A_LL)^-1,  T_HH = (I - A_HH)^-1,  T_HL = T_HH A_HL T_LL.
+    // The diagonal blocks by forward substitution over tokens, in registers, both at once: lane (r, half, column) builds
+    // one column of the rows (r, i) of its half, one token per step, the entries of the other rank's rows coming from the
+    // lane 32 positions away (eight steps and a quarter of the dependent multiply-adds of one substitution over all
+    // sixteen tokens).  The block below the diagonal is two 16 x 16 x 16 products, in split operands like the score
+    // products for 2-byte elements (the error of fp32 products), in fp32 products otherwise.
     {
-        const int r = l >> 5, col = l & 31;
-        float x[16], y[16];                      // own rows (r, j) and the partner's rows (1-r, j) of column col
+        const int r = l >> 5, hf = (l >> 4) & 1, sc = (l >> 3) & 1, jc = l & 7;
+        const int col = 16 * sc + 8 * hf + jc;
+        float x[8], y[8];                        // own rows (r, j) and the partner's rows (1-r, j) of column col
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const float* nrow = &sN[(16 * r + i) * LDP];
-            float acc0 = (col == 16 * r + i) ? 1.f : 0.f, acc1 = 0.f;
+        for (int i = 0; i < 8; ++i) {
+            const float* nrow = &sN[(16 * r + 8 * hf + i) * LDP + 8 * hf];
+            float acc0 = (sc == r && jc == i) ? 1.f : 0.f, acc1 = 0.f;
 #pragma unroll
             for (int j4 = 0; j4 < (i + 3) / 4; ++j4) {
                 const f32x4 co = *reinterpret_cast<const f32x4*>(nrow + 16 * r + 4 * j4);         // own rank block
@@ -251,7 +256,26 @@ __global__ __launch_bounds__(K) __attribute__((amdgpu_waves_per_eu(2, 2))) void 
             y[i] = xor32(x[i]);
         }
 #pragma unroll
-        for (int i = 0; i < 16; ++i) sT[(16 * r + i) * LDP + col] = x[i];
+        for (int i = 0; i < 8; ++i) {
+            sT[(16 * r + 8 * hf + i) * LDP + col] = x[i];
+            if (hf == 0) sT[(16 * r + i) * LDP + col + 8] = 0.f;      // rows of L, columns of H: zero
+        }
+        // (the wave reads below what its other lanes wrote above: LDS accesses of one wave complete in order)
+        // 16 x 16 matrices in (rank, token of the half) order: row c = 8 rank + token, inner 4g .. 4g+3 likewise
+        const int rr = c >> 3, ii = c & 7, ss = g >> 1, j0 = 4 * (g & 1);
+        const f32x4 ahl = *reinterpret_cast<const f32x4*>(&sN[(16 * rr + 8 + ii) * LDP + 16 * ss + j0]);
+        const f32x4 thh = *reinterpret_cast<const f32x4*>(&sT[(16 * rr + 8 + ii) * LDP + 16 * ss + 8 + j0]);
+        f32x4 tllT;                              // T_LL^T: row c is column c of T_LL
+#pragma unroll
+        for (int e = 0; e < 4; ++e) tllT[e] = sT[(16 * ss + j0 + e) * LDP + 16 * rr + ii];
+        Split<T> pa, pb;
+        split(tllT, pa);
+        split(ahl, pb);
+        const f32x4 xT = mm3(pa, pb, zero4());   // (A_HL T_LL)^T = T_LL^T A_HL^T
+        split(thh, pa);
+        split(xT, pb);
+        const f32x4 thl = mm3(pa, pb, zero4());  // T_HH (A_HL T_LL)
+        *reinterpret_cast<f32x4*>(&sT[(16 * rr + 8 + ii) * LDP + 16 * ss + j0]) = thl;
         __syncthreads();
     }
     Frag<T> tm[2][2];   // F(Tm^{s s'}): rows i, inner j
