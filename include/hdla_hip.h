@@ -89,8 +89,9 @@ typedef struct hdla_dims {
  * tile pairs are stored interleaved, element 8*lane + 4*which + i), "rows" are row-major, all laid out
  * [H][nch][...].  W, BGT, KGT, QG, AQB, AQK, EGL are parts of one block per (head, chunk) slot: the value given
  * is the offset for slot 0 and consecutive slots are SA_STRIDE bytes apart; likewise QGT, AQBT
- * with SB_STRIDE.  On the fused route the scans' operands never reach the workspace: only UT, TM, HC, DHC, DVN,
- * STRONG (and W where chunk_grad reads it) exist, in the backward pass. */
+ * with SB_STRIDE.  On the fused route the scans' operands never reach the workspace: only TM, HC, DHC, DVN, STRONG
+ * (and W, UT where chunk_grad reads them instead of rebuilding them: the hdla_param_ forms, fp32 decays beside bf16
+ * inputs) are written, in the backward pass. */
 typedef struct hdla_ws_layout {
     int64_t nch;               /* chunk slots per head */
     int64_t W, UT, KGT, BGT, VTT, EGL, QG, AQK, AQB, AQBT, QGT, TM, HC, DHC, DVN;
