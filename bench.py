@@ -37,8 +37,10 @@ METRIC = "chunked fwd+bwd tokens/s (B4,T2048,H16,K=V=64 bf16) + % of MFMA/HBM ro
 def _args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=5)
+    # Defaults: the clocks of an idle device take some tens of steps of this length to settle (measured: 0.39 ms a step
+    # over steps 6 .. 35 of a fresh process, 0.354 over steps 51 .. 250), so the untimed part is long enough for that
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="train", choices=["train", "fwd", "varlen", "decode", "copy", "hdla", "hdla_decode", "norm", "layer", "layer_decode", "shapes"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--brief", action="store_true", help="the named workload only: no other configurations, no keep_forward "
@@ -730,14 +732,14 @@ def main():
         n_other = max(5, args.steps // 3)
         others = {}
         for name, owl, ocfg in (("config1_fwd", "fwd", 1), ("config3_varlen", "varlen", 3)):
-            r = run_chunk_workload(owl, ocfg, n_other, 3, dev)
+            r = run_chunk_workload(owl, ocfg, n_other, max(3, args.warmup // 3), dev)
             others[name] = {"workload": r["config"]["workload"], "tokens/s": r["value"], "ms_per_step": r["ms_per_step"],
                             "dominant_kernel": r["roofline"]["kernel"], "frac": r["roofline"]["frac"],
                             "achieved_GB/s": r["roofline"]["achieved"], "traffic": r["roofline"]["traffic"],
                             "whole_step_frac_hbm": r["whole_step"]["frac_hbm"],
                             **({"keep_forward": r["keep_forward"]} if "keep_forward" in r else {}),
                             "kernels": [{k: x[k] for k in ("kernel", "ms", "frac_hbm", "frac_interface")} for x in r["kernels"]]}
-        r = run_decode_workload(4 * n_other, 5, dev)
+        r = run_decode_workload(4 * n_other, max(5, args.warmup), dev)
         others["config4_decode"] = {"workload": r["config"]["workload"], "tokens/s": r["value"], "ms_per_step": r["ms_per_step"],
                                     "dominant_kernel": "recurrent_kernel", "frac": r["roofline"]["frac"],
                                     "achieved_GB/s": r["roofline"]["achieved"], "traffic": r["roofline"]["traffic"],

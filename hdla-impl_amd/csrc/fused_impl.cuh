@@ -70,9 +70,14 @@ template <typename T, int K, int V, int MODE> struct FusedLds {
     static constexpr int OBOX = OPER, GBOX = OBOX + (MODE == FUSED_FWD ? CH * OROW : 0);
     static constexpr int SOLVE = GBOX + (MODE == FUSED_FWD ? CH * GROW : 0);
     static constexpr int SLOT = SOLVE + 2 * 32 * FLDP * 4;
-    // int ready[4], consumed[4], abort, -, -, -, part[4], inv[4], strong[4] (per producer pair; see fused_producer)
+    // int ready[4], consumed[4], abort, -, -, -, part[4], inv[4], strong[4] (per producer pair; see fused_producer), then
+    // two counters of the reverse kernel's consumers (records staged, records used: fused_consumer_rev)
     static constexpr int FLAGS = FNP * SLOT;
-    static constexpr int BYTES = FLAGS + 128;
+    // reverse kernel: transition records of the segments to the right, as split operands, for the consumers' chain
+    // (CHAIN_STAGE records of K x K at a time: every consumer wave needs them whole, each loads a quarter)
+    static constexpr int CHAIN_STAGE = 2;
+    static constexpr int CHAIN = FLAGS + 128;
+    static constexpr int BYTES = CHAIN + (REV ? CHAIN_STAGE * 2 * KT * KT * TB : 0);
 };
 
 // ---- hand-over counters ------------------------------------------------------------------------------------------
@@ -862,32 +867,6 @@ __device__ __forceinline__ void fused_consumer_fwd(const FusedArgs<T>& a, char* 
     }
 }
 
-// One step of chaining two segments, in split 2-byte products (three per tile pair: the error is that of fp32 products):
-//   X^T <- X^T Q^T + A^T   with X^T as KT fragments (rows value, inner channel) and Q as KT x KT tiles qt[kt_out][kt_in]
-template <typename T, int KT>
-__device__ __forceinline__ void chain_step(f32x4 (&X)[KT], const float* q_tiles, const float* add_tiles, int add_stride, bool out_major) {
-    const int l = lane_id();
-    Split<T> xs[KT];
-#pragma unroll
-    for (int kt = 0; kt < KT; ++kt) split(X[kt], xs[kt]);
-    f32x4 Y[KT];
-#pragma unroll
-    for (int ko = 0; ko < KT; ++ko) {
-        f32x4 acc = *reinterpret_cast<const f32x4*>(add_tiles + ko * add_stride + 4 * l);
-#pragma unroll
-        for (int ki = 0; ki < KT; ++ki) {
-            // tile (out, in) of the transition record
-            const float* qt = q_tiles + (out_major ? (ko * KT + ki) : (ki * KT + ko)) * TILE;
-            Split<T> qs;
-            split(*reinterpret_cast<const f32x4*>(qt + 4 * l), qs);
-            acc = mm3(xs[ki], qs, acc);
-        }
-        Y[ko] = acc;
-    }
-#pragma unroll
-    for (int kt = 0; kt < KT; ++kt) X[kt] = Y[kt];
-}
-
 // ---- consumers, reverse direction ------------------------------------------------------------------------------------
 template <typename T, int K, int V>
 __device__ __forceinline__ void fused_consumer_rev(const FusedArgs<T>& a, char* smem, int n, int h, int seg, int s0, int s1, int wv) {
@@ -910,14 +889,91 @@ __device__ __forceinline__ void fused_consumer_rev(const FusedArgs<T>& a, char* 
 #pragma unroll
             for (int i = 0; i < 4; ++i) dS[kt][i] = p.dht[soff + (int64_t)(16 * kt + 4 * g + i) * V];
     }
-    // the gradient entering this segment from the right: through the later segments, last one first
-    for (int s = a.nseg - 1; s > seg; --s) {
-        int q0, q1;
-        seg_range(p.st, n, a.nseg, s, q0, q1);
-        if (q1 <= q0) continue;                            // uniform
-        const int64_t rec = ((int64_t)n * H + h) * a.nseg + s;
-        // tile (kt, k't) of the record holds rows k', inner k: the output index is the tile's second index
-        chain_step<T, KT>(dS, a.mseg + rec * (K * K), a.rseg + rec * (K * V) + vt * KT * TILE, TILE, false);
+    // The gradient entering this segment from the right: through the later segments, last one first,
+    //   dS <- M_s^T dS + R_s   (as fragments: X^T <- X^T Q^T + A^T, tile (in, out) of the record at index in * KT + out).
+    // Nothing waits for the producers here, so only the chain's own latency counts: the records of up to CHAIN_STAGE
+    // segments are requested at once, a quarter of each transition record by each of the four consumer waves, which
+    // share them through LDS as split operands; the consumers meet at two counters of their own (the producers are
+    // at work meanwhile, so no workgroup barrier).
+    {
+        static_assert(VT == 4 && KT == 4, "a quarter of a record per consumer wave");
+        constexpr int NQ = KT * KT / 4, STG = L::CHAIN_STAGE;
+        // (one lane address for the whole area, opaque to the compiler: the area lies beyond the reach of an LDS
+        // instruction's immediate offset from zero, and a register per tile address would not fit)
+        int sMo = L::CHAIN + 4 * l * (int)sizeof(T);
+        asm volatile("" : "+v"(sMo));
+        T* const sM = reinterpret_cast<T*>(smem + sMo);
+        const int64_t rec0 = ((int64_t)n * H + h) * a.nseg;
+        int batch = 0, s = a.nseg - 1;
+        while (s > seg) {
+            int step[STG], ns = 0, q0, q1;
+#pragma unroll
+            for (int b = 0; b < STG; ++b) {
+                step[b] = 0;
+                while (s > seg) {
+                    seg_range(p.st, n, a.nseg, s, q0, q1);
+                    if (q1 > q0) break;
+                    --s;
+                }
+                if (s > seg) { step[b] = s--; ns = b + 1; }
+            }
+            f32x4 mq[STG][NQ], add[STG][KT];
+#pragma unroll
+            for (int b = 0; b < STG; ++b) {
+                if (b < ns) {
+                    const float* mrec = a.mseg + (rec0 + step[b]) * (K * K) + wv * NQ * TILE + 4 * l;
+#pragma unroll
+                    for (int i = 0; i < NQ; ++i) mq[b][i] = *reinterpret_cast<const f32x4*>(mrec + i * TILE);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int b = 0; b < STG; ++b) {
+                if (b < ns) {
+                    const float* rrec = a.rseg + (rec0 + step[b]) * (K * V) + vt * KT * TILE + 4 * l;
+#pragma unroll
+                    for (int kt = 0; kt < KT; ++kt) add[b][kt] = *reinterpret_cast<const f32x4*>(rrec + kt * TILE);
+                }
+            }
+            // every consumer has read the previous round's records out of LDS
+            if (batch > 0 && !wait_ge(&flags[25], VT * batch, &flags[8])) { if (l == 0) *a.err = FUSED_ABORTED + 3; return; }
+#pragma unroll
+            for (int b = 0; b < STG; ++b) {
+                if (b < ns) {
+#pragma unroll
+                    for (int i = 0; i < NQ; ++i) {
+                        Split<T> q;
+                        split(mq[b][i], q);
+                        st_frag(sM + ((b * 2 + 0) * KT * KT + wv * NQ + i) * TILE, q.hi);
+                        st_frag(sM + ((b * 2 + 1) * KT * KT + wv * NQ + i) * TILE, q.lo);
+                    }
+                }
+            }
+            signal_add(&flags[24]);
+            if (!wait_ge(&flags[24], VT * (batch + 1), &flags[8])) { if (l == 0) *a.err = FUSED_ABORTED + 3; return; }
+#pragma unroll
+            for (int b = 0; b < STG; ++b) {
+                if (b < ns) {
+                    Split<T> xs[KT];
+#pragma unroll
+                    for (int kt = 0; kt < KT; ++kt) split(dS[kt], xs[kt]);
+#pragma unroll
+                    for (int ko = 0; ko < KT; ++ko) {
+                        f32x4 acc = add[b][ko];
+#pragma unroll
+                        for (int ki = 0; ki < KT; ++ki) {
+                            Split<T> q;
+                            q.hi = ld_frag(sM + ((b * 2 + 0) * KT * KT + ki * KT + ko) * TILE);
+                            q.lo = ld_frag(sM + ((b * 2 + 1) * KT * KT + ki * KT + ko) * TILE);
+                            acc = mm3(xs[ki], q, acc);
+                        }
+                        dS[ko] = acc;
+                    }
+                }
+            }
+            signal_add(&flags[25]);
+            ++batch;
+        }
     }
 
     for (int t = 0; t < nst; ++t) {
@@ -1005,34 +1061,44 @@ __global__ __launch_bounds__(64 * (V / 16 + 2 * FNP)) void fused_kernel(FusedArg
 }
 
 // ---- forward pass, second kernel: the true entering states, and their part of the output ----------------------------
-// grid = (H, nseg, N), 256 threads.  blockIdx.y = s in 1 .. nseg-1: segment s (chain the records of segments 0 .. s-1
-// into S_in(s), keep it as the boundary record, add G S_in(s) to the segment's local outputs); blockIdx.y = 0: the
-// final state (all segments chained).  Wave j chains column block j of the state (the blocks are independent), the
-// waves exchange their blocks through LDS, and each then takes every fourth chunk of the segment, four chunks' loads in
-// flight at a time.
+// grid = (H, nseg * FIXUP_PARTS, N), 256 threads.  blockIdx.y / FIXUP_PARTS = s in 1 .. nseg-1: segment s (chain the
+// records of segments 0 .. s-1 into S_in(s), keep it as the boundary record, add G S_in(s) to the segment's local
+// outputs); 0: the final state (all segments chained).  The kernel is a chain of dependent steps between two launches,
+// so everything is arranged for its latency: all loads that do not depend on the chain are issued at the start (the
+// first chunks' operands, the records of up to FIXUP_STAGE chain steps); the transition records, which every wave needs
+// whole, are loaded a quarter by each wave and shared through LDS as split operands; wave j chains column block j of
+// the state (the blocks are independent); FIXUP_PARTS workgroups share the chunks of a segment, each repeating the
+// chain, so that a workgroup's share of the chunks is in flight from the start as well.
+constexpr int FIXUP_PARTS = 2;                            // workgroups that share one segment's chunks (measured: 1, 2, 4 -> 17.1, 16.8, 18.8 us)
+constexpr int FIXUP_STAGE = 3;                            // chain steps whose records are in LDS at a time
 template <typename T, int K, int V>
 __global__ __launch_bounds__(256) void fixup_kernel(FusedArgs<T> a) {
-    constexpr int KT = K / 16, VT = V / 16, NB = 4;
-    static_assert(VT == 4, "one column block per wave");
+    constexpr int KT = K / 16, VT = V / 16, NB = 2, NQ = KT * KT / 4;
+    static_assert(VT == 4 && KT == 4 && sizeof(T) == 2, "one column block per wave, a quarter of a transition record per wave");
     constexpr int OROW = V * (int)sizeof(T) + 16;
     __shared__ __attribute__((aligned(16))) char stage[4][CH * OROW];
     __shared__ __attribute__((aligned(16))) T sS[VT * KT * TILE];          // S_in as operand tiles [vt][kt]
+    __shared__ __attribute__((aligned(16))) T sM[FIXUP_STAGE][2][KT * KT * TILE];   // transition records, hi and lo halves
     const ChunkArgs<T>& p = a.c;
     const int h = blockIdx.x;
     const int n = p.st.cu ? p.st.order[blockIdx.z] : (int)blockIdx.z;
-    const int target = blockIdx.y == 0 ? a.nseg : (int)blockIdx.y;       // chain segments 0 .. target-1
+    const int ty = (int)blockIdx.y / FIXUP_PARTS, part = (int)blockIdx.y % FIXUP_PARTS;
+    const int target = ty == 0 ? a.nseg : ty;                            // chain segments 0 .. target-1
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int l = lane_id(), g = l >> 4, c = l & 15;
     const int H = p.H, vt = wv;
     int s0 = 0, s1 = 0;
     if (target < a.nseg) {
         seg_range(p.st, n, a.nseg, target, s0, s1);
-        if (s1 <= s0) return;
-    } else if (!p.ht) return;
+        // this workgroup's share of the segment's chunks
+        const int per = (s1 - s0 + FIXUP_PARTS - 1) / FIXUP_PARTS;
+        s0 = min(s0 + part * per, s1);
+        s1 = min(s0 + per, s1);
+        if (s1 <= s0 || (part > 0 && !a.gw)) return;
+    } else if (!p.ht || part > 0) return;
     const int64_t rec0 = ((int64_t)n * H + h) * a.nseg;
     const int64_t soff = ((int64_t)n * H + h) * K * V + 16 * vt + c;
 
-    // the chunks' operands are requested before the chain, whose loads are dependent round trips
     int c0, c1;
     seq_chunks(p.st, n, c0, c1);
     int64_t bos, eos;
@@ -1055,26 +1121,84 @@ __global__ __launch_bounds__(256) void fixup_kernel(FusedArgs<T> a) {
     const bool outputs = target < a.nseg && a.gw != nullptr;
     if (outputs) request(s0 + wv);
 
-    // S[kt]: lane (g,c) reg i = S[16kt + 4g + i][16vt + c]
+    // S[kt]: lane (g,c) reg i = S[16kt + 4g + i][16vt + c].  Segment 0 ran from the initial state itself; only where it
+    // is empty does the chain start from the initial state here.
     f32x4 S[KT];
+    int q0, q1;
+    seg_range(p.st, n, a.nseg, 0, q0, q1);
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
-        S[kt] = zero4();
-        if (p.h0) {
+        if (q1 > q0) {
+            S[kt] = *reinterpret_cast<const f32x4*>(a.sloc + rec0 * (K * V) + (vt * KT + kt) * TILE + 4 * l);
+        } else {
+            S[kt] = zero4();
+            if (p.h0) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) S[kt][i] = p.h0[soff + (int64_t)(16 * kt + 4 * g + i) * V];
+                for (int i = 0; i < 4; ++i) S[kt][i] = p.h0[soff + (int64_t)(16 * kt + 4 * g + i) * V];
+            }
         }
     }
-    for (int s = 0; s < target; ++s) {
-        int q0, q1;
-        seg_range(p.st, n, a.nseg, s, q0, q1);
-        if (q1 <= q0) continue;
-        const float* sloc = a.sloc + (rec0 + s) * (K * V) + vt * KT * TILE;
-        if (s == 0) {
+    // the chain, FIXUP_STAGE non-empty segments at a time
+    int s = 1;
+    while (s < target) {
+        int step[FIXUP_STAGE], ns = 0;
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt) S[kt] = *reinterpret_cast<const f32x4*>(sloc + kt * TILE + 4 * l);
-        } else {
-            chain_step<T, KT>(S, a.mseg + (rec0 + s) * (K * K), sloc, TILE, true);
+        for (int b = 0; b < FIXUP_STAGE; ++b) {
+            step[b] = 0;
+            while (s < target) {
+                seg_range(p.st, n, a.nseg, s, q0, q1);
+                if (q1 > q0) break;
+                ++s;
+            }
+            if (s < target) { step[b] = s++; ns = b + 1; }
+        }
+        f32x4 mq[FIXUP_STAGE][NQ], add[FIXUP_STAGE][KT];
+#pragma unroll
+        for (int b = 0; b < FIXUP_STAGE; ++b) {
+            if (b < ns) {
+                const float* mrec = a.mseg + (rec0 + step[b]) * (K * K) + wv * NQ * TILE + 4 * l;
+                const float* srec = a.sloc + (rec0 + step[b]) * (K * V) + vt * KT * TILE + 4 * l;
+#pragma unroll
+                for (int i = 0; i < NQ; ++i) mq[b][i] = *reinterpret_cast<const f32x4*>(mrec + i * TILE);
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) add[b][kt] = *reinterpret_cast<const f32x4*>(srec + kt * TILE);
+            }
+        }
+        __syncthreads();                                  // the previous round's records have been used
+#pragma unroll
+        for (int b = 0; b < FIXUP_STAGE; ++b) {
+            if (b < ns) {
+#pragma unroll
+                for (int i = 0; i < NQ; ++i) {
+                    Split<T> q;
+                    split(mq[b][i], q);
+                    st_tile(sM[b][0] + (wv * NQ + i) * TILE, q.hi);
+                    st_tile(sM[b][1] + (wv * NQ + i) * TILE, q.lo);
+                }
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int b = 0; b < FIXUP_STAGE; ++b) {
+            if (b < ns) {
+                // X^T <- X^T Q^T + A^T in split 2-byte products (three per tile pair: the error of fp32 products); tile
+                // (out, in) of the record is at index out * KT + in
+                Split<T> xs[KT];
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) split(S[kt], xs[kt]);
+#pragma unroll
+                for (int ko = 0; ko < KT; ++ko) {
+                    f32x4 acc = add[b][ko];
+#pragma unroll
+                    for (int ki = 0; ki < KT; ++ki) {
+                        Split<T> q;
+                        q.hi = ld_tile(sM[b][0] + (ko * KT + ki) * TILE);
+                        q.lo = ld_tile(sM[b][1] + (ko * KT + ki) * TILE);
+                        acc = mm3(xs[ki], q, acc);
+                    }
+                    S[ko] = acc;
+                }
+            }
         }
     }
     if (target == a.nseg) {
@@ -1084,7 +1208,7 @@ __global__ __launch_bounds__(256) void fixup_kernel(FusedArgs<T> a) {
             for (int i = 0; i < 4; ++i) p.ht[soff + (int64_t)(16 * kt + 4 * g + i) * V] = S[kt][i];
         return;
     }
-    if (a.sin_out) {
+    if (a.sin_out && part == 0) {
         float* so = a.sin_out + (rec0 + target) * (K * V) + vt * KT * TILE;
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<f32x4*>(so + kt * TILE + 4 * l) = S[kt];
