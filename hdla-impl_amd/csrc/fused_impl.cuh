@@ -398,7 +398,13 @@ __device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem
             // temporaries would all be live at once)
             __builtin_amdgcn_sched_barrier(0);
             const f32x4 gl = bcast16<CH - 1>(gi);
-            const f32x4 egi = exp4<T>(gi), ege = exp4<T>(ge), edn = exp4<T>(gl - gi);
+            const f32x4 egi = exp4<T>(gi), edn = exp4<T>(gl - gi);
+            // e^{ge} of a token is e^{gi} of the token before it (1 for the first), e^{gl} is e^{gi} of the last token:
+            // lane moves in place of two more rounds of exponentials
+            f32x4 ege = dpp0<0x111>(egi);                 // row_shr:1 (lanes of one token group are a DPP row)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ege[i] = c == 0 ? 1.f : ege[i];
+            const f32x4 egl = bcast16<CH - 1>(egi);
             st_pair(sWW + (0 * KT2 + half) * PAIR, j, transpose(to_frag<T>(a0 * ege), ident));
             st_pair(sWW + (1 * KT2 + half) * PAIR, j, transpose(to_frag<T>(a1 * ege), ident));
             const Frag<T> fqg = to_frag<T>(q4 * egi * scale);
@@ -415,7 +421,7 @@ __device__ __forceinline__ void fused_producer(const FusedArgs<T>& a, char* smem
                 st_pair(reinterpret_cast<T*>(slot + SB.BGT) + (1 * KT2 + half) * PAIR, j, fbg[1]);
                 st_pair(reinterpret_cast<T*>(slot + SB.QGT) + half * PAIR, j, transpose(fqg, ident));
             }
-            if (c == 0) *reinterpret_cast<f32x4*>(slot + (REV ? SB.EGL : BF.EGL) + (16 * (kt0 + j) + 4 * g) * 4) = exp4<T>(gl);
+            if (c == 0) *reinterpret_cast<f32x4*>(slot + (REV ? SB.EGL : BF.EGL) + (16 * (kt0 + j) + 4 * g) * 4) = egl;
             __builtin_amdgcn_sched_barrier(0);
         }
         // Each wave decides for its own channels (the parts of the score tiles add up whichever way they were formed).
