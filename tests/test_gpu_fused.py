@@ -175,3 +175,37 @@ def test_config2_full_size_against_classic_route():
         errs = {n: O.rel_l2(g_f[n], g_c[n]) for n in g_c}
         print("config 2 backward, fused vs classic:", {k: f"{v:.1e}" for k, v in errs.items()}, flush=True)
         assert all(e <= 6e-3 for e in errs.values()), errs
+
+
+@pytest.mark.parametrize("segments", [1, 4])
+def test_stage_wise_launches_reproduce_the_single_calls(segments):
+    """hdla_chunk_stages on the fused route (what bench.py times kernel by kernel): the stages launched one at a time
+    leave the same bits as hdla_chunk_fwd / hdla_chunk_bwd."""
+    lib = _lib.load()
+    x = _dev(make_inputs(28, 2, 520, 3, 64, 64, gk_div=8.0))
+    B, T, H, K = x["q"].shape
+    dims = _lib.make_dims(B, T, H, K, 64, 2, B, torch.bfloat16, torch.bfloat16, 0.7, None, route=_lib.ROUTE_FUSED, segments=segments)
+    P, stream = _lib.ptr, _lib.current_stream(torch.device(DEV))
+    o_1, ht_1, _ = forward(x, _lib.ROUTE_FUSED, segments)
+    g_1 = backward(x, _lib.ROUTE_FUSED, segments)                    # no boundary record: the summary pass runs first
+    ws = _lib.workspace(dims, 0, DEV)
+    o = torch.zeros_like(x["v"])
+    ht = torch.empty(B, H, K, 64, dtype=torch.float32, device=DEV)
+    g = {n: torch.zeros_like(x[n]) for n in NAMES}
+    dh0 = torch.empty(B, H, K, 64, dtype=torch.float32, device=DEV)
+
+    def stage(pass_, mask, w):
+        rc = lib.hdla_chunk_stages(ctypes.byref(dims), pass_, mask, P(x["q"]), P(x["k"]), P(x["v"]), P(x["a"]), P(x["b"]), P(x["gk"]),
+                                   P(x["h0"]), P(o), P(ht), P(x["do"]), P(x["dht"]), P(g["q"]), P(g["k"]), P(g["v"]), P(g["a"]),
+                                   P(g["b"]), P(g["gk"]), P(dh0), P(w), w.numel(), stream)
+        _lib.check(rc, "hdla_chunk_stages")
+    for mask in ([2, 16] if segments > 1 else [2]):
+        stage(0, mask, ws)
+    assert torch.equal(o, o_1) and torch.equal(ht, ht_1)
+    wb = _lib.workspace(dims, 1, DEV)
+    for mask in (([16] if segments > 1 else []) + [2, 4, 8]):
+        stage(1, mask, wb)
+    _check_err(wb, dims, 1)
+    g["h0"] = dh0
+    for n in g_1:
+        assert torch.equal(g[n], g_1[n]), n
